@@ -1,0 +1,98 @@
+"""ctypes declarations for the C ABI in ``include/ellm_attn.h``."""
+import ctypes
+import os
+
+DTYPE_F16 = 0
+DTYPE_BF16 = 1
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+
+
+def lib_path():
+    return os.path.join(_HERE, "lib", "libellm_attn.so")
+
+
+class LibraryMissing(RuntimeError):
+    """libellm_attn.so has not been built (run ``__graft_entry__.build()``)."""
+
+
+class EllmError(RuntimeError):
+    def __init__(self, status, message):
+        super().__init__(f"ellm status {status}: {message}")
+        self.status = status
+        self.message = message
+
+
+class AttnDesc(ctypes.Structure):
+    _fields_ = [
+        ("q", ctypes.c_void_p),
+        ("k", ctypes.c_void_p),
+        ("v", ctypes.c_void_p),
+        ("out", ctypes.c_void_p),
+        ("lse", ctypes.c_void_p),
+        ("batch_size", ctypes.c_size_t),
+        ("attention_head_num", ctypes.c_size_t),
+        ("kv_head_num", ctypes.c_size_t),
+        ("head_size", ctypes.c_size_t),
+        ("kv_strides", ctypes.c_size_t * 4),
+        ("inverse_sqrt_head", ctypes.c_float),
+        ("dtype", ctypes.c_int),
+        ("sequence_capacity", ctypes.c_size_t),
+        ("max_position_interval", ctypes.c_size_t),
+    ]
+
+
+class KvDesc(ctypes.Structure):
+    _fields_ = [
+        ("layers", ctypes.c_size_t),
+        ("sequences", ctypes.c_size_t),
+        ("kv_head_num", ctypes.c_size_t),
+        ("head_size", ctypes.c_size_t),
+        ("capacity", ctypes.c_size_t),
+        ("dtype", ctypes.c_int),
+    ]
+
+
+_sz = ctypes.c_size_t
+_vp = ctypes.c_void_p
+_pvp = ctypes.POINTER(ctypes.c_void_p)
+
+# name -> (restype, argtypes); every entry point include/ellm_attn.h declares.
+ABI_SYMBOLS = {
+    "ellm_last_error_string": (ctypes.c_char_p, []),
+    "ellm_attn_version": (ctypes.c_int, []),
+    "ellm_device_count": (ctypes.c_int, []),
+    "ellm_attn_create": (ctypes.c_int, [ctypes.POINTER(AttnDesc), _pvp]),
+    "ellm_attn_destroy": (ctypes.c_int, [_vp]),
+    "ellm_attn_run": (ctypes.c_int, [_vp, _sz, _sz, _sz, _vp]),
+    "ellm_attn_run_ragged": (ctypes.c_int, [_vp, _vp, _sz, _sz, _vp]),
+    "ellm_kv_create": (ctypes.c_int, [ctypes.POINTER(KvDesc), _pvp]),
+    "ellm_kv_destroy": (ctypes.c_int, [_vp]),
+    "ellm_kv_layer": (ctypes.c_int, [_vp, _sz, _pvp, _pvp, ctypes.POINTER(_sz * 4)]),
+    "ellm_kv_append": (ctypes.c_int, [_vp, _sz, _sz, _sz, _sz, _vp, _vp, _sz, _vp]),
+}
+
+_lib = None
+
+
+def load_library():
+    """Load libellm_attn.so once; raises LibraryMissing when it is not built."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    path = lib_path()
+    if not os.path.exists(path):
+        raise LibraryMissing(f"{path} not found; build it with __graft_entry__.build()")
+    lib = ctypes.CDLL(path)
+    for name, (res, args) in ABI_SYMBOLS.items():
+        fn = getattr(lib, name)
+        fn.restype = res
+        fn.argtypes = args
+    _lib = lib
+    return lib
+
+
+def check(status):
+    if status != 0:
+        msg = load_library().ellm_last_error_string()
+        raise EllmError(status, msg.decode() if msg else "")

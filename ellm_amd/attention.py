@@ -1,0 +1,147 @@
+"""Host-side mirror of the reference's attention operator over the C ABI.
+
+``Attention`` takes the argument list of ``Attention::new`` and exposes ``run``
+with the meaning of ``Attention::run`` (reference:
+src/compiler/mul/attention.rs:41-67 and 69-76).  The reference's ``cpu_num`` /
+``thread_id`` pair is accepted and follows its calling convention — every
+worker thread calls ``run`` and then meets a barrier (src/serving/start.rs:69-73)
+— by letting thread 0 enqueue the launch and every other thread return at once.
+
+Tensors are torch CUDA tensors used as plain device buffers; nothing here
+computes with torch.
+"""
+import ctypes
+
+from . import _lib
+from ._lib import AttnDesc, KvDesc, check, load_library
+
+
+def _dtype_code(t):
+    import torch
+
+    if t.dtype == torch.float16:
+        return _lib.DTYPE_F16
+    if t.dtype == torch.bfloat16:
+        return _lib.DTYPE_BF16
+    raise TypeError(f"unsupported storage type {t.dtype}")
+
+
+def _stream_ptr(stream):
+    import torch
+
+    if stream is None:
+        stream = torch.cuda.current_stream()
+    return ctypes.c_void_p(stream.cuda_stream)
+
+
+class Attention:
+    """Attention::new / run over device buffers.
+
+    q, out: [max_position_interval, batch_capacity, attention_head_num, head_size]
+    k, v:   any 4-d view [sequence, kv_head, position, head_size] (strides are passed on)
+    """
+
+    def __init__(self, q, k, v, out, batch_size, attention_head_num, kv_head_num, head_size,
+                 kv_strides, inverse_sqrt_head, lse=None, sequence_capacity=None,
+                 max_position_interval=None):
+        self._lib = load_library()
+        self._keep = (q, k, v, out, lse)
+        d = AttnDesc()
+        d.q, d.k, d.v, d.out = q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr()
+        d.lse = lse.data_ptr() if lse is not None else None
+        d.batch_size = batch_size
+        d.attention_head_num = attention_head_num
+        d.kv_head_num = kv_head_num
+        d.head_size = head_size
+        for i in range(4):
+            d.kv_strides[i] = int(kv_strides[i])
+        d.inverse_sqrt_head = float(inverse_sqrt_head)
+        d.dtype = _dtype_code(q)
+        d.sequence_capacity = int(sequence_capacity if sequence_capacity is not None else k.shape[2])
+        d.max_position_interval = int(
+            max_position_interval if max_position_interval is not None else q.shape[0])
+        self.desc = d
+        self._handle = ctypes.c_void_p()
+        check(self._lib.ellm_attn_create(ctypes.byref(d), ctypes.byref(self._handle)))
+
+    @classmethod
+    def new(cls, *args, **kwargs):
+        return cls(*args, **kwargs)
+
+    def run(self, position_index, position_interval, batch_size, cpu_num=1, thread_id=0,
+            stream=None):
+        if thread_id != 0:
+            return  # the launch is enqueued once, by thread 0
+        check(self._lib.ellm_attn_run(self._handle, position_index, position_interval, batch_size,
+                                      _stream_ptr(stream)))
+
+    def run_ragged(self, positions, max_position, batch_size, stream=None):
+        """Single-token step; positions: uint32/int32 device tensor, one entry per sequence."""
+        check(self._lib.ellm_attn_run_ragged(self._handle, ctypes.c_void_p(positions.data_ptr()),
+                                             int(max_position), batch_size, _stream_ptr(stream)))
+
+    def close(self):
+        if self._handle:
+            check(self._lib.ellm_attn_destroy(self._handle))
+            self._handle = ctypes.c_void_p()
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+
+class KVCache:
+    """[layer][sequence][kv_head][position][128] keys and values in one allocation each."""
+
+    def __init__(self, layers, sequences, kv_head_num, capacity, dtype_code, head_size=128):
+        self._lib = load_library()
+        d = KvDesc(layers, sequences, kv_head_num, head_size, capacity, dtype_code)
+        self.desc = d
+        self._handle = ctypes.c_void_p()
+        check(self._lib.ellm_kv_create(ctypes.byref(d), ctypes.byref(self._handle)))
+
+    def layer(self, layer):
+        k, v = ctypes.c_void_p(), ctypes.c_void_p()
+        strides = (ctypes.c_size_t * 4)()
+        check(self._lib.ellm_kv_layer(self._handle, layer, ctypes.byref(k), ctypes.byref(v),
+                                      ctypes.byref(strides)))
+        return k.value, v.value, list(strides)
+
+    def layer_tensors(self, layer, torch_dtype):
+        """Borrow one layer's K and V as torch tensors [sequence, kv_head, position, 128]."""
+        import torch
+
+        k, v, _ = self.layer(layer)
+        d = self.desc
+        shape = (d.sequences, d.kv_head_num, d.capacity, d.head_size)
+        n = d.sequences * d.kv_head_num * d.capacity * d.head_size
+
+        def wrap(ptr):
+            iface = {"shape": (n,), "typestr": "<i2", "data": (ptr, False), "version": 2}
+            holder = type("DevBuf", (), {"__cuda_array_interface__": iface})()
+            return torch.as_tensor(holder, device="cuda").view(torch_dtype).view(shape)
+
+        return wrap(k), wrap(v)
+
+    def append(self, layer, position_index, k_src, v_src, batch_size=None, stream=None):
+        """k_src / v_src: [n_tokens, src_batch_pitch, kv_head, 128] device tensors."""
+        n_tokens, pitch = k_src.shape[0], k_src.shape[1]
+        if batch_size is None:
+            batch_size = pitch
+        check(self._lib.ellm_kv_append(self._handle, layer, position_index, n_tokens, batch_size,
+                                       ctypes.c_void_p(k_src.data_ptr()),
+                                       ctypes.c_void_p(v_src.data_ptr()), pitch,
+                                       _stream_ptr(stream)))
+
+    def close(self):
+        if self._handle:
+            check(self._lib.ellm_kv_destroy(self._handle))
+            self._handle = ctypes.c_void_p()
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass

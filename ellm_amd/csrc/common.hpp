@@ -1,0 +1,116 @@
+// Shared device helpers for the gfx950 attention kernels: storage-type traits,
+// MFMA wrappers with their operand layouts, and small wave-level utilities.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace ellm {
+
+constexpr int kHeadDim = 128;  // the reference kernel is hard-wired to 128 too
+constexpr int kWave = 64;
+
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x4 __attribute__((ext_vector_type(4)));
+typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef short s16x4 __attribute__((ext_vector_type(4)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+
+struct F16 {};   // IEEE binary16 storage
+struct BF16 {};  // bfloat16 storage
+
+// ---- MFMA wrappers ---------------------------------------------------------
+// Operands travel as raw 128-bit / 64-bit register groups (8 or 4 packed 16-bit
+// values per lane).  Layouts (lane l of the 64-wide wave):
+//   32x32x16: A[i][k], B[k][j]: i or j = l % 32, k = 8*(l/32) + 0..7
+//             C[i][j]: j = l % 32, i = 8*(r/4) + 4*(l/32) + r%4 for register r of 16
+//   16x16x32: A[i][k], B[k][j]: i or j = l % 16, k = 8*(l/16) + 0..7
+//             C[i][j]: j = l % 16, i = 4*(l/16) + r for register r of 4
+//   16x16x16: A[i][k], B[k][j]: i or j = l % 16, k = 4*(l/16) + 0..3; C as 16x16x32
+
+template <typename T>
+struct Mfma;
+
+template <>
+struct Mfma<F16> {
+  static __device__ __forceinline__ f32x16 m32x32x16(u32x4 a, u32x4 b, f32x16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a),
+                                                  __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
+  }
+  static __device__ __forceinline__ f32x4 m16x16x32(u32x4 a, u32x4 b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, a),
+                                                  __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
+  }
+  static __device__ __forceinline__ f32x4 m16x16x16(u32x2 a, u32x2 b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x16f16(__builtin_bit_cast(f16x4, a),
+                                                 __builtin_bit_cast(f16x4, b), c, 0, 0, 0);
+  }
+  // two binary32 -> packed pair, round to nearest even
+  static __device__ __forceinline__ uint32_t pack2(float lo, float hi) {
+    f16x2 v = {(_Float16)lo, (_Float16)hi};
+    return __builtin_bit_cast(uint32_t, v);
+  }
+  static __device__ __forceinline__ float to_float(uint16_t bits) {
+    return (float)__builtin_bit_cast(_Float16, bits);
+  }
+};
+
+template <>
+struct Mfma<BF16> {
+  static __device__ __forceinline__ f32x16 m32x32x16(u32x4 a, u32x4 b, f32x16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a),
+                                                   __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+  }
+  static __device__ __forceinline__ f32x4 m16x16x32(u32x4 a, u32x4 b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a),
+                                                   __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+  }
+  static __device__ __forceinline__ f32x4 m16x16x16(u32x2 a, u32x2 b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(__builtin_bit_cast(s16x4, a),
+                                                     __builtin_bit_cast(s16x4, b), c, 0, 0, 0);
+  }
+  static __device__ __forceinline__ uint32_t pack2(float lo, float hi) {
+    bf16x2 v = {(__bf16)lo, (__bf16)hi};
+    return __builtin_bit_cast(uint32_t, v);
+  }
+  static __device__ __forceinline__ float to_float(uint16_t bits) {
+    return __builtin_bit_cast(float, (uint32_t)bits << 16);
+  }
+};
+
+// ---- small utilities -------------------------------------------------------
+
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+__device__ __forceinline__ float fast_log2(float x) { return __builtin_amdgcn_logf(x); }
+
+__device__ __forceinline__ u32x4 load16(const void* p) { return *(const u32x4*)p; }
+__device__ __forceinline__ void store16(void* p, u32x4 v) { *(u32x4*)p = v; }
+
+// Exchange with the lane whose index differs in the given bit (16 or 32).
+__device__ __forceinline__ float xor_shuffle(float v, int mask) { return __shfl_xor(v, mask, 64); }
+
+// Regroup packed 16-bit pairs: given four registers holding (x[k][2c], x[k][2c+1])
+// for k = 0..3, return the two registers holding (x[0][e], x[1][e]) and
+// (x[2][e], x[3][e]) for e = 2c (hi = false) or 2c+1 (hi = true).
+__device__ __forceinline__ u32x2 gather_column(uint32_t r0, uint32_t r1, uint32_t r2, uint32_t r3,
+                                               bool hi) {
+  u32x2 o;
+  if (hi) {
+    o[0] = (r0 >> 16) | (r1 & 0xffff0000u);
+    o[1] = (r2 >> 16) | (r3 & 0xffff0000u);
+  } else {
+    o[0] = (r0 & 0xffffu) | (r1 << 16);
+    o[1] = (r2 & 0xffffu) | (r3 << 16);
+  }
+  return o;
+}
+
+constexpr float kLog2e = 1.4426950408889634f;
+constexpr float kLn2 = 0.6931471805599453f;
+
+}  // namespace ellm

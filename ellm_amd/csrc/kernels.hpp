@@ -1,0 +1,59 @@
+// Internal interface between the C ABI (api.hip) and the kernel launchers.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stddef.h>
+#include <stdint.h>
+
+namespace ellm {
+
+// Everything a launch needs; filled by the C ABI after validation.
+struct AttnArgs {
+  const void* q;
+  const void* k;
+  const void* v;
+  void* out;
+  float* lse;             // may be null
+  uint32_t batch_pitch;   // sequences per token row of Q/O (capacity)
+  uint32_t n_q_heads;
+  uint32_t n_kv_heads;
+  uint32_t group;         // n_q_heads / n_kv_heads
+  size_t kv_stride_seq;   // elements
+  size_t kv_stride_head;  // elements
+  size_t kv_stride_pos;   // elements
+  float scale;
+  int dtype;              // 0 = binary16, 1 = bfloat16
+  uint32_t capacity;      // positions per K/V plane
+  // per run
+  uint32_t position_index;
+  uint32_t position_interval;
+  uint32_t batch;
+  const uint32_t* positions;  // device, per sequence; null = position_index for all
+  // single-token path workspace
+  float* ws_acc;  // [batch][kv_head][split][group][128]
+  float* ws_ml;   // [batch][kv_head][split][group][2]  (max in log2 units, sum)
+  uint32_t split_len;  // keys per split, multiple of 64
+  uint32_t n_split;
+};
+
+// Keys handled by one workgroup step of the single-token kernel.
+constexpr uint32_t kDecodeStepKeys = 64;
+// Upper bound on the number of partial rows (sequence x head x split) the
+// workspace must hold for a given capacity; see decode_plan().
+struct DecodePlan {
+  uint32_t split_len;
+  uint32_t n_split;
+};
+DecodePlan decode_plan(uint32_t max_len, uint32_t batch, uint32_t n_kv_heads, uint32_t n_cu);
+size_t decode_workspace_rows(uint32_t batch_capacity, uint32_t n_q_heads, uint32_t n_kv_heads,
+                             uint32_t n_cu);
+
+hipError_t launch_decode(const AttnArgs& a, hipStream_t stream);
+hipError_t launch_prefill(const AttnArgs& a, hipStream_t stream);
+
+hipError_t launch_kv_append(void* k_dst, void* v_dst, const void* k_src, const void* v_src,
+                            uint32_t n_tokens, uint32_t batch, uint32_t src_batch_pitch,
+                            uint32_t n_kv_heads, uint32_t capacity, uint32_t position_index,
+                            hipStream_t stream);
+
+}  // namespace ellm

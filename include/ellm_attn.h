@@ -1,0 +1,168 @@
+/*
+ * ellm_attn.h — C ABI of the MI355X (gfx950) attention path for eLLM.
+ *
+ * What this replaces in the reference (paths relative to the eLLM tree):
+ *   - compiler::mul::attention::Attention::{new,run}   src/compiler/mul/attention.rs:41-67, 69-156
+ *   - its leaf kernels                                 src/kernel/x86_64/f16_512/flash_attention.rs:30-92
+ *                                                      src/kernel/generic/flash_attention.rs:60-89
+ *   - the per-layer key/value buffers of memory::Cache src/memory/cache.rs:23, 69-75
+ *
+ * All pointers named "device" are HIP device pointers.  Every function returns
+ * ELLM_OK (0) or an ellm_status; nothing aborts the process.  Functions taking a
+ * stream enqueue work on it and return without waiting (stream = NULL is the
+ * HIP null stream).  A handle may be used from one host thread at a time.
+ *
+ * Only head_size == 128 and 16-bit storage (binary16 / bfloat16) are supported,
+ * like the reference's AVX-512 kernel (head_size hard-wired to 128 there,
+ * flash_attention.rs:51-56).  Scores, soft-max state and output accumulation are
+ * binary32.
+ */
+#ifndef ELLM_ATTN_H_
+#define ELLM_ATTN_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef enum ellm_status {
+  ELLM_OK = 0,
+  ELLM_ERR_INVALID_ARGUMENT = 1, /* null pointer, zero size, bad dtype, strides, ... */
+  ELLM_ERR_UNSUPPORTED = 2,      /* head_size != 128, group size not supported, ...   */
+  ELLM_ERR_OUT_OF_RANGE = 3,     /* position / batch / slot beyond the stated capacity */
+  ELLM_ERR_HIP = 4,              /* a HIP runtime call failed; see ellm_last_error_string */
+  ELLM_ERR_NO_DEVICE = 5         /* no gfx950 device visible                           */
+} ellm_status;
+
+typedef enum ellm_dtype {
+  ELLM_DTYPE_F16 = 0,
+  ELLM_DTYPE_BF16 = 1
+} ellm_dtype;
+
+/* Message for the last non-OK status returned on the calling thread. */
+const char* ellm_last_error_string(void);
+
+/* Library version (major*10000 + minor*100 + patch). */
+int ellm_attn_version(void);
+
+/* Number of visible devices this library can run on (gfx950); 0 when none.
+ * Never fails: returns 0 on any HIP error. */
+int ellm_device_count(void);
+
+/* ------------------------------------------------------------------------ *
+ * Attention operator
+ * ------------------------------------------------------------------------ */
+
+/*
+ * Mirrors the argument list of Attention::new (src/compiler/mul/attention.rs:41-54)
+ * as called from Tensor::attention (src/ptensor/tensor.rs:123-135):
+ *
+ *   q, out : device, [position_interval][batch_capacity][attention_head_num][head_size],
+ *            row-major (src/compiler/mul/attention.rs:78, 116-119).
+ *   k, v   : device, viewed as [sequence][kv_head][position][head_size] through
+ *            kv_strides (elements): kv_strides[0] per sequence, [1] per kv head,
+ *            [2] per position, [3] must be 1.  The dimension-first cache of this
+ *            library has kv_strides = {kv_heads*capacity*128, capacity*128, 128, 1}.
+ *   inverse_sqrt_head : soft-max scale applied to q.k (attention.rs:52, 66).
+ *
+ * Additions the reference does not have:
+ *   lse    : optional device [position_interval][batch_capacity][attention_head_num]
+ *            float, receives log(sum_j exp(scale * q.k_j)) per query row.
+ *   dtype, sequence_capacity (positions per K/V plane; run() rejects positions
+ *            at or beyond it), max_position_interval (largest position_interval
+ *            run() will be given; sizes q/out).
+ */
+typedef struct ellm_attn_desc {
+  const void* q;
+  const void* k;
+  const void* v;
+  void* out;
+  float* lse; /* may be NULL */
+  size_t batch_size; /* capacity in sequences: the Q/O row pitch, as in the reference */
+  size_t attention_head_num;
+  size_t kv_head_num;
+  size_t head_size;
+  size_t kv_strides[4];
+  float inverse_sqrt_head;
+  int dtype; /* ellm_dtype */
+  size_t sequence_capacity;
+  size_t max_position_interval;
+} ellm_attn_desc;
+
+typedef struct ellm_attn ellm_attn;
+
+/* Validates the description and allocates the operator's own workspace (split
+ * partial results for the single-token path).  Borrowed pointers are not owned. */
+int ellm_attn_create(const ellm_attn_desc* desc, ellm_attn** out_handle);
+
+/* Frees the handle and its workspace only.  NULL is accepted. */
+int ellm_attn_destroy(ellm_attn* handle);
+
+/*
+ * Attention::run (src/compiler/mul/attention.rs:69-76) without the cpu_num /
+ * thread_id pair: queries at positions [position_index, position_index +
+ * position_interval) of the first batch_size sequences; the query at position p
+ * attends to keys 0..=p of its own sequence (flash_attention.rs:57-58).
+ * position_interval == 1 takes the split-KV single-token kernel, larger
+ * intervals the tiled MFMA kernel.  Zero batch_size or position_interval is a
+ * no-op returning ELLM_OK.
+ */
+int ellm_attn_run(ellm_attn* handle, size_t position_index, size_t position_interval,
+                  size_t batch_size, void* stream);
+
+/*
+ * Single-token step with one position per sequence (the reference has a single
+ * shared position_index, which cannot express sequences of different lengths).
+ * positions: device, batch_size uint32 values; sequence i attends to keys
+ * 0..=positions[i].  max_position: an upper bound (inclusive) on every entry,
+ * known on the host; it sizes the launch.  Entries above max_position or at or
+ * beyond sequence_capacity are clamped to that bound on the device.
+ */
+int ellm_attn_run_ragged(ellm_attn* handle, const uint32_t* positions, size_t max_position,
+                         size_t batch_size, void* stream);
+
+/* ------------------------------------------------------------------------ *
+ * Key/value cache: one allocation, [layer][sequence][kv_head][position][128],
+ * for keys and one for values, written in place at token coordinates.
+ * Replaces the per-layer "key_position_tensor" / "value_tensor" buffers of
+ * memory::Cache (src/memory/cache.rs:23, 69-75) and the 64-byte aligned,
+ * zero-filled, never-moved allocation of src/memory/allocator.rs:4-27.
+ * ------------------------------------------------------------------------ */
+
+typedef struct ellm_kv_cache ellm_kv_cache;
+
+typedef struct ellm_kv_desc {
+  size_t layers;
+  size_t sequences;  /* slots */
+  size_t kv_head_num;
+  size_t head_size;  /* 128 */
+  size_t capacity;   /* positions per plane */
+  int dtype;         /* ellm_dtype */
+} ellm_kv_desc;
+
+/* Allocates and zero-fills both tensors on the current device. */
+int ellm_kv_create(const ellm_kv_desc* desc, ellm_kv_cache** out_cache);
+int ellm_kv_destroy(ellm_kv_cache* cache);
+
+/* Device base pointers of one layer's K and V ([sequence][kv_head][position][128])
+ * and the four element strides to hand to ellm_attn_desc.kv_strides. */
+int ellm_kv_layer(const ellm_kv_cache* cache, size_t layer, void** k, void** v,
+                  size_t kv_strides[4]);
+
+/*
+ * Writes n_tokens new positions [position_index, position_index + n_tokens) of
+ * sequences [0, batch_size) of one layer.  k_src / v_src: device,
+ * [n_tokens][src_batch_pitch][kv_head_num][128] — the layout in which the
+ * projection produces them (src/qwen3_moe/attention.rs:142-166, before its
+ * permute).  src_batch_pitch is the source's sequence capacity (>= batch_size).
+ */
+int ellm_kv_append(ellm_kv_cache* cache, size_t layer, size_t position_index, size_t n_tokens,
+                   size_t batch_size, const void* k_src, const void* v_src,
+                   size_t src_batch_pitch, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* ELLM_ATTN_H_ */

@@ -1,0 +1,192 @@
+"""ctypes access to the CPU oracle (oracle/libellm_oracle.so) for the tests.
+
+The oracle is test infrastructure: it restates the reference's attention
+arithmetic in binary32 and is only ever used as the checker.
+"""
+import ctypes
+import os
+import subprocess
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+ORACLE_DIR = os.path.join(ROOT, "oracle")
+ORACLE_SO = os.path.join(ORACLE_DIR, "libellm_oracle.so")
+
+F16, BF16, F32 = 0, 1, 2
+
+
+class OracleAttn(ctypes.Structure):
+    _fields_ = [
+        ("q", ctypes.c_void_p),
+        ("k", ctypes.c_void_p),
+        ("v", ctypes.c_void_p),
+        ("out", ctypes.c_void_p),
+        ("lse", ctypes.c_void_p),
+        ("batch_capacity", ctypes.c_size_t),
+        ("attention_head_num", ctypes.c_size_t),
+        ("kv_head_num", ctypes.c_size_t),
+        ("head_size", ctypes.c_size_t),
+        ("kv_strides", ctypes.c_size_t * 4),
+        ("inverse_sqrt_head", ctypes.c_float),
+        ("dtype", ctypes.c_int),
+    ]
+
+
+_lib = None
+
+
+def load():
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(ORACLE_SO):
+        subprocess.check_call(["make", "-C", ORACLE_DIR])
+    lib = ctypes.CDLL(ORACLE_SO)
+    sz, vp, f = ctypes.c_size_t, ctypes.c_void_p, ctypes.c_float
+    lib.ellm_oracle_dot_product_f32.restype = f
+    lib.ellm_oracle_dot_product_f32.argtypes = [vp, vp, sz]
+    lib.ellm_oracle_scalar_vector_mul_and_acc_f32.restype = None
+    lib.ellm_oracle_scalar_vector_mul_and_acc_f32.argtypes = [f, vp, f, vp, sz]
+    lib.ellm_oracle_scale_softmax_f32.restype = None
+    lib.ellm_oracle_scale_softmax_f32.argtypes = [vp, vp, sz, f]
+    lib.ellm_oracle_flash_attention.restype = None
+    lib.ellm_oracle_flash_attention.argtypes = [vp, vp, vp, vp, vp, f, sz, sz, sz, ctypes.c_int]
+    lib.ellm_oracle_assign.restype = ctypes.c_int
+    lib.ellm_oracle_assign.argtypes = [sz, sz, sz, ctypes.POINTER(sz), ctypes.POINTER(sz)]
+    lib.ellm_oracle_attention_run.restype = ctypes.c_int
+    lib.ellm_oracle_attention_run.argtypes = [ctypes.POINTER(OracleAttn), sz, sz, sz, vp, sz, sz]
+    lib.ellm_oracle_attention_run_threads.restype = ctypes.c_double
+    lib.ellm_oracle_attention_run_threads.argtypes = [
+        ctypes.POINTER(OracleAttn), sz, sz, sz, vp, sz, ctypes.c_int, sz]
+    lib.ellm_oracle_attention_rows_threads.restype = ctypes.c_double
+    lib.ellm_oracle_attention_rows_threads.argtypes = [
+        ctypes.POINTER(OracleAttn), sz, vp, sz, vp, vp, sz]
+    lib.ellm_oracle_f32_to_f16.restype = ctypes.c_uint16
+    lib.ellm_oracle_f32_to_f16.argtypes = [f]
+    lib.ellm_oracle_f16_to_f32.restype = f
+    lib.ellm_oracle_f16_to_f32.argtypes = [ctypes.c_uint16]
+    lib.ellm_oracle_f32_to_bf16.restype = ctypes.c_uint16
+    lib.ellm_oracle_f32_to_bf16.argtypes = [f]
+    lib.ellm_oracle_bf16_to_f32.restype = f
+    lib.ellm_oracle_bf16_to_f32.argtypes = [ctypes.c_uint16]
+    lib.ellm_oracle_barrier_selftest.restype = ctypes.c_int
+    lib.ellm_oracle_barrier_selftest.argtypes = [sz, sz]
+    _lib = lib
+    return lib
+
+
+def _ptr(a):
+    return ctypes.c_void_p(a.ctypes.data) if a is not None else None
+
+
+# ---- storage conversions on numpy arrays (bit patterns in uint16) -------------
+
+def to_storage(x32, dtype):
+    """binary32 array -> storage array (float16 / uint16 bf16 bits / float32)."""
+    x32 = np.ascontiguousarray(x32, dtype=np.float32)
+    if dtype == F16:
+        return x32.astype(np.float16)
+    if dtype == BF16:
+        u = x32.view(np.uint32).astype(np.uint64)
+        u = (u + 0x7FFF + ((u >> 16) & 1)) >> 16
+        return u.astype(np.uint16)
+    return x32
+
+
+def from_storage(a, dtype):
+    if dtype == F16:
+        return np.asarray(a).view(np.float16).astype(np.float32)
+    if dtype == BF16:
+        return (np.asarray(a).view(np.uint16).astype(np.uint32) << 16).view(np.float32)
+    return np.asarray(a, dtype=np.float32)
+
+
+def storage_np_dtype(dtype):
+    return {F16: np.float16, BF16: np.uint16, F32: np.float32}[dtype]
+
+
+def assign(length, num, idx):
+    lib = load()
+    b, e = ctypes.c_size_t(), ctypes.c_size_t()
+    ok = lib.ellm_oracle_assign(length, num, idx, ctypes.byref(b), ctypes.byref(e))
+    return (b.value, e.value) if ok else None
+
+
+def flash_attention_row(q, K, V, scale, position, dtype, stride=None, o_init=None):
+    """One query row against rows 0..=position of K/V (storage arrays). Returns (o, lse)."""
+    lib = load()
+    length = q.shape[-1]
+    stride = stride if stride is not None else length
+    o = np.zeros(length, dtype=storage_np_dtype(dtype)) if o_init is None else o_init.copy()
+    lse = np.zeros(1, dtype=np.float32)
+    lib.ellm_oracle_flash_attention(_ptr(q), _ptr(K), _ptr(V), _ptr(o), _ptr(lse),
+                                    ctypes.c_float(scale), length, stride, position, dtype)
+    return o, float(lse[0])
+
+
+class Operator:
+    """The oracle's Attention operator over numpy storage arrays.
+
+    q/out: [interval, batch_capacity, heads, D]; k/v: [sequence, kv_head, capacity, D]
+    (or any layout described by kv_strides, in elements).
+    """
+
+    def __init__(self, q, k, v, out, lse, batch_capacity, heads, kv_heads, head_size, kv_strides,
+                 scale, dtype):
+        self.keep = (q, k, v, out, lse)
+        d = OracleAttn()
+        d.q, d.k, d.v, d.out = q.ctypes.data, k.ctypes.data, v.ctypes.data, out.ctypes.data
+        d.lse = lse.ctypes.data if lse is not None else None
+        d.batch_capacity, d.attention_head_num, d.kv_head_num, d.head_size = (
+            batch_capacity, heads, kv_heads, head_size)
+        for i in range(4):
+            d.kv_strides[i] = int(kv_strides[i])
+        d.inverse_sqrt_head = scale
+        d.dtype = dtype
+        self.desc = d
+
+    def run(self, position_index, position_interval, batch_size, cpu_num=1, thread_id=0,
+            positions=None):
+        rc = load().ellm_oracle_attention_run(ctypes.byref(self.desc), position_index,
+                                              position_interval, batch_size, _ptr(positions),
+                                              cpu_num, thread_id)
+        if rc:
+            raise RuntimeError("oracle rejected the arguments")
+
+    def run_threads(self, position_index, position_interval, batch_size, n_threads,
+                    positions=None, pin=False, repeats=1):
+        t = load().ellm_oracle_attention_run_threads(ctypes.byref(self.desc), position_index,
+                                                     position_interval, batch_size,
+                                                     _ptr(positions), n_threads, int(pin), repeats)
+        if t < 0:
+            raise RuntimeError("oracle rejected the arguments")
+        return t
+
+    def run_rows(self, position_index, rows, n_threads):
+        """rows: uint32 [n, 3] of (token_in_chunk, sequence, head). Returns (out_rows, lse, secs)."""
+        rows = np.ascontiguousarray(rows, dtype=np.uint32)
+        n = rows.shape[0]
+        out = np.zeros((n, self.desc.head_size), dtype=storage_np_dtype(self.desc.dtype))
+        lse = np.zeros(n, dtype=np.float32)
+        t = load().ellm_oracle_attention_rows_threads(ctypes.byref(self.desc), position_index,
+                                                      _ptr(rows), n, _ptr(out), _ptr(lse),
+                                                      n_threads)
+        if t < 0:
+            raise RuntimeError("oracle rejected the arguments")
+        return out, lse, t
+
+
+def attention(q, k, v, scale, dtype, position_index=0, positions=None, n_threads=8, batch=None):
+    """Convenience: run the whole operator on numpy storage arrays.
+
+    q: [S, Bcap, Hq, D]; k, v: [B, Hkv, cap, D] contiguous.  Returns (out, lse[S, Bcap, Hq]).
+    """
+    S, bcap, hq, D = q.shape
+    hkv, cap = k.shape[1], k.shape[2]
+    out = np.zeros_like(q)
+    lse = np.zeros((S, bcap, hq), dtype=np.float32)
+    op = Operator(q, k, v, out, lse, bcap, hq, hkv, D, [hkv * cap * D, cap * D, D, 1], scale, dtype)
+    op.run_threads(position_index, S, batch if batch is not None else bcap, n_threads,
+                   positions=positions)
+    return out, lse
