@@ -1,0 +1,241 @@
+#!/usr/bin/env python3
+"""Benchmark of the attention hot path on one MI355X.
+
+Primary workload (the JSON line's value): single-token attention, Qwen3-30B-A3B
+shapes — 16 sequences x 8192 cached tokens, 32 query / 4 KV heads, head_dim 128,
+fp16, dimension-first cache.  One step = one Attention::run(position 8191,
+interval 1, batch 16).  K/V are already resident in HBM; four cache copies are
+rotated between steps so a step never re-reads lines still sitting in the
+256 MB infinity cache.
+
+Also reported on the same line (`also`): the 32k-token causal GQA prefill
+(TFLOP/s against the dense fp16 MFMA peak) and single-token attention over one
+128k-token cache.
+
+`cpu_baseline` times the CPU oracle (a port of the reference's per-row
+recurrence, binary32) on this machine's host cores.
+
+Usage: python bench.py [--gpus 1] [--steps K] [--warmup W] [--skip-cpu] [--only NAME]
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+sys.path.insert(0, os.path.join(ROOT, "tests"))
+
+HBM_PEAK_GBS = 8000.0       # MI355X HBM3E, published
+MFMA_F16_PEAK_TFLOPS = 2500.0  # MI355X dense fp16/bf16 MFMA, published
+D = 128
+
+
+def _dev_normal(shape, dtype, seed, scale=1.0):
+    import torch
+
+    g = torch.Generator(device="cuda")
+    g.manual_seed(seed)
+    x = torch.randn(shape, generator=g, device="cuda", dtype=torch.float32)
+    if scale != 1.0:
+        x *= scale
+    return x.to(dtype)
+
+
+def _time_steps(fn, steps, warmup):
+    """Per-step durations (ms) from HIP events recorded on the launch stream."""
+    import torch
+
+    for i in range(warmup):
+        fn(i)
+    torch.cuda.synchronize()
+    starts = [torch.cuda.Event(enable_timing=True) for _ in range(steps)]
+    stops = [torch.cuda.Event(enable_timing=True) for _ in range(steps)]
+    t0 = time.perf_counter()
+    for i in range(steps):
+        starts[i].record()
+        fn(warmup + i)
+        stops[i].record()
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3
+    per = [s.elapsed_time(e) for s, e in zip(starts, stops)]
+    whole_ms = starts[0].elapsed_time(stops[-1])
+    return per, whole_ms, wall_ms
+
+
+def bench_decode(batch, length, steps, warmup, hq=32, hkv=4, copies=4):
+    import torch
+
+    import ellm_amd
+
+    cap = length
+    scale = 1.0 / D ** 0.5
+    ops = []
+    for c in range(copies):
+        k = _dev_normal((batch, hkv, cap, D), torch.float16, 100 + c)
+        v = _dev_normal((batch, hkv, cap, D), torch.float16, 200 + c)
+        q = _dev_normal((1, batch, hq, D), torch.float16, 300 + c)
+        out = torch.zeros_like(q)
+        lse = torch.zeros((1, batch, hq), dtype=torch.float32, device="cuda")
+        op = ellm_amd.Attention(q, k, v, out, batch, hq, hkv, D, [hkv * cap * D, cap * D, D, 1],
+                                scale, lse=lse, sequence_capacity=cap, max_position_interval=1)
+        ops.append(op)
+    per, whole_ms, _ = _time_steps(lambda i: ops[i % copies].run(length - 1, 1, batch), steps, warmup)
+    alg_bytes = 2 * batch * hkv * length * D * 2 + 2 * batch * hq * D * 2
+    step_ms = whole_ms / steps
+    kern_ms = sum(per) / len(per)
+    for op in ops:
+        op.close()
+    return {
+        "alg_bytes": alg_bytes,
+        "ms_per_step": step_ms,
+        "kernel_ms": kern_ms,
+        "gbs": alg_bytes / (step_ms * 1e-3) / 1e9,
+        "kernel_gbs": alg_bytes / (kern_ms * 1e-3) / 1e9,
+    }
+
+
+def bench_prefill(seq, steps, warmup, hq=32, hkv=4, dtype_name="f16", p0=0):
+    import torch
+
+    import ellm_amd
+
+    dt = torch.float16 if dtype_name == "f16" else torch.bfloat16
+    cap = p0 + seq
+    scale = 1.0 / D ** 0.5
+    g = torch.Generator(device="cuda")
+    g.manual_seed(5)
+    qs = torch.rand((1, 1, hq, 1), generator=g, device="cuda") * 1.5 + 0.5   # per-head scale U[0.5, 2]
+    ks = torch.rand((1, hkv, 1, 1), generator=g, device="cuda") * 1.5 + 0.5
+    q = (_dev_normal((seq, 1, hq, D), torch.float32, 11) * qs).to(dt)
+    k = (_dev_normal((1, hkv, cap, D), torch.float32, 12) * ks).to(dt)
+    v = (_dev_normal((1, hkv, cap, D), torch.float32, 13) * ks).to(dt)
+    out = torch.zeros_like(q)
+    lse = torch.zeros((seq, 1, hq), dtype=torch.float32, device="cuda")
+    op = ellm_amd.Attention(q, k, v, out, 1, hq, hkv, D, [hkv * cap * D, cap * D, D, 1], scale,
+                            lse=lse, sequence_capacity=cap, max_position_interval=seq)
+    per, whole_ms, _ = _time_steps(lambda i: op.run(p0, seq, 1), steps, warmup)
+    flops = 4 * D * hq * (seq * p0 + seq * (seq + 1) // 2)
+    step_ms = whole_ms / steps
+    kern_ms = sum(per) / len(per)
+    op.close()
+    return {
+        "flops": flops,
+        "ms_per_step": step_ms,
+        "kernel_ms": kern_ms,
+        "tflops": flops / (step_ms * 1e-3) / 1e12,
+        "kernel_tflops": flops / (kern_ms * 1e-3) / 1e12,
+    }
+
+
+def cpu_baseline_decode(batch, length, hq=32, hkv=4, budget_s=20.0):
+    """The CPU oracle on the full single-token workload (all host cores)."""
+    import numpy as np
+    import oracle_lib as orc
+
+    cores = min(os.cpu_count() or 1, 16)
+    rng = np.random.default_rng(1)
+    q = rng.standard_normal((1, batch, hq, D), dtype=np.float32).astype(np.float16)
+    k = rng.standard_normal((batch, hkv, length, D), dtype=np.float32).astype(np.float16)
+    v = rng.standard_normal((batch, hkv, length, D), dtype=np.float32).astype(np.float16)
+    out = np.zeros_like(q)
+    op = orc.Operator(q, k, v, out, None, batch, hq, hkv, D, [hkv * length * D, length * D, D, 1],
+                      1.0 / D ** 0.5, orc.F16)
+    t1 = op.run_threads(length - 1, 1, batch, cores, pin=False)
+    repeats = max(1, min(10, int(budget_s / max(t1, 1e-3)) - 1))
+    t = op.run_threads(length - 1, 1, batch, cores, pin=False, repeats=repeats) / repeats
+    alg_bytes = 2 * batch * hkv * length * D * 2 + 2 * batch * hq * D * 2
+    return {
+        "value": alg_bytes / t / 1e9,
+        "unit": "GB/s",
+        "cores": cores,
+        "kind": "port",
+        "sample": f"full workload ({batch} seq x {length} keys x {hq} heads), {repeats} passes, "
+                  f"{t * 1e3:.1f} ms per pass, one thread per core with the reference's static split",
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--skip-cpu", action="store_true")
+    ap.add_argument("--only", default="", help="decode | prefill | decode128k")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on one GPU only (no collectives); use --gpus 1",
+              file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+
+    import ellm_amd
+
+    ellm_amd.load_library()  # fail loudly if the HIP library is missing
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(1)
+
+    also = []
+    dec = None
+    if args.only in ("", "decode"):
+        dec = bench_decode(16, 8192, args.steps, args.warmup)
+    if args.only in ("", "prefill"):
+        pf_steps = max(3, min(args.steps, 10))
+        pf = bench_prefill(32768, pf_steps, min(args.warmup, 2))
+        also.append({
+            "workload": "prefill: 1 seq x 32768 tokens, 32q/4kv heads, fp16, causal",
+            "metric": "prefill attn TFLOP/s", "value": round(pf["tflops"], 2), "unit": "TFLOP/s",
+            "ms_per_step": round(pf["ms_per_step"], 4), "steps": pf_steps,
+            "roofline": {"bound": "mfma", "achieved": round(pf["kernel_tflops"], 2),
+                         "peak": MFMA_F16_PEAK_TFLOPS, "unit": "TFLOP/s",
+                         "frac": round(pf["kernel_tflops"] / MFMA_F16_PEAK_TFLOPS, 4),
+                         "traffic": None},
+        })
+    if args.only in ("", "decode128k"):
+        d128 = bench_decode(1, 131072, args.steps, args.warmup)
+        also.append({
+            "workload": "decode: 1 seq x 131072 cached tokens, 32q/4kv heads, fp16",
+            "metric": "decode attn HBM GB/s", "value": round(d128["gbs"], 1), "unit": "GB/s",
+            "ms_per_step": round(d128["ms_per_step"], 5), "steps": args.steps,
+            "roofline": {"bound": "hbm", "achieved": round(d128["kernel_gbs"], 1),
+                         "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                         "frac": round(d128["kernel_gbs"] / HBM_PEAK_GBS, 4), "traffic": None},
+        })
+
+    cpu = None
+    if not args.skip_cpu and dec is not None:
+        cpu = cpu_baseline_decode(16, 8192)
+
+    if dec is None:  # partial run for profiling
+        print(json.dumps({"also": also}))
+        return
+    line = {
+        "metric": "decode attn HBM GB/s (Qwen3 GQA, 1 GPU)",
+        "value": round(dec["gbs"], 1),
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(dec["ms_per_step"], 5),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f16",
+        "data": "synthetic",
+        "config": {"workload": "decode: 16 seq x 8192 cached tokens, 32q/4kv heads, head_dim 128, "
+                               "fp16, dimension-first cache (BASELINE configs[1])",
+                   "batch": 16, "cache_len": 8192, "q_heads": 32, "kv_heads": 4},
+        "roofline": {"bound": "hbm", "achieved": round(dec["kernel_gbs"], 1), "peak": HBM_PEAK_GBS,
+                     "unit": "GB/s", "frac": round(dec["kernel_gbs"] / HBM_PEAK_GBS, 4),
+                     "traffic": None},
+        "cpu_baseline": cpu,
+        "also": also,
+    }
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

@@ -50,7 +50,10 @@ struct ellm_attn {
   int n_cu;
   float* ws_acc;
   float* ws_ml;
-  size_t ws_rows;
+  float* ws2_acc;
+  float* ws2_ml;
+  uint32_t* counters;
+  ellm::DecodeWorkspace ws;
 };
 
 struct ellm_kv_cache {
@@ -59,6 +62,19 @@ struct ellm_kv_cache {
   void* v;
   size_t layer_elems;  // elements per layer
 };
+
+static hipError_t free_workspace(ellm_attn* h) {
+  hipError_t first = hipSuccess;
+  void* ptrs[] = {h->ws_acc, h->ws_ml, h->ws2_acc, h->ws2_ml, h->counters};
+  for (void* p : ptrs) {
+    if (!p) continue;
+    hipError_t e = hipFree(p);
+    if (e != hipSuccess && first == hipSuccess) first = e;
+  }
+  h->ws_acc = h->ws_ml = h->ws2_acc = h->ws2_ml = nullptr;
+  h->counters = nullptr;
+  return first;
+}
 
 extern "C" {
 
@@ -127,14 +143,19 @@ int ellm_attn_create(const ellm_attn_desc* d, ellm_attn** out_handle) {
   if (!h) return fail(ELLM_ERR_INVALID_ARGUMENT, "out of host memory");
   h->desc = *d;
   h->n_cu = n_cu;
-  h->ws_rows = ellm::decode_workspace_rows((uint32_t)d->batch_size, (uint32_t)d->attention_head_num,
-                                           (uint32_t)d->kv_head_num, (uint32_t)n_cu);
-  h->ws_acc = nullptr;
-  h->ws_ml = nullptr;
-  hipError_t e = hipMalloc((void**)&h->ws_acc, h->ws_rows * 128 * sizeof(float));
-  if (e == hipSuccess) e = hipMalloc((void**)&h->ws_ml, h->ws_rows * 2 * sizeof(float));
+  h->ws = ellm::decode_workspace((uint32_t)d->batch_size, (uint32_t)d->attention_head_num,
+                                 (uint32_t)d->kv_head_num, (uint32_t)n_cu);
+  h->ws_acc = h->ws_ml = h->ws2_acc = h->ws2_ml = nullptr;
+  h->counters = nullptr;
+  hipError_t e = hipMalloc((void**)&h->ws_acc, h->ws.rows * 128 * sizeof(float));
+  if (e == hipSuccess) e = hipMalloc((void**)&h->ws_ml, h->ws.rows * 2 * sizeof(float));
+  if (e == hipSuccess) e = hipMalloc((void**)&h->ws2_acc, h->ws.rows2 * 128 * sizeof(float));
+  if (e == hipSuccess) e = hipMalloc((void**)&h->ws2_ml, h->ws.rows2 * 2 * sizeof(float));
+  // arrival counters of the single-token kernel; they return to zero by themselves
+  if (e == hipSuccess) e = hipMalloc((void**)&h->counters, h->ws.counters * sizeof(uint32_t));
+  if (e == hipSuccess) e = hipMemset(h->counters, 0, h->ws.counters * sizeof(uint32_t));
   if (e != hipSuccess) {
-    if (h->ws_acc) (void)hipFree(h->ws_acc);
+    free_workspace(h);
     delete h;
     return fail_hip(e, "hipMalloc(workspace)");
   }
@@ -144,11 +165,9 @@ int ellm_attn_create(const ellm_attn_desc* d, ellm_attn** out_handle) {
 
 int ellm_attn_destroy(ellm_attn* h) {
   if (!h) return ELLM_OK;
-  hipError_t e1 = hipFree(h->ws_acc);
-  hipError_t e2 = hipFree(h->ws_ml);
+  hipError_t e = free_workspace(h);
   delete h;
-  if (e1 != hipSuccess) return fail_hip(e1, "hipFree");
-  if (e2 != hipSuccess) return fail_hip(e2, "hipFree");
+  if (e != hipSuccess) return fail_hip(e, "hipFree");
   return ELLM_OK;
 }
 
@@ -171,6 +190,9 @@ static void fill_args(const ellm_attn* h, ellm::AttnArgs* a) {
   a->capacity = (uint32_t)d.sequence_capacity;
   a->ws_acc = h->ws_acc;
   a->ws_ml = h->ws_ml;
+  a->ws2_acc = h->ws2_acc;
+  a->ws2_ml = h->ws2_ml;
+  a->counters = h->counters;
   a->positions = nullptr;
 }
 
@@ -179,7 +201,7 @@ static int run_decode(ellm_attn* h, ellm::AttnArgs* a, uint32_t max_position, hi
       ellm::decode_plan(max_position + 1, a->batch, a->n_kv_heads, (uint32_t)h->n_cu);
   a->split_len = plan.split_len;
   a->n_split = plan.n_split;
-  if ((size_t)a->batch * a->n_q_heads * a->n_split > h->ws_rows)
+  if (!ellm::decode_plan_fits(h->ws, a->batch, a->n_q_heads, a->n_kv_heads, a->group, a->n_split))
     return fail(ELLM_ERR_OUT_OF_RANGE, "internal: split plan exceeds the workspace");
   hipError_t e = ellm::launch_decode(*a, stream);
   if (e != hipSuccess) return fail_hip(e, "single-token attention launch");

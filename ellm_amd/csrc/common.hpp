@@ -16,6 +16,7 @@ typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
 typedef short s16x4 __attribute__((ext_vector_type(4)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
@@ -50,10 +51,15 @@ struct Mfma<F16> {
     return __builtin_amdgcn_mfma_f32_16x16x16f16(__builtin_bit_cast(f16x4, a),
                                                  __builtin_bit_cast(f16x4, b), c, 0, 0, 0);
   }
-  // two binary32 -> packed pair, round to nearest even
+  // two binary32 -> packed pair, round to nearest even (v_cvt_pk_f16_f32)
   static __device__ __forceinline__ uint32_t pack2(float lo, float hi) {
-    f16x2 v = {(_Float16)lo, (_Float16)hi};
-    return __builtin_bit_cast(uint32_t, v);
+    f32x2 x = {lo, hi};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(x, f16x2));
+  }
+  // acc + lo + hi of a packed pair, accumulated in binary32 (v_dot2c_f32_f16)
+  static __device__ __forceinline__ float add_pair(uint32_t packed, float acc) {
+    const f16x2 ones = {(_Float16)1.0f, (_Float16)1.0f};
+    return __builtin_amdgcn_fdot2(__builtin_bit_cast(f16x2, packed), ones, acc, false);
   }
   static __device__ __forceinline__ float to_float(uint16_t bits) {
     return (float)__builtin_bit_cast(_Float16, bits);
@@ -75,8 +81,12 @@ struct Mfma<BF16> {
                                                      __builtin_bit_cast(s16x4, b), c, 0, 0, 0);
   }
   static __device__ __forceinline__ uint32_t pack2(float lo, float hi) {
-    bf16x2 v = {(__bf16)lo, (__bf16)hi};
-    return __builtin_bit_cast(uint32_t, v);
+    f32x2 x = {lo, hi};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(x, bf16x2));
+  }
+  static __device__ __forceinline__ float add_pair(uint32_t packed, float acc) {
+    const bf16x2 ones = {(__bf16)1.0f, (__bf16)1.0f};
+    return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, packed), ones, acc, false);
   }
   static __device__ __forceinline__ float to_float(uint16_t bits) {
     return __builtin_bit_cast(float, (uint32_t)bits << 16);

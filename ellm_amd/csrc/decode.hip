@@ -19,8 +19,11 @@
 //   V is transposed on the way into LDS with 4-key x 8-dim register blocks.
 //   Soft-max state (running max, denominator) is one scalar per lane.
 //   At the end the four waves are merged through LDS; with more than one split
-//   the partial (max, sum, acc[128]) goes to the workspace and merge_kernel
-//   combines the splits.
+//   the partial (max, sum, acc[128]) goes to the workspace, and the workgroup
+//   that finishes last for a (sequence, head group) combines that group's
+//   splits (a self-resetting arrival counter per group; no second launch).
+#include <cstdlib>
+
 #include "common.hpp"
 #include "kernels.hpp"
 
@@ -33,6 +36,7 @@ constexpr int kKPitch = kHeadDim + 8;           // halves per K row in LDS (272 
 constexpr int kVtPitch = kChunk + 4;            // halves per V^T row in LDS (40 B)
 constexpr int kWaveLdsHalves = kChunk * kKPitch + kHeadDim * kVtPitch;
 constexpr int kMaxHeadsPerGroup = 16;
+constexpr int kMergeFan = 16;                   // partials folded per merge step
 
 struct DecodeKernelArgs {
   const uint16_t* q;
@@ -43,6 +47,12 @@ struct DecodeKernelArgs {
   const uint32_t* positions;
   float* ws_acc;
   float* ws_ml;
+  float* ws2_acc;      // cluster partials [sequence][query head][n_cluster_max][128]
+  float* ws2_ml;
+  uint32_t* counters;  // per (sequence, kv head, head group): [0] clusters done, [1 + c] splits of
+                       // cluster c done; all zero between launches
+  uint32_t counters_per_plane, n_cluster_max;
+  uint32_t rotate;
   size_t kv_stride_seq, kv_stride_head, kv_stride_pos;
   uint32_t n_q_heads, n_kv_heads, group, head_groups;
   uint32_t position;  // shared position (positions == null) or upper bound
@@ -50,8 +60,38 @@ struct DecodeKernelArgs {
   float scale_log2;   // scale * log2(e)
 };
 
+// Agent-scope (device-wide coherent) relaxed store / load of one float.
+__device__ __forceinline__ void store_coherent(float* p, float v) {
+  __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ float load_coherent(const float* p) {
+  return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ uint64_t load_coherent64(const float* p) {
+  return __hip_atomic_load((const uint64_t*)p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ void store_coherent64(float* p, float lo, float hi) {
+  const uint64_t bits = (uint64_t)__builtin_bit_cast(uint32_t, lo) |
+                        ((uint64_t)__builtin_bit_cast(uint32_t, hi) << 32);
+  __hip_atomic_store((uint64_t*)p, bits, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+// Block until every vector-memory operation this wave has issued is complete
+// (s_waitcnt vmcnt(0); expcnt and lgkmcnt left at their maxima).
+__device__ __forceinline__ void wait_vm_done() { __builtin_amdgcn_s_waitcnt(0x0F70); }
+
+// Final value of one output element: normalise, round to the storage type, and
+// (thread d == 0) write the row's log-sum-exp in natural-log units.
 template <typename T>
-__global__ __launch_bounds__(kDecWaves* kWave) void decode_split_kernel(DecodeKernelArgs p) {
+__device__ __forceinline__ void store_row_elem(const DecodeKernelArgs& p, uint32_t seq,
+                                               uint32_t head, uint32_t d, float a, float lsum,
+                                               float mmax) {
+  const size_t row = (size_t)seq * p.n_q_heads + head;
+  p.out[row * kHeadDim + d] = (uint16_t)(Mfma<T>::pack2(a / lsum, 0.0f) & 0xffffu);
+  if (p.lse && d == 0) p.lse[row] = (mmax + fast_log2(lsum)) * kLn2;
+}
+
+template <typename T>
+__global__ __launch_bounds__(kDecWaves* kWave, 4) void decode_split_kernel(DecodeKernelArgs p) {
   __shared__ __attribute__((aligned(16))) uint16_t smem[kDecWaves * kWaveLdsHalves];
 
   const uint32_t split = blockIdx.x;
@@ -67,8 +107,8 @@ __global__ __launch_bounds__(kDecWaves* kWave) void decode_split_kernel(DecodeKe
   const uint32_t k_begin = split * p.split_len;
   const uint32_t k_end = min(len, k_begin + p.split_len);
   const uint32_t heads_here = min((uint32_t)kMaxHeadsPerGroup, p.group - hgrp * kMaxHeadsPerGroup);
-  // A split that starts beyond this sequence's keys has nothing to add; the
-  // merge kernel derives the number of live splits from the same length.
+  // A split that starts beyond this sequence's keys has nothing to add and is
+  // not counted: the merge below derives the live split count from the length.
   if (k_begin >= len) return;
 
   const uint16_t* kplane = p.k + seq * p.kv_stride_seq + kvh * p.kv_stride_head;
@@ -112,9 +152,20 @@ __global__ __launch_bounds__(kDecWaves* kWave) void decode_split_kernel(DecodeKe
 #pragma unroll
   for (int b = 0; b < 8; ++b) acc[b] = f32x4{0, 0, 0, 0};
 
-  uint32_t chunk = wave;
-  if (chunk < n_chunks) issue_loads(chunk);
-  for (; chunk < n_chunks; chunk += kDecWaves) {
+  // Chunks are visited in a rotated order that differs from workgroup to
+  // workgroup (soft-max accumulation does not care about order): all splits
+  // start at offsets that are multiples of split_len, and walking them in
+  // lockstep would keep every stream on the same few HBM channels.
+  const uint32_t my_chunks = (n_chunks > (uint32_t)wave) ? (n_chunks - wave + kDecWaves - 1) / kDecWaves : 0;
+  const uint32_t rot = p.rotate ? ((split * 7u + blockIdx.y * 3u + seq * 5u) % max(my_chunks, 1u)) : 0u;
+  auto chunk_at = [&](uint32_t it) {
+    uint32_t r = it + rot;
+    if (r >= my_chunks) r -= my_chunks;
+    return wave + r * kDecWaves;
+  };
+  if (my_chunks) issue_loads(chunk_at(0));
+  for (uint32_t it = 0; it < my_chunks; ++it) {
+    const uint32_t chunk = chunk_at(it);
     const uint32_t kb = k_begin + chunk * kChunk;
     // registers -> LDS: K row-major, V transposed.
 #pragma unroll
@@ -125,7 +176,7 @@ __global__ __launch_bounds__(kDecWaves* kWave) void decode_split_kernel(DecodeKe
                                 vreg[3][e >> 1], (e & 1) != 0);
       *(u32x2*)(vt + (8 * c + e) * kVtPitch + 4 * g) = col;
     }
-    if (chunk + kDecWaves < n_chunks) issue_loads(chunk + kDecWaves);
+    if (it + 1 < my_chunks) issue_loads(chunk_at(it + 1));
     __builtin_amdgcn_wave_barrier();
 
     // S^T[key][head], lane (head c, group g) register r <-> key kb + 4 g + r.
@@ -207,69 +258,175 @@ __global__ __launch_bounds__(kDecWaves* kWave) void decode_split_kernel(DecodeKe
     }
     const uint32_t head = head0 + h;
     if (p.n_split == 1) {
-      const size_t o = ((size_t)seq * p.n_q_heads + head) * kHeadDim + d;
-      const float val = a / lsum;
-      p.out[o] = (uint16_t)(Mfma<T>::pack2(val, 0.0f) & 0xffffu);
-      if (p.lse && d == 0)
-        p.lse[(size_t)seq * p.n_q_heads + head] = (mmax + fast_log2(lsum)) * kLn2;
+      store_row_elem<T>(p, seq, head, d, a, lsum, mmax);
     } else {
       const size_t prow = ((size_t)seq * p.n_q_heads + head) * p.n_split + split;
-      p.ws_acc[prow * kHeadDim + d] = a;
+      store_coherent(p.ws_acc + prow * kHeadDim + d, a);
       if (d == 0) {
-        p.ws_ml[prow * 2] = mmax;
-        p.ws_ml[prow * 2 + 1] = lsum;
+        store_coherent(p.ws_ml + prow * 2, mmax);
+        store_coherent(p.ws_ml + prow * 2 + 1, lsum);
       }
     }
   }
-}
+  if (p.n_split == 1) return;
 
-// One workgroup of 128 threads per (sequence, query head): combine the live
-// splits' (max, sum, acc) into the normalised output row and its log-sum-exp.
-template <typename T>
-__global__ __launch_bounds__(kHeadDim) void merge_kernel(DecodeKernelArgs p) {
-  const uint32_t row = blockIdx.x;  // seq * n_q_heads + head
-  const uint32_t seq = row / p.n_q_heads;
-  const uint32_t d = threadIdx.x;
-  uint32_t pos = p.position;
-  if (p.positions) pos = min(p.positions[seq], p.position);
-  const uint32_t live = min(p.n_split, (pos + p.split_len) / p.split_len);  // ceil((pos+1)/split_len)
-  const float* ml = p.ws_ml + (size_t)row * p.n_split * 2;
-  const float* accp = p.ws_acc + (size_t)row * p.n_split * kHeadDim;
-  float mmax = -INFINITY;
-  for (uint32_t s = 0; s < live; ++s) mmax = fmaxf(mmax, ml[2 * s]);
-  float lsum = 0.0f, a = 0.0f;
-  for (uint32_t s = 0; s < live; ++s) {
-    const float wgt = fast_exp2(ml[2 * s] - mmax);
-    lsum += wgt * ml[2 * s + 1];
-    a += wgt * accp[(size_t)s * kHeadDim + d];
+  // ---- the last workgroup to arrive merges: two levels, 16 partials each -----
+  // Partials are written and read with agent-scope atomic accesses, which go
+  // through to the device-wide point of coherence on their own (each XCD has
+  // its own L2), so no cache write-back or invalidate is needed: a device-scope
+  // fence costs a whole-L2 operation per wave and, with a thousand workgroups,
+  // several times the kernel itself.  Ordering is explicit instead: every thread
+  // waits until its own partial stores have been acknowledged, the workgroup
+  // barrier collects all of them, and only then is the arrival counted; the
+  // merging workgroup issues its loads only after the counter's return value
+  // has been seen by all of its threads.
+  // Splits are grouped in clusters of 16.  The last arrival of a cluster folds
+  // its partials into one cluster partial; the last cluster to finish folds the
+  // cluster partials into the output.  A merge is one workgroup reading from
+  // L2/HBM, so its cost grows with the bytes it reads: two short levels keep
+  // the tail of the launch at a few microseconds even with 256 splits a plane.
+  const uint32_t live = min(p.n_split, (pos + p.split_len) / p.split_len);
+  const uint32_t n_clusters = (live + kMergeFan - 1) / kMergeFan;
+  const uint32_t cluster = split / kMergeFan;
+  const uint32_t in_cluster = min((uint32_t)kMergeFan, live - cluster * kMergeFan);
+  uint32_t* ctr = p.counters + ((size_t)seq * gridDim.y + blockIdx.y) * p.counters_per_plane;
+  __shared__ uint32_t s_last;
+  auto arrive = [&](uint32_t* c, uint32_t expected) -> bool {
+    wait_vm_done();
+    __syncthreads();
+    if (tid == 0) {
+      const uint32_t old = __hip_atomic_fetch_add(c, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      const uint32_t last = (old + 1 == expected) ? 1u : 0u;
+      // back to zero for the next launch; nobody else touches it in this one
+      if (last) __hip_atomic_store(c, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      s_last = last;
+    }
+    __syncthreads();
+    return s_last != 0;
+  };
+  // Fold `count` (<= 16) partials of every head of this group, starting at
+  // partial `first` of a table with `pitch` partials per row.  Every load a
+  // thread needs is issued before anything is waited for, so a fold costs one
+  // trip to memory: an 8-byte (max, sum) pair per thread, shared through LDS,
+  // and 8-byte accumulator pairs for the thread's (head, d pair) items.
+  // emit(h, dp, a0, a1, sum, max) receives columns 2 dp and 2 dp + 1.
+  auto fold = [&](const float* acc_tab, const float* ml_tab, uint32_t pitch, uint32_t first,
+                  uint32_t count, auto emit) {
+    float* sm = (float*)smem;  // [head][kMergeFan][2]; the staging buffers are idle by now
+    const uint32_t n_ml = heads_here * count;
+    const uint32_t h_e = tid / count, s_e = tid % count;
+    uint64_t ml_bits = 0;
+    if ((uint32_t)tid < n_ml)
+      ml_bits = load_coherent64(
+          ml_tab + (((size_t)seq * p.n_q_heads + head0 + h_e) * pitch + first + s_e) * 2);
+    const uint32_t items = heads_here * (kHeadDim / 2);
+    bool published = false;
+    for (uint32_t item = tid; item < (items + kDecWaves * kWave - 1) / (kDecWaves * kWave) *
+                                         (kDecWaves * kWave);
+         item += kDecWaves * kWave) {  // same trip count for every thread: the loop holds a barrier
+      const bool mine = item < items;
+      const uint32_t h = mine ? item / (kHeadDim / 2) : 0, dp = item % (kHeadDim / 2);
+      const float* ac =
+          acc_tab + (((size_t)seq * p.n_q_heads + head0 + h) * pitch + first) * kHeadDim + 2 * dp;
+      uint64_t av[kMergeFan];
+#pragma unroll
+      for (int i = 0; i < kMergeFan; ++i) {
+        const uint32_t sidx = min((uint32_t)i, count - 1);
+        av[i] = mine ? load_coherent64(ac + (size_t)sidx * kHeadDim) : 0;
+      }
+      if (!published) {
+        if ((uint32_t)tid < n_ml) *(uint64_t*)(sm + (h_e * kMergeFan + s_e) * 2) = ml_bits;
+        __syncthreads();
+        published = true;
+      }
+      if (!mine) continue;
+      const float* hm = sm + h * kMergeFan * 2;
+      float m_new = hm[0];
+      for (uint32_t i = 1; i < count; ++i) m_new = fmaxf(m_new, hm[2 * i]);
+      float l_acc = 0.0f, a0 = 0.0f, a1 = 0.0f;
+#pragma unroll
+      for (int i = 0; i < kMergeFan; ++i) {
+        if ((uint32_t)i < count) {
+          const float wgt = fast_exp2(hm[2 * i] - m_new);
+          l_acc += wgt * hm[2 * i + 1];
+          a0 += wgt * __builtin_bit_cast(float, (uint32_t)av[i]);
+          a1 += wgt * __builtin_bit_cast(float, (uint32_t)(av[i] >> 32));
+        }
+      }
+      emit(h, dp, a0, a1, l_acc, m_new);
+    }
+  };
+  auto emit_final = [&](uint32_t h, uint32_t dp, float a0, float a1, float l, float m) {
+    const size_t row = (size_t)seq * p.n_q_heads + head0 + h;
+    const float inv = 1.0f / l;
+    *(uint32_t*)(p.out + row * kHeadDim + 2 * dp) = Mfma<T>::pack2(a0 * inv, a1 * inv);
+    if (p.lse && dp == 0) p.lse[row] = (m + fast_log2(l)) * kLn2;
+  };
+
+  if (!arrive(ctr + 1 + cluster, in_cluster)) return;
+  if (n_clusters == 1) {
+    fold(p.ws_acc, p.ws_ml, p.n_split, 0, live, emit_final);
+    return;
   }
-  const float val = a / lsum;
-  p.out[(size_t)row * kHeadDim + d] = (uint16_t)(Mfma<T>::pack2(val, 0.0f) & 0xffffu);
-  if (p.lse && d == 0) p.lse[row] = (mmax + fast_log2(lsum)) * kLn2;
+  fold(p.ws_acc, p.ws_ml, p.n_split, cluster * kMergeFan, in_cluster,
+       [&](uint32_t h, uint32_t dp, float a0, float a1, float l, float m) {
+         const size_t crow = ((size_t)seq * p.n_q_heads + head0 + h) * p.n_cluster_max + cluster;
+         store_coherent64(p.ws2_acc + crow * kHeadDim + 2 * dp, a0, a1);
+         if (dp == 0) store_coherent64(p.ws2_ml + crow * 2, m, l);
+       });
+  if (!arrive(ctr, n_clusters)) return;
+  fold(p.ws2_acc, p.ws2_ml, p.n_cluster_max, 0, n_clusters, emit_final);
 }
 
 }  // namespace
 
 DecodePlan decode_plan(uint32_t max_len, uint32_t batch, uint32_t n_kv_heads, uint32_t n_cu) {
-  // Aim for about four resident workgroups per compute unit (the LDS footprint
-  // allows four), but never make a split shorter than four 64-key steps.
-  const uint32_t target = n_cu * 4;
+  // Two workgroups per compute unit measured best on MI355X (each workgroup has
+  // fixed costs — query load, wave merge, partial write, arrival — that more,
+  // shorter workgroups pay more often); never make a split shorter than four
+  // 64-key steps.
+  static const int per_cu = [] {
+    const char* e = getenv("ELLM_DECODE_WG_PER_CU");  // tuning override
+    const int v = e ? atoi(e) : 0;
+    return (v >= 1 && v <= 16) ? v : 2;
+  }();
+  const uint32_t target = n_cu * per_cu;
   const uint32_t planes = batch * n_kv_heads;
   const uint32_t want = (target + planes - 1) / planes;
   uint32_t split_len = (max_len + want - 1) / want;
   split_len = (split_len + kDecodeStepKeys - 1) / kDecodeStepKeys * kDecodeStepKeys;
   if (split_len < 4 * kDecodeStepKeys) split_len = 4 * kDecodeStepKeys;
+  // both merge levels fold at most 16 partials: at most 16 * 16 splits per plane
+  const uint32_t floor_len =
+      ((max_len + kMergeFan * kMergeFan - 1) / (kMergeFan * kMergeFan) + kDecodeStepKeys - 1) /
+      kDecodeStepKeys * kDecodeStepKeys;
+  if (split_len < floor_len) split_len = floor_len;
   DecodePlan plan;
   plan.split_len = split_len;
   plan.n_split = (max_len + split_len - 1) / split_len;
   return plan;
 }
 
-size_t decode_workspace_rows(uint32_t batch_capacity, uint32_t n_q_heads, uint32_t n_kv_heads,
-                             uint32_t n_cu) {
+DecodeWorkspace decode_workspace(uint32_t batch_capacity, uint32_t n_q_heads, uint32_t n_kv_heads,
+                                 uint32_t n_cu) {
   // rows = batch * heads * n_split with n_split <= ceil(4*n_cu / (batch*kv_heads))
   const size_t group = n_q_heads / n_kv_heads;
-  return (size_t)batch_capacity * n_q_heads + (size_t)n_cu * 4 * group;
+  DecodeWorkspace w;
+  w.rows = (size_t)batch_capacity * n_q_heads + (size_t)n_cu * 16 * group;
+  // cluster partials: ceil(n_split / 16) per row of batch * heads
+  w.rows2 = w.rows / kMergeFan + (size_t)batch_capacity * n_q_heads;
+  // counters: (1 + clusters) per plane, planes <= batch * heads
+  w.counters = w.rows2 + (size_t)batch_capacity * n_q_heads;
+  return w;
+}
+
+bool decode_plan_fits(const DecodeWorkspace& w, uint32_t batch, uint32_t n_q_heads,
+                      uint32_t n_kv_heads, uint32_t group, uint32_t n_split) {
+  const size_t n_cluster = (n_split + kMergeFan - 1) / kMergeFan;
+  const size_t head_groups = (group + kMaxHeadsPerGroup - 1) / kMaxHeadsPerGroup;
+  return (size_t)batch * n_q_heads * n_split <= w.rows &&
+         (size_t)batch * n_q_heads * n_cluster <= w.rows2 &&
+         (size_t)batch * n_kv_heads * head_groups * (1 + n_cluster) <= w.counters;
 }
 
 hipError_t launch_decode(const AttnArgs& a, hipStream_t stream) {
@@ -282,6 +439,16 @@ hipError_t launch_decode(const AttnArgs& a, hipStream_t stream) {
   p.positions = a.positions;
   p.ws_acc = a.ws_acc;
   p.ws_ml = a.ws_ml;
+  p.ws2_acc = a.ws2_acc;
+  p.ws2_ml = a.ws2_ml;
+  p.counters = a.counters;
+  p.n_cluster_max = (a.n_split + kMergeFan - 1) / kMergeFan;
+  p.counters_per_plane = 1 + p.n_cluster_max;
+  static const int rotate = [] {
+    const char* e = getenv("ELLM_DECODE_ROTATE");
+    return e ? atoi(e) : 1;
+  }();
+  p.rotate = rotate;
   p.kv_stride_seq = a.kv_stride_seq;
   p.kv_stride_head = a.kv_stride_head;
   p.kv_stride_pos = a.kv_stride_pos;
@@ -300,17 +467,7 @@ hipError_t launch_decode(const AttnArgs& a, hipStream_t stream) {
     hipLaunchKernelGGL(decode_split_kernel<F16>, grid, block, 0, stream, p);
   else
     hipLaunchKernelGGL(decode_split_kernel<BF16>, grid, block, 0, stream, p);
-  hipError_t err = hipGetLastError();
-  if (err != hipSuccess) return err;
-  if (a.n_split > 1) {
-    dim3 mgrid(a.batch * a.n_q_heads);
-    if (a.dtype == 0)
-      hipLaunchKernelGGL(merge_kernel<F16>, mgrid, dim3(kHeadDim), 0, stream, p);
-    else
-      hipLaunchKernelGGL(merge_kernel<BF16>, mgrid, dim3(kHeadDim), 0, stream, p);
-    err = hipGetLastError();
-  }
-  return err;
+  return hipGetLastError();
 }
 
 }  // namespace ellm

@@ -30,23 +30,34 @@ struct AttnArgs {
   uint32_t batch;
   const uint32_t* positions;  // device, per sequence; null = position_index for all
   // single-token path workspace
-  float* ws_acc;  // [batch][kv_head][split][group][128]
-  float* ws_ml;   // [batch][kv_head][split][group][2]  (max in log2 units, sum)
+  float* ws_acc;  // [sequence][query head][split][128]
+  float* ws_ml;   // [sequence][query head][split][2]  (max in log2 units, sum)
+  float* ws2_acc;      // second merge level: [sequence][query head][cluster][128]
+  float* ws2_ml;
+  uint32_t* counters;  // arrival counters, zero between launches
   uint32_t split_len;  // keys per split, multiple of 64
   uint32_t n_split;
 };
 
 // Keys handled by one workgroup step of the single-token kernel.
 constexpr uint32_t kDecodeStepKeys = 64;
-// Upper bound on the number of partial rows (sequence x head x split) the
-// workspace must hold for a given capacity; see decode_plan().
 struct DecodePlan {
   uint32_t split_len;
   uint32_t n_split;
 };
 DecodePlan decode_plan(uint32_t max_len, uint32_t batch, uint32_t n_kv_heads, uint32_t n_cu);
-size_t decode_workspace_rows(uint32_t batch_capacity, uint32_t n_q_heads, uint32_t n_kv_heads,
-                             uint32_t n_cu);
+
+// Sizes (in partial rows / counters) that cover every plan decode_plan() can
+// return for up to batch_capacity sequences.
+struct DecodeWorkspace {
+  size_t rows;      // first-level partials  (x 128 and x 2 floats)
+  size_t rows2;     // cluster partials      (x 128 and x 2 floats)
+  size_t counters;  // uint32 arrival counters
+};
+DecodeWorkspace decode_workspace(uint32_t batch_capacity, uint32_t n_q_heads, uint32_t n_kv_heads,
+                                 uint32_t n_cu);
+bool decode_plan_fits(const DecodeWorkspace& w, uint32_t batch, uint32_t n_q_heads,
+                      uint32_t n_kv_heads, uint32_t group, uint32_t n_split);
 
 hipError_t launch_decode(const AttnArgs& a, hipStream_t stream);
 hipError_t launch_prefill(const AttnArgs& a, hipStream_t stream);

@@ -21,6 +21,8 @@
 // blocks.  Stacking the group's heads makes each LDS tile feed 4*NB times more
 // MFMA work and keeps the token span (and so the masked part of the diagonal
 // tile) short.
+#include <cstdlib>
+
 #include "common.hpp"
 #include "kernels.hpp"
 
@@ -35,6 +37,7 @@ constexpr int kVtsPitch = kBK + 8;          // halves per V^T row (144 B)
 constexpr int kKsHalves = kBK * kKsPitch;
 constexpr int kVtsHalves = kHeadDim * kVtsPitch;
 constexpr int kStageHalves = kKsHalves + kVtsHalves;
+constexpr float kRescaleStep = 8.0f;        // log2 units
 
 struct PrefillKernelArgs {
   const uint16_t* q;
@@ -53,11 +56,12 @@ struct PrefillKernelArgs {
   uint32_t combos;           // batch * kv_heads * head_groups
   uint32_t xcd_mode;         // 1: workgroup id % 8 selects the K/V plane
   uint32_t position_index, interval;
-  float scale_log2;
+  uint32_t negate_q;         // scale < 0: fold the sign into Q (exact) so that c > 0
+  float c;                   // |scale| * log2(e), > 0
 };
 
 template <typename T, int NB>
-__global__ __launch_bounds__(kPfThreads) void prefill_kernel(PrefillKernelArgs p) {
+__global__ __launch_bounds__(kPfThreads, NB == 1 ? 2 : 1) void prefill_kernel(PrefillKernelArgs p) {
   __shared__ __attribute__((aligned(16))) uint16_t smem[2 * kStageHalves];
 
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
@@ -113,8 +117,12 @@ __global__ __launch_bounds__(kPfThreads) void prefill_kernel(PrefillKernelArgs p
     const uint16_t* qrow =
         p.q + (size_t)tok[n] * p.q_token_stride + ((size_t)seq * p.n_q_heads + head[n]) * kHeadDim;
 #pragma unroll
-    for (int s = 0; s < 8; ++s) qreg[n][s] = load16(qrow + 16 * s + 8 * g);
+    for (int s = 0; s < 8; ++s) {
+      qreg[n][s] = load16(qrow + 16 * s + 8 * g);
+      if (p.negate_q) qreg[n][s] ^= 0x80008000u;
+    }
   }
+  const float c = p.c;
 
   const uint16_t* kplane = p.k + seq * p.kv_stride_seq + kvh * p.kv_stride_head;
   const uint16_t* vplane = p.v + seq * p.kv_stride_seq + kvh * p.kv_stride_head;
@@ -204,52 +212,59 @@ __global__ __launch_bounds__(kPfThreads) void prefill_kernel(PrefillKernelArgs p
       }
 
       // ---- online soft-max, one query row per lane --------------------------
+      // Scores stay unscaled; scale*log2(e) (c > 0) is folded into the exponent's
+      // FMA.  The reference max m is only moved when the tile's max exceeds it by
+      // more than kRescaleStep (log2 units), so most tiles skip the rescale of
+      // O^T; probabilities are then at most 2^kRescaleStep, well inside binary16
+      // and bfloat16 range.  The row sum adds the unrounded binary32
+      // probabilities: summing the rounded ones is cheaper but moves the
+      // log-sum-exp by up to half a storage ulp, beyond its 1e-4 tolerance.
       u32x4 pk[NB][4];
 #pragma unroll
       for (int n = 0; n < NB; ++n) {
-        const bool need_mask = kb + kBK - 1 > first_pos[n];
-        const uint32_t rowpos = P0 + tok[n];
-        float tmax = -INFINITY;
+        if (kb + kBK - 1 > first_pos[n]) {  // tile crosses this block's diagonal
+          const uint32_t rowpos = P0 + tok[n];
 #pragma unroll
-        for (int mb = 0; mb < 2; ++mb)
+          for (int mb = 0; mb < 2; ++mb)
 #pragma unroll
-          for (int r = 0; r < 16; ++r) {
-            float t = st[n][mb][r] * p.scale_log2;
-            if (need_mask) {
+            for (int r = 0; r < 16; ++r) {
               const uint32_t key = kb + 32 * mb + 8 * (r >> 2) + 4 * g + (r & 3);
-              t = (key <= rowpos) ? t : -INFINITY;
+              st[n][mb][r] = (key <= rowpos) ? st[n][mb][r] : -INFINITY;
             }
-            st[n][mb][r] = t;
-            tmax = fmaxf(tmax, t);
-          }
-        tmax = fmaxf(tmax, xor_shuffle(tmax, 32));
-        // m stays -inf only while every key so far was masked for this row,
-        // which cannot happen from tile 0 on (key 0 is visible to every row);
-        // the guard keeps exp2(-inf - -inf) out of the arithmetic regardless.
-        const float m_new = fmaxf(m_run[n], tmax);
-        const float m_safe = (m_new == -INFINITY) ? 0.0f : m_new;
-        const float alpha = fast_exp2(m_run[n] - m_safe);
-        float psum = 0.0f;
+        }
+        float rmax = st[n][0][0];
 #pragma unroll
         for (int mb = 0; mb < 2; ++mb)
 #pragma unroll
-          for (int r = 0; r < 16; ++r) {
-            const float pv = fast_exp2(st[n][mb][r] - m_safe);
-            st[n][mb][r] = pv;
-            psum += pv;
-          }
-        l_run[n] = l_run[n] * alpha + psum;
-        m_run[n] = m_new;
+          for (int r = 0; r < 16; ++r) rmax = fmaxf(rmax, st[n][mb][r]);
+        rmax = fmaxf(rmax, xor_shuffle(rmax, 32));
+        const float tmax = rmax * c;
+        const bool grow = tmax > m_run[n] + kRescaleStep;
+        if (__any(grow)) {
+          const float m_new = grow ? tmax : m_run[n];
+          const float alpha = grow ? fast_exp2(m_run[n] - m_new) : 1.0f;
+          m_run[n] = m_new;
+          l_run[n] *= alpha;
 #pragma unroll
-        for (int db = 0; db < 4; ++db) oacc[n][db] *= alpha;
-        // registers 8c'..8c'+7 of block mb are the B operand of key chunk 2 mb + c'
+          for (int db = 0; db < 4; ++db) oacc[n][db] *= alpha;
+        }
+        // m_run is finite from tile 0 on (key 0 is visible to every row); the
+        // guard only keeps -inf - -inf out of the arithmetic.
+        const float neg_m = (m_run[n] == -INFINITY) ? 0.0f : -m_run[n];
+        float psum = 0.0f;
 #pragma unroll
         for (int cc = 0; cc < 4; ++cc) {
           const int mb = cc >> 1, r0 = 8 * (cc & 1);
 #pragma unroll
-          for (int w = 0; w < 4; ++w)
-            pk[n][cc][w] = Mfma<T>::pack2(st[n][mb][r0 + 2 * w], st[n][mb][r0 + 2 * w + 1]);
+          for (int w = 0; w < 4; ++w) {
+            const float p0 = fast_exp2(__builtin_fmaf(st[n][mb][r0 + 2 * w], c, neg_m));
+            const float p1 = fast_exp2(__builtin_fmaf(st[n][mb][r0 + 2 * w + 1], c, neg_m));
+            const uint32_t word = Mfma<T>::pack2(p0, p1);
+            pk[n][cc][w] = word;
+            psum += p0 + p1;
+          }
         }
+        l_run[n] += psum;
       }
 
       // ---- O^T += V^T . P^T --------------------------------------------------
@@ -327,7 +342,11 @@ hipError_t launch_nb(const AttnArgs& a, hipStream_t stream) {
   p.xcd_mode = (p.combos <= 8 && 8 % p.combos == 0) ? 1 : 0;
   p.position_index = a.position_index;
   p.interval = a.position_interval;
-  p.scale_log2 = a.scale * kLog2e;
+  float c = a.scale * kLog2e;
+  p.negate_q = c < 0.0f ? 1u : 0u;
+  c = c < 0.0f ? -c : c;
+  // scale == 0 (uniform attention): a tiny positive c keeps -inf * c == -inf for masked keys
+  p.c = c > 0.0f ? c : 1e-37f;
 
   uint32_t n_wg;
   if (p.xcd_mode) {
@@ -343,6 +362,14 @@ hipError_t launch_nb(const AttnArgs& a, hipStream_t stream) {
 }  // namespace
 
 hipError_t launch_prefill(const AttnArgs& a, hipStream_t stream) {
+  static const int nb = [] {
+    const char* e = getenv("ELLM_PREFILL_NB");
+    return (e && e[0] == '1') ? 1 : 2;
+  }();
+  if (nb == 1) {
+    if (a.dtype == 0) return launch_nb<F16, 1>(a, stream);
+    return launch_nb<BF16, 1>(a, stream);
+  }
   if (a.dtype == 0) return launch_nb<F16, 2>(a, stream);
   return launch_nb<BF16, 2>(a, stream);
 }
