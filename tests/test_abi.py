@@ -1,0 +1,115 @@
+"""The C ABI without a GPU: the library loads, exports every symbol the header
+declares, and rejects bad descriptions with a status instead of aborting
+(the reference has no error path at all: src/compiler/operator.rs:243 panics,
+Cargo.toml:49 makes a panic an abort)."""
+import ctypes
+import os
+import re
+
+import pytest
+
+import ellm_amd
+from ellm_amd import _lib
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+OK, INVALID, UNSUPPORTED, OUT_OF_RANGE, HIP, NO_DEVICE = range(6)
+
+
+def test_library_exports_every_declared_symbol():
+    header = open(os.path.join(ROOT, "include", "ellm_attn.h")).read()
+    header = re.sub(r"/\*.*?\*/", "", header, flags=re.S)
+    declared = set(re.findall(r"\b(ellm_[a-z_0-9]+)\s*\(", header))
+    assert declared == set(_lib.ABI_SYMBOLS), declared ^ set(_lib.ABI_SYMBOLS)
+    lib = ctypes.CDLL(ellm_amd.lib_path())
+    for name in declared:
+        assert getattr(lib, name) is not None
+
+
+def test_missing_library_fails_loudly(monkeypatch, tmp_path):
+    monkeypatch.setattr(_lib, "_lib", None)
+    monkeypatch.setattr(_lib, "lib_path", lambda: str(tmp_path / "nope.so"))
+    with pytest.raises(ellm_amd.LibraryMissing):
+        _lib.load_library()
+
+
+def test_version_and_device_count():
+    lib = ellm_amd.load_library()
+    assert lib.ellm_attn_version() >= 100
+    assert lib.ellm_device_count() >= 0
+
+
+def _desc(**over):
+    d = _lib.AttnDesc()
+    d.q = d.k = d.v = d.out = 0x1000
+    d.lse = None
+    d.batch_size, d.attention_head_num, d.kv_head_num, d.head_size = 2, 8, 2, 128
+    for i, s in enumerate((2 * 64 * 128, 64 * 128, 128, 1)):
+        d.kv_strides[i] = s
+    d.inverse_sqrt_head = 0.088
+    d.dtype = _lib.DTYPE_F16
+    d.sequence_capacity, d.max_position_interval = 64, 16
+    for k, v in over.items():
+        if k == "kv_strides":
+            for i, s in enumerate(v):
+                d.kv_strides[i] = s
+        else:
+            setattr(d, k, v)
+    return d
+
+
+@pytest.mark.parametrize("over,status", [
+    (dict(q=None), INVALID),
+    (dict(out=None), INVALID),
+    (dict(k=0x1008), INVALID),                       # not 16-byte aligned
+    (dict(dtype=7), INVALID),
+    (dict(head_size=64), UNSUPPORTED),               # like the AVX-512 kernel: 128 only
+    (dict(attention_head_num=7), INVALID),           # not a multiple of kv_head_num
+    (dict(kv_head_num=0), INVALID),
+    (dict(kv_strides=(2 * 64 * 128, 64 * 128, 128, 2)), INVALID),
+    (dict(kv_strides=(2 * 64 * 128, 64 * 128, 100, 1)), INVALID),
+    (dict(sequence_capacity=0), INVALID),
+    (dict(max_position_interval=65), INVALID),
+    (dict(inverse_sqrt_head=float("nan")), INVALID),
+])
+def test_create_rejects_bad_descriptions(over, status):
+    lib = ellm_amd.load_library()
+    h = ctypes.c_void_p()
+    rc = lib.ellm_attn_create(ctypes.byref(_desc(**over)), ctypes.byref(h))
+    assert rc == status
+    assert not h.value
+    assert lib.ellm_last_error_string()
+
+
+def test_null_arguments():
+    lib = ellm_amd.load_library()
+    h = ctypes.c_void_p()
+    assert lib.ellm_attn_create(None, ctypes.byref(h)) == INVALID
+    assert lib.ellm_attn_run(None, 0, 1, 1, None) == INVALID
+    assert lib.ellm_attn_run_ragged(None, None, 0, 1, None) == INVALID
+    assert lib.ellm_attn_destroy(None) == OK
+    assert lib.ellm_kv_destroy(None) == OK
+    c = ctypes.c_void_p()
+    assert lib.ellm_kv_create(None, ctypes.byref(c)) == INVALID
+    kd = _lib.KvDesc(1, 1, 1, 64, 16, 0)
+    assert lib.ellm_kv_create(ctypes.byref(kd), ctypes.byref(c)) == UNSUPPORTED
+    kd = _lib.KvDesc(0, 1, 1, 128, 16, 0)
+    assert lib.ellm_kv_create(ctypes.byref(kd), ctypes.byref(c)) == INVALID
+
+
+def test_valid_description_without_a_device_reports_no_device():
+    lib = ellm_amd.load_library()
+    if lib.ellm_device_count() > 0:
+        pytest.skip("a device is present")
+    h = ctypes.c_void_p()
+    assert lib.ellm_attn_create(ctypes.byref(_desc()), ctypes.byref(h)) in (NO_DEVICE, HIP)
+    assert not h.value
+
+
+def test_host_mirror_only_thread_zero_launches():
+    """Every worker thread calls run() in the reference (src/serving/start.rs:69-73);
+    here all but thread 0 must return without touching the library."""
+    op = ellm_amd.Attention.__new__(ellm_amd.Attention)
+    op._handle = None
+    op._lib = None
+    op.run(0, 1, 1, cpu_num=8, thread_id=3)   # would raise if it reached the library
