@@ -44,24 +44,34 @@ def _dev_normal(shape, dtype, seed, scale=1.0):
 
 
 def _time_steps(fn, steps, warmup):
-    """Per-step durations (ms) from HIP events recorded on the launch stream."""
+    """W untimed steps, then exactly K steps between two synchronisation points.
+
+    Returns ([average launch duration in ms], host-clock ms per step).  The host clock
+    brackets the first K-step pass with torch.cuda.synchronize() on both sides.  The
+    launch duration comes from a second K-step pass bracketed by two HIP events on the
+    launch stream (the library launches on torch's current stream, where the events
+    are recorded too): one step of either workload is a single kernel launch and the
+    launches run back to back, so elapsed / K is that kernel's average duration
+    (an event pair around every single launch adds several microseconds of
+    command-processor work per step and overstates a 50 us kernel by 10 %)."""
     import torch
 
     for i in range(warmup):
         fn(i)
     torch.cuda.synchronize()
-    starts = [torch.cuda.Event(enable_timing=True) for _ in range(steps)]
-    stops = [torch.cuda.Event(enable_timing=True) for _ in range(steps)]
     t0 = time.perf_counter()
     for i in range(steps):
-        starts[i].record()
         fn(warmup + i)
-        stops[i].record()
     torch.cuda.synchronize()
-    wall_ms = (time.perf_counter() - t0) * 1e3
-    per = [s.elapsed_time(e) for s, e in zip(starts, stops)]
-    whole_ms = starts[0].elapsed_time(stops[-1])
-    return per, whole_ms, wall_ms
+    step_ms = (time.perf_counter() - t0) * 1e3 / steps
+    start = torch.cuda.Event(enable_timing=True)
+    stop = torch.cuda.Event(enable_timing=True)
+    start.record()
+    for i in range(steps):
+        fn(warmup + i)
+    stop.record()
+    torch.cuda.synchronize()
+    return [start.elapsed_time(stop) / steps], step_ms
 
 
 def bench_decode(batch, length, steps, warmup, hq=32, hkv=4, copies=4):
@@ -81,9 +91,8 @@ def bench_decode(batch, length, steps, warmup, hq=32, hkv=4, copies=4):
         op = ellm_amd.Attention(q, k, v, out, batch, hq, hkv, D, [hkv * cap * D, cap * D, D, 1],
                                 scale, lse=lse, sequence_capacity=cap, max_position_interval=1)
         ops.append(op)
-    per, whole_ms, _ = _time_steps(lambda i: ops[i % copies].run(length - 1, 1, batch), steps, warmup)
+    per, step_ms = _time_steps(lambda i: ops[i % copies].run(length - 1, 1, batch), steps, warmup)
     alg_bytes = 2 * batch * hkv * length * D * 2 + 2 * batch * hq * D * 2
-    step_ms = whole_ms / steps
     kern_ms = sum(per) / len(per)
     for op in ops:
         op.close()
@@ -115,9 +124,8 @@ def bench_prefill(seq, steps, warmup, hq=32, hkv=4, dtype_name="f16", p0=0):
     lse = torch.zeros((seq, 1, hq), dtype=torch.float32, device="cuda")
     op = ellm_amd.Attention(q, k, v, out, 1, hq, hkv, D, [hkv * cap * D, cap * D, D, 1], scale,
                             lse=lse, sequence_capacity=cap, max_position_interval=seq)
-    per, whole_ms, _ = _time_steps(lambda i: op.run(p0, seq, 1), steps, warmup)
+    per, step_ms = _time_steps(lambda i: op.run(p0, seq, 1), steps, warmup)
     flops = 4 * D * hq * (seq * p0 + seq * (seq + 1) // 2)
-    step_ms = whole_ms / steps
     kern_ms = sum(per) / len(per)
     op.close()
     return {
@@ -163,6 +171,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--skip-cpu", action="store_true")
     ap.add_argument("--only", default="", help="decode | prefill | decode128k")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="first run one plain 256 MiB device copy (a known-traffic dispatch "
+                         "for scaling rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE readings)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU only (no collectives); use --gpus 1",
@@ -177,6 +188,14 @@ def main():
     if not torch.cuda.is_available():
         print("bench.py: no GPU visible", file=sys.stderr)
         sys.exit(1)
+
+    if args.copy_calibration:
+        src = torch.ones(256 * 1024 * 1024 // 4, dtype=torch.float32, device="cuda")
+        dst = torch.empty_like(src)
+        torch.cuda.synchronize()
+        dst.copy_(src)      # one elementwise copy kernel: reads 256 MiB, writes 256 MiB
+        torch.cuda.synchronize()
+        del src, dst
 
     also = []
     dec = None

@@ -127,6 +127,10 @@ int ellm_attn_create(const ellm_attn_desc* d, ellm_attn** out_handle) {
                 d->kv_strides[2]);
   if (d->sequence_capacity == 0 || d->sequence_capacity > 0x7fffffffu)
     return fail(ELLM_ERR_INVALID_ARGUMENT, "sequence_capacity %zu out of range", d->sequence_capacity);
+  if (d->sequence_capacity * d->kv_strides[2] > 0x7fffffffu)
+    return fail(ELLM_ERR_UNSUPPORTED,
+                "a K/V plane spans %zu elements; offsets inside a plane are 32-bit (max 2^31 - 1)",
+                d->sequence_capacity * d->kv_strides[2]);
   if (d->max_position_interval == 0 || d->max_position_interval > d->sequence_capacity)
     return fail(ELLM_ERR_INVALID_ARGUMENT,
                 "max_position_interval %zu must be in 1..sequence_capacity", d->max_position_interval);

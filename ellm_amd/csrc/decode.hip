@@ -90,8 +90,17 @@ __device__ __forceinline__ void store_row_elem(const DecodeKernelArgs& p, uint32
   if (p.lse && d == 0) p.lse[row] = (mmax + fast_log2(lsum)) * kLn2;
 }
 
-template <typename T>
-__global__ __launch_bounds__(kDecWaves* kWave, 4) void decode_split_kernel(DecodeKernelArgs p) {
+template <bool NT>
+__device__ __forceinline__ u32x4 stream_load16(const uint16_t* p) {
+  if (NT) return __builtin_nontemporal_load((const u32x4*)p);
+  return *(const u32x4*)p;
+}
+
+// DEPTH = 16-key chunks each wave keeps in flight (register staging buffers);
+// NT = mark the K/V loads non-temporal (read once, never reused).
+template <typename T, int DEPTH, bool NT>
+__global__ __launch_bounds__(kDecWaves* kWave, DEPTH == 1 ? 4 : 3) void decode_split_kernel(
+    DecodeKernelArgs p) {
   __shared__ __attribute__((aligned(16))) uint16_t smem[kDecWaves * kWaveLdsHalves];
 
   const uint32_t split = blockIdx.x;
@@ -133,16 +142,16 @@ __global__ __launch_bounds__(kDecWaves* kWave, 4) void decode_split_kernel(Decod
   uint16_t* vt = ks + kChunk * kKPitch;         // [128][kVtPitch]
 
   const uint32_t n_chunks = (k_end - k_begin + kChunk - 1) / kChunk;
-  u32x4 kreg[4], vreg[4];
-  auto issue_loads = [&](uint32_t chunk) {
+  u32x4 kreg[DEPTH][4], vreg[DEPTH][4];
+  auto issue_loads = [&](u32x4* kr, u32x4* vr, uint32_t chunk) {
     const uint32_t kb = k_begin + chunk * kChunk;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       // rows past the last valid key are clamped onto it: always in bounds,
       // always initialised, and their probabilities are forced to zero below.
       const uint32_t row = min(kb + 4 * g + i, pos);
-      kreg[i] = load16(kplane + (size_t)row * p.kv_stride_pos + 8 * c);
-      vreg[i] = load16(vplane + (size_t)row * p.kv_stride_pos + 8 * c);
+      kr[i] = stream_load16<NT>(kplane + (size_t)row * p.kv_stride_pos + 8 * c);
+      vr[i] = stream_load16<NT>(vplane + (size_t)row * p.kv_stride_pos + 8 * c);
     }
   };
 
@@ -163,20 +172,26 @@ __global__ __launch_bounds__(kDecWaves* kWave, 4) void decode_split_kernel(Decod
     if (r >= my_chunks) r -= my_chunks;
     return wave + r * kDecWaves;
   };
-  if (my_chunks) issue_loads(chunk_at(0));
-  for (uint32_t it = 0; it < my_chunks; ++it) {
+#pragma unroll
+  for (int u = 0; u < DEPTH; ++u)
+    if ((uint32_t)u < my_chunks) issue_loads(kreg[u], vreg[u], chunk_at(u));
+  for (uint32_t it0 = 0; it0 < my_chunks; it0 += DEPTH) {
+#pragma unroll
+   for (int u = 0; u < DEPTH; ++u) {
+    const uint32_t it = it0 + u;
+    if (it >= my_chunks) break;
     const uint32_t chunk = chunk_at(it);
     const uint32_t kb = k_begin + chunk * kChunk;
     // registers -> LDS: K row-major, V transposed.
 #pragma unroll
-    for (int i = 0; i < 4; ++i) store16(ks + (4 * g + i) * kKPitch + 8 * c, kreg[i]);
+    for (int i = 0; i < 4; ++i) store16(ks + (4 * g + i) * kKPitch + 8 * c, kreg[u][i]);
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
-      u32x2 col = gather_column(vreg[0][e >> 1], vreg[1][e >> 1], vreg[2][e >> 1],
-                                vreg[3][e >> 1], (e & 1) != 0);
+      u32x2 col = gather_column(vreg[u][0][e >> 1], vreg[u][1][e >> 1], vreg[u][2][e >> 1],
+                                vreg[u][3][e >> 1], (e & 1) != 0);
       *(u32x2*)(vt + (8 * c + e) * kVtPitch + 4 * g) = col;
     }
-    if (it + 1 < my_chunks) issue_loads(chunk_at(it + 1));
+    if (it + DEPTH < my_chunks) issue_loads(kreg[u], vreg[u], chunk_at(it + DEPTH));
     __builtin_amdgcn_wave_barrier();
 
     // S^T[key][head], lane (head c, group g) register r <-> key kb + 4 g + r.
@@ -216,6 +231,7 @@ __global__ __launch_bounds__(kDecWaves* kWave, 4) void decode_split_kernel(Decod
       acc[b] = Mfma<T>::m16x16x16(a, pb, acc[b]);
     }
     __builtin_amdgcn_wave_barrier();
+   }
   }
 
   l_run += xor_shuffle(l_run, 16);
@@ -463,10 +479,22 @@ hipError_t launch_decode(const AttnArgs& a, hipStream_t stream) {
 
   dim3 grid(a.n_split, a.n_kv_heads * p.head_groups, a.batch);
   dim3 block(kDecWaves * kWave);
-  if (a.dtype == 0)
-    hipLaunchKernelGGL(decode_split_kernel<F16>, grid, block, 0, stream, p);
-  else
-    hipLaunchKernelGGL(decode_split_kernel<BF16>, grid, block, 0, stream, p);
+  static const int depth = [] {
+    const char* e = getenv("ELLM_DECODE_DEPTH");  // tuning override
+    return (e && e[0] == '2') ? 2 : 1;  // a second chunk in flight per wave measured no faster
+  }();
+  static const int nt = [] {
+    const char* e = getenv("ELLM_DECODE_NT");  // tuning override
+    return (e && e[0] == '0') ? 0 : 1;
+  }();
+  auto go = [&](auto kernel) { hipLaunchKernelGGL(kernel, grid, block, 0, stream, p); };
+  if (a.dtype == 0) {
+    if (depth == 1) nt ? go(decode_split_kernel<F16, 1, true>) : go(decode_split_kernel<F16, 1, false>);
+    else nt ? go(decode_split_kernel<F16, 2, true>) : go(decode_split_kernel<F16, 2, false>);
+  } else {
+    if (depth == 1) nt ? go(decode_split_kernel<BF16, 1, true>) : go(decode_split_kernel<BF16, 1, false>);
+    else nt ? go(decode_split_kernel<BF16, 2, true>) : go(decode_split_kernel<BF16, 2, false>);
+  }
   return hipGetLastError();
 }
 
