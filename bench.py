@@ -28,6 +28,14 @@ sys.path.insert(0, ROOT)
 sys.path.insert(0, os.path.join(ROOT, "tests"))
 
 HBM_PEAK_GBS = 8000.0       # MI355X HBM3E, published
+# HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (scaled by a plain
+# copy of known size; summaries and commands under profiles/).  Not measurable from inside
+# this script; null for workloads without a counter run.
+TRAFFIC_BYTES = {
+    "decode": (264960 + 2459) * 1024,          # 16 x 8192 and 1 x 131072 dispatches averaged
+    "decode128k": (264960 + 2459) * 1024,
+    "prefill": (1363420 + 362270) * 1024,
+}
 MFMA_F16_PEAK_TFLOPS = 2500.0  # MI355X dense fp16/bf16 MFMA, published
 D = 128
 
@@ -211,7 +219,7 @@ def main():
             "roofline": {"bound": "mfma", "achieved": round(pf["kernel_tflops"], 2),
                          "peak": MFMA_F16_PEAK_TFLOPS, "unit": "TFLOP/s",
                          "frac": round(pf["kernel_tflops"] / MFMA_F16_PEAK_TFLOPS, 4),
-                         "traffic": None},
+                         "traffic": TRAFFIC_BYTES["prefill"]},
         })
     if args.only in ("", "decode128k"):
         d128 = bench_decode(1, 131072, args.steps, args.warmup)
@@ -221,7 +229,8 @@ def main():
             "ms_per_step": round(d128["ms_per_step"], 5), "steps": args.steps,
             "roofline": {"bound": "hbm", "achieved": round(d128["kernel_gbs"], 1),
                          "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                         "frac": round(d128["kernel_gbs"] / HBM_PEAK_GBS, 4), "traffic": None},
+                         "frac": round(d128["kernel_gbs"] / HBM_PEAK_GBS, 4),
+                         "traffic": TRAFFIC_BYTES["decode128k"]},
         })
 
     cpu = None
@@ -249,7 +258,7 @@ def main():
                    "batch": 16, "cache_len": 8192, "q_heads": 32, "kv_heads": 4},
         "roofline": {"bound": "hbm", "achieved": round(dec["kernel_gbs"], 1), "peak": HBM_PEAK_GBS,
                      "unit": "GB/s", "frac": round(dec["kernel_gbs"] / HBM_PEAK_GBS, 4),
-                     "traffic": None},
+                     "traffic": TRAFFIC_BYTES["decode"]},
         "cpu_baseline": cpu,
         "also": also,
     }
