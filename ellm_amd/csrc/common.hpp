@@ -104,6 +104,28 @@ __device__ __forceinline__ void store16(void* p, u32x4 v) { *(u32x4*)p = v; }
 // Exchange with the lane whose index differs in the given bit (16 or 32).
 __device__ __forceinline__ float xor_shuffle(float v, int mask) { return __shfl_xor(v, mask, 64); }
 
+// v_permlane32_swap exchanges the upper half of one register with the lower half
+// of another; swapping a value with a copy of itself (in a second register: a
+// register swapped with itself keeps its lower half) yields, in every lane l, the
+// value of lane l % 32 in one register and of lane 32 + l % 32 in the other, i.e.
+// the lane's own value and its partner's (lane l ^ 32), without a trip through LDS.
+// Written as inline asm: with the builtin the optimiser folds max / add of the two
+// results as if they were equal.  The s_nop pairs cover the VALU-write -> permlane
+// read and permlane write -> VALU read wait states the compiler cannot see here.
+__device__ __forceinline__ void swap_halves(float& a, float& b) {
+  asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1\n\ts_nop 1" : "+v"(a), "+v"(b));
+}
+__device__ __forceinline__ float max_with_partner_half(float v) {
+  float a = v, b = v;
+  swap_halves(a, b);
+  return fmaxf(a, b);
+}
+__device__ __forceinline__ float sum_with_partner_half(float v) {
+  float a = v, b = v;
+  swap_halves(a, b);
+  return a + b;
+}
+
 // Regroup packed 16-bit pairs: given four registers holding (x[k][2c], x[k][2c+1])
 // for k = 0..3, return the two registers holding (x[0][e], x[1][e]) and
 // (x[2][e], x[3][e]) for e = 2c (hi = false) or 2c+1 (hi = true).

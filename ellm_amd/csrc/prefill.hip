@@ -603,7 +603,7 @@ __global__ __launch_bounds__(kPpThreads, 2) void prefill_pingpong_kernel(Prefill
     for (int mb = 0; mb < 2; ++mb)
 #pragma unroll
       for (int r = 0; r < 16; ++r) rmax = fmaxf(rmax, st[mb][r]);
-    rmax = fmaxf(rmax, xor_shuffle(rmax, 32));
+    rmax = max_with_partner_half(rmax);
     const float tmax = rmax * c;
     const bool grow = tmax > m_run + kRescaleStep;
     if (__any(grow)) {
@@ -657,7 +657,7 @@ __global__ __launch_bounds__(kPpThreads, 2) void prefill_pingpong_kernel(Prefill
   if (grp == 1) matrix_any(n_tiles);
 
   {
-    const float l = l_run + xor_shuffle(l_run, 32);
+    const float l = sum_with_partner_half(l_run);
     if (row_valid) {
       const float inv = 1.0f / l;
       uint16_t* orow =
