@@ -561,8 +561,10 @@ __global__ __launch_bounds__(kPpThreads, 2) void prefill_pingpong_kernel(Prefill
         else
           oacc[i & 3] = Mfma<T>::m32x32x16(ring[n % kLdsAhead], pk[i >> 2], oacc[i & 3]);
         if (n + kLdsAhead < 32) ring[n % kLdsAhead] = operand(n + kLdsAhead);
-        if (n >= 8 && n < 16) store_piece(grp ? (int)(kt & 1) : (int)((kt + 1) & 1), n - 8);
-        if (n >= 16 && n < 20) load_piece(grp ? kt + 1 : kt + 2, n - 16);
+        // staging last: the loads issued at the end of the previous matrix step have had
+        // almost a whole iteration (~2 us) to arrive before their registers are stored
+        if (n >= 20 && n < 28) store_piece(grp ? (int)(kt & 1) : (int)((kt + 1) & 1), n - 20);
+        if (n >= 28 && n < 32) load_piece(grp ? kt + 1 : kt + 2, n - 28);
         __builtin_amdgcn_sched_barrier(0);
       }
       return;
