@@ -382,6 +382,7 @@ __global__ __launch_bounds__(kPfThreads, NB == 1 ? 2 : 1) void prefill_kernel(Pr
 constexpr int kPpWaves = 8;
 constexpr int kPpThreads = kPpWaves * kWave;
 constexpr int kLdsAhead = 8;  // LDS operand reads in flight ahead of their MFMA
+constexpr int kBufferFlags = 0x00020000;  // raw buffer of 32-bit data, no swizzle (word 3 of the descriptor)
 
 template <typename T>
 __global__ __launch_bounds__(kPpThreads, 2) void prefill_pingpong_kernel(PrefillKernelArgs p) {
@@ -454,6 +455,22 @@ __global__ __launch_bounds__(kPpThreads, 2) void prefill_pingpong_kernel(Prefill
   const uint32_t stride_pos = (uint32_t)p.kv_stride_pos;
   const uint32_t row0 = grp ? 4 * ld_r : ld_r;                    // row of piece 0 inside a tile
   const uint32_t row_step = grp ? 1 : 16;                         // rows between pieces
+  // Tiles are fetched with buffer loads: the descriptor (base of tile kt, bytes
+  // left up to the last key this workgroup may see) is scalar arithmetic, the
+  // per-lane byte offsets of the four pieces never change, and rows past the
+  // last key read as zero instead of needing a clamp: no vector instruction
+  // per load.  The plane base goes through readfirstlane because the compiler
+  // cannot see that it is wave-uniform.
+  // (readfirstlane returns a signed int: the casts keep the low word from sign-extending)
+  const uint32_t plane_lo = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(uint64_t)plane);
+  const uint32_t plane_hi = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)((uint64_t)plane >> 32));
+  const uint64_t plane_u = ((uint64_t)plane_hi << 32) | (uint64_t)plane_lo;
+  const uint32_t ahead_u = __builtin_amdgcn_readfirstlane(grp ? 1u : 2u);  // tiles a steady step fetches ahead
+  const uint32_t tile_bytes = kBK * stride_pos * 2;
+  const uint32_t valid_bytes = (kmax * stride_pos + kHeadDim) * 2;  // API bound: a plane spans < 2^32 bytes
+  uint32_t piece_off[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) piece_off[i] = ((row0 + row_step * i) * stride_pos + 8 * ld_c) * 2;
   // LDS store offsets (halves): K rows ld_r + 16 i; V^T rows 8 ld_c + e, two chunk bases
   uint16_t* const ks_store = smem + ld_r * kKsPitch + 8 * ld_c;
   uint16_t* const vt_store_lo = smem + 2 * kKsHalves + (8 * ld_c) * kVtsPitch +
@@ -461,9 +478,13 @@ __global__ __launch_bounds__(kPpThreads, 2) void prefill_pingpong_kernel(Prefill
   uint16_t* const vt_store_hi = smem + 2 * kKsHalves + (8 * ld_c) * kVtsPitch +
                                 8 * ((vt_grp >> 1) ^ vt_swz ^ 1) + 4 * (vt_grp & 1);
   u32x4 stg[4];
-  auto load_piece = [&](uint32_t kt, int i) {
-    const uint32_t row = min(kt * kBK + row0 + row_step * i, kmax);  // clamped: see above
-    stg[i] = load16(plane + (row * stride_pos + 8 * ld_c));
+  auto load_piece = [&](uint32_t kt, int i) {  // kt must be wave-uniform to the compiler
+    const uint32_t off = kt * tile_bytes;
+    // (written as a scalar min and subtract: a saturating subtract would be a vector instruction)
+    const uint32_t left = valid_bytes - __builtin_amdgcn_readfirstlane(min(valid_bytes, off));
+    const __amdgpu_buffer_rsrc_t rsrc =
+        __builtin_amdgcn_make_buffer_rsrc((void*)(plane_u + off), 0, left, kBufferFlags);
+    stg[i] = __builtin_amdgcn_raw_buffer_load_b128(rsrc, piece_off[i], 0, 0);
   };
   // group 0: pieces 0..3 are K rows (4..7 empty); group 1: piece e is V^T row 8 ld_c + e
   auto store_piece = [&](int buf, int e) {
@@ -564,7 +585,7 @@ __global__ __launch_bounds__(kPpThreads, 2) void prefill_pingpong_kernel(Prefill
         // staging last: the loads issued at the end of the previous matrix step have had
         // almost a whole iteration (~2 us) to arrive before their registers are stored
         if (n >= 20 && n < 28) store_piece(grp ? (int)(kt & 1) : (int)((kt + 1) & 1), n - 20);
-        if (n >= 28 && n < 32) load_piece(grp ? kt + 1 : kt + 2, n - 28);
+        if (n >= 28 && n < 32) load_piece(kt + ahead_u, n - 28);
         __builtin_amdgcn_sched_barrier(0);
       }
       return;
