@@ -379,6 +379,9 @@ __global__ __launch_bounds__(kPfThreads, NB == 1 ? 2 : 1) void prefill_kernel(Pr
 // Rows: wave w owns row block w (32 rows) of 8; all 256 rows read the same K/V
 // tiles.  Waves 0-3 stage the K tiles, waves 4-7 the (transposed) V tiles.
 // ---------------------------------------------------------------------------
+typedef __attribute__((address_space(3))) uint16_t LdsHalf;
+typedef __attribute__((address_space(3))) u32x4 LdsU32x4;
+typedef __attribute__((address_space(3))) u32x2 LdsU32x2;
 constexpr int kPpWaves = 8;
 constexpr int kPpThreads = kPpWaves * kWave;
 constexpr int kLdsAhead = 8;  // LDS operand reads in flight ahead of their MFMA
@@ -386,7 +389,10 @@ constexpr int kBufferFlags = 0x00020000;  // raw buffer of 32-bit data, no swizz
 
 template <typename T>
 __global__ __launch_bounds__(kPpThreads, 2) void prefill_pingpong_kernel(PrefillKernelArgs p) {
-  __shared__ __attribute__((aligned(16))) uint16_t smem[2 * kKsHalves + 2 * kVtsHalves];
+  // K tiles [2][64][kKsPitch] then V^T tiles [3][128][kVtsPitch]: V is staged one step
+  // earlier than it is read, so that every operand of a matrix step is in LDS a whole
+  // phase before the step starts and can be requested ahead of the barrier.
+  __shared__ __attribute__((aligned(16))) uint16_t smem[2 * kKsHalves + 3 * kVtsHalves];
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = tid >> 6;
@@ -465,18 +471,25 @@ __global__ __launch_bounds__(kPpThreads, 2) void prefill_pingpong_kernel(Prefill
   const uint32_t plane_lo = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(uint64_t)plane);
   const uint32_t plane_hi = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)((uint64_t)plane >> 32));
   const uint64_t plane_u = ((uint64_t)plane_hi << 32) | (uint64_t)plane_lo;
-  const uint32_t ahead_u = __builtin_amdgcn_readfirstlane(grp ? 1u : 2u);  // tiles a steady step fetches ahead
   const uint32_t tile_bytes = kBK * stride_pos * 2;
   const uint32_t valid_bytes = (kmax * stride_pos + kHeadDim) * 2;  // API bound: a plane spans < 2^32 bytes
   uint32_t piece_off[4];
 #pragma unroll
   for (int i = 0; i < 4; ++i) piece_off[i] = ((row0 + row_step * i) * stride_pos + 8 * ld_c) * 2;
-  // LDS store offsets (halves): K rows ld_r + 16 i; V^T rows 8 ld_c + e, two chunk bases
-  uint16_t* const ks_store = smem + ld_r * kKsPitch + 8 * ld_c;
-  uint16_t* const vt_store_lo = smem + 2 * kKsHalves + (8 * ld_c) * kVtsPitch +
-                                8 * ((vt_grp >> 1) ^ vt_swz) + 4 * (vt_grp & 1);
-  uint16_t* const vt_store_hi = smem + 2 * kKsHalves + (8 * ld_c) * kVtsPitch +
-                                8 * ((vt_grp >> 1) ^ vt_swz ^ 1) + 4 * (vt_grp & 1);
+  // LDS addresses are kept as byte offsets: the buffers span more than the 64 KB an
+  // instruction's immediate offset reaches, so each step forms one base register
+  // per tile (step_base) and everything else is an immediate on top of it.
+  const uint32_t lds0 = (uint32_t)(uintptr_t)(LdsHalf*)smem;
+  auto step_base = [](uint32_t addr) {
+    asm volatile("" : "+v"(addr));  // opaque: keeps the compiler from folding the sum another way
+    return addr;
+  };
+  // store offsets: K rows ld_r + 16 i; V^T rows 8 ld_c + e, two chunk bases
+  const uint32_t ks_store = lds0 + 2 * (ld_r * kKsPitch + 8 * ld_c);
+  const uint32_t vt_store_lo = lds0 + 2 * (2 * kKsHalves + (8 * ld_c) * kVtsPitch +
+                                           8 * ((vt_grp >> 1) ^ vt_swz) + 4 * (vt_grp & 1));
+  const uint32_t vt_store_hi = lds0 + 2 * (2 * kKsHalves + (8 * ld_c) * kVtsPitch +
+                                           8 * ((vt_grp >> 1) ^ vt_swz ^ 1) + 4 * (vt_grp & 1));
   u32x4 stg[4];
   auto load_piece = [&](uint32_t kt, int i) {  // kt must be wave-uniform to the compiler
     const uint32_t off = kt * tile_bytes;
@@ -487,25 +500,34 @@ __global__ __launch_bounds__(kPpThreads, 2) void prefill_pingpong_kernel(Prefill
     stg[i] = __builtin_amdgcn_raw_buffer_load_b128(rsrc, piece_off[i], 0, 0);
   };
   // group 0: pieces 0..3 are K rows (4..7 empty); group 1: piece e is V^T row 8 ld_c + e
-  auto store_piece = [&](int buf, int e) {
-    if (grp == 0) {
-      if (e < 4) store16(ks_store + buf * kKsHalves + 16 * e * kKsPitch, stg[e]);
+  // (the group comes as a compile-time constant where the caller runs behind the scalar
+  // branch on the group, as the run-time value in the prologue)
+  // base_lo / base_hi: step_base of the destination buffer (group 0 uses base_lo only)
+  auto store_piece = [&](auto group, uint32_t base_lo, uint32_t base_hi, int e) {
+    if (group == 0) {
+      if (e < 4) *(LdsU32x4*)(base_lo + 2 * 16 * e * kKsPitch) = stg[e];
     } else {
       const uint32_t sel = (e & 1) ? 0x07060302u : 0x05040100u;  // high or low halves of a pair
       u32x2 col;  // (key 0, key 1), (key 2, key 3) of column e: one byte permute each
       col[0] = __builtin_amdgcn_perm(stg[1][e >> 1], stg[0][e >> 1], sel);
       col[1] = __builtin_amdgcn_perm(stg[3][e >> 1], stg[2][e >> 1], sel);
-      uint16_t* dst = (e < 4 ? vt_store_lo : vt_store_hi) + buf * kVtsHalves + e * kVtsPitch;
-      *(u32x2*)dst = col;
+      *(LdsU32x2*)((e < 4 ? base_lo : base_hi) + 2 * e * kVtsPitch) = col;
     }
   };
   auto load_tile = [&](uint32_t kt) {
 #pragma unroll
     for (int i = 0; i < 4; ++i) load_piece(kt, i);
   };
+  auto store_bases = [&](auto group, int buf, uint32_t& lo, uint32_t& hi) {
+    const uint32_t off = 2 * buf * (group ? kVtsHalves : kKsHalves);
+    lo = step_base((group ? vt_store_lo : ks_store) + off);
+    hi = step_base((group ? vt_store_hi : ks_store) + off);
+  };
   auto store_tile = [&](int buf) {
+    uint32_t lo, hi;
+    store_bases(grp, buf, lo, hi);
 #pragma unroll
-    for (int e = 0; e < 8; ++e) store_piece(buf, e);
+    for (int e = 0; e < 8; ++e) store_piece(grp, lo, hi, e);
   };
 
   float m_run = -INFINITY, l_run = 0.0f;
@@ -516,96 +538,92 @@ __global__ __launch_bounds__(kPpThreads, 2) void prefill_pingpong_kernel(Prefill
     for (int r = 0; r < 16; ++r) oacc[db][r] = 0.0f;
   f32x16 st[2];
   u32x4 pk[4];
+#pragma unroll
+  for (int cc = 0; cc < 4; ++cc) pk[cc] = u32x4{0u, 0u, 0u, 0u};  // P(-1) = 0
 
-  // prologue: K(0) into LDS, K(1) and V(0) on their way into the staging registers
-  if (grp == 0) {
-    load_tile(0);
-    store_tile(0);
-    if (n_tiles > 1) load_tile(1);
-  } else {
-    load_tile(0);
+  // Every matrix step runs the same straight-line code, the first and the last
+  // included: step 0 multiplies P(-1) = 0 by a zeroed "V(-1)" buffer, step n_tiles
+  // multiplies Q by whatever finite K tile its buffer still holds and nobody reads
+  // the result; tiles past the last one are fetched as zeros (the buffer
+  // descriptor has no bytes left) and stored where nothing reads them.
+  // prologue: K(0) and V(0) into LDS, K(1) and V(1) on their way into the staging
+  // registers, zeros into the V^T buffer that step 0 reads.
+  if (grp) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) stg[i] = u32x4{0u, 0u, 0u, 0u};
+    store_tile(2);
   }
+  load_tile(0);
+  store_tile(0);
+  load_tile(1);
   __syncthreads();
 
   // Matrix step kt = P.V of tile kt-1 and Q.K of tile kt, their MFMAs interleaved
   // (six accumulator chains instead of four or two, so no MFMA waits on the
-  // one before it); group 0 then stores K(kt+1) and fetches K(kt+2), group 1
-  // stores V(kt) and fetches V(kt+1).  Operands come from LDS kLdsAhead reads
-  // ahead of the MFMA that consumes them: issued just in time, every pair of
-  // MFMAs (64 cycles) would wait out a full LDS round trip (100+ cycles).  The
-  // sched_group_barrier sequence pins that order.  STEADY: 1 <= kt and
-  // kt + 2 < n_tiles, so nothing in the step is conditional and the staging
-  // work can be scheduled between the MFMAs.
+  // one before it); then the group stores its tile kt+1 (group 0: K, group 1: V)
+  // and fetches tile kt+2.  K(kt) sits in buffer kt % 2, V(kt) in buffer kt % 3: V is
+  // staged one step before the first step that reads it, so that all operands of
+  // a matrix step are in LDS a whole phase before it starts.  Operands come from
+  // LDS kLdsAhead reads ahead of the MFMA that consumes them: issued just in
+  // time, every pair of MFMAs (64 cycles) would wait out a full LDS round trip
+  // (100+ cycles).  The first kLdsAhead are requested before the barrier that
+  // opens the step (prefetch_ring), so the round trip overlaps the barrier wait.
   const int fj = ((j >> 2) ^ (j >> 3) ^ (j >> 4)) & 1;  // V^T read swizzle, lane part
-  const uint16_t* const k_read = smem + j * kKsPitch + 8 * g;
-  const uint16_t* const vt_read = smem + 2 * kKsHalves + j * kVtsPitch + 8 * (g ^ fj);
-  auto matrix_step = [&](auto steady, uint32_t kt) __attribute__((always_inline)) {
-    constexpr bool kSteady = decltype(steady)::value;
-    const bool do_pv = kSteady || (kt > 0);
-    const bool do_qk = kSteady || (kt < n_tiles);
-    // lane part of the address once, operand part as a compile-time offset
-    const uint16_t* vts = vt_read + ((kt + 1) & 1) * kVtsHalves;  // V(kt-1)
-    const uint16_t* ks = k_read + (kt & 1) * kKsHalves;
-    auto vt_operand = [&](int i) {  // i = 4 cc + db; chunk = (2 cc + g) ^ f = ((2 cc) ^ (2 db)) + (g ^ fj)
-      const int cc = i >> 2, db = i & 3;
-      return load16(vts + 32 * db * kVtsPitch + 8 * ((2 * cc) ^ (2 * db)));
-    };
-    auto k_operand = [&](int i) {  // i = 2 s + mb
+  const uint32_t k_read = lds0 + 2 * (j * kKsPitch + 8 * g);
+  const uint32_t vt_read = lds0 + 2 * (2 * kKsHalves + j * kVtsPitch + 8 * (g ^ fj));
+  auto mod3 = [](uint32_t x) { return x % 3u; };
+  // operand n of the stream of matrix step kt: P.V 0, Q.K 0, P.V 1, Q.K 1, ...
+  // (lane part of the address once per step, operand part as a compile-time offset)
+  auto stream_operand = [&](uint32_t ks, uint32_t vts, int n) {
+    const int i = n >> 1;
+    if (n & 1) {  // K rows: i = 2 s + mb
       const int s = i >> 1, mb = i & 1;
-      return load16(ks + 32 * mb * kKsPitch + 16 * s);
-    };
-    auto qk_mfma = [&](int i, u32x4 a) {
-      const int s = i >> 1, mb = i & 1;
-      if (s == 0) {
-        f32x16 z;
+      return *(const LdsU32x4*)(ks + 2 * (32 * mb * kKsPitch + 16 * s));
+    }
+    // V^T rows: i = 4 cc + db; chunk = (2 cc + g) ^ f = ((2 cc) ^ (2 db)) + (g ^ fj)
+    const int cc = i >> 2, db = i & 3;
+    return *(const LdsU32x4*)(vts + 2 * (32 * db * kVtsPitch + 8 * ((2 * cc) ^ (2 * db))));
+  };
+  u32x4 ring[kLdsAhead];
+  auto prefetch_ring = [&](uint32_t kt) __attribute__((always_inline)) {
+    const uint32_t ks = step_base(k_read + 2 * (kt & 1) * kKsHalves);
+    const uint32_t vts = step_base(vt_read + 2 * mod3(kt + 2) * kVtsHalves);  // V(kt-1)
 #pragma unroll
-        for (int r = 0; r < 16; ++r) z[r] = 0.0f;
-        st[mb] = Mfma<T>::m32x32x16(a, qreg[s], z);
+    for (int n = 0; n < kLdsAhead; ++n) ring[n] = stream_operand(ks, vts, n);
+  };
+  auto matrix_step = [&](auto group, uint32_t kt) __attribute__((always_inline)) {
+    const uint32_t ks = step_base(k_read + 2 * (kt & 1) * kKsHalves);
+    const uint32_t vts = step_base(vt_read + 2 * mod3(kt + 2) * kVtsHalves);
+    uint32_t store_lo, store_hi;
+    store_bases(group, group ? (int)mod3(kt + 1) : (int)((kt + 1) & 1), store_lo, store_hi);
+    // staging work is dealt out between the MFMAs, and a full scheduling barrier
+    // after every MFMA keeps the compiler from regrouping any of it
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int n = 0; n < 32; ++n) {
+      const int i = n >> 1;
+      if (n & 1) {
+        const int s = i >> 1, mb = i & 1;
+        if (s == 0) {
+          f32x16 z;
+#pragma unroll
+          for (int r = 0; r < 16; ++r) z[r] = 0.0f;
+          st[mb] = Mfma<T>::m32x32x16(ring[n % kLdsAhead], qreg[s], z);
+        } else {
+          st[mb] = Mfma<T>::m32x32x16(ring[n % kLdsAhead], qreg[s], st[mb]);
+        }
       } else {
-        st[mb] = Mfma<T>::m32x32x16(a, qreg[s], st[mb]);
+        oacc[i & 3] = Mfma<T>::m32x32x16(ring[n % kLdsAhead], pk[i >> 2], oacc[i & 3]);
       }
-    };
-    if (kSteady) {
-      // operand stream: P.V 0, Q.K 0, P.V 1, Q.K 1, ...; staging work is dealt out
-      // between the MFMAs, and a full scheduling barrier after every MFMA keeps
-      // the compiler from regrouping any of it.
-      auto operand = [&](int n) { return (n & 1) ? k_operand(n >> 1) : vt_operand(n >> 1); };
-      u32x4 ring[kLdsAhead];
-#pragma unroll
-      for (int n = 0; n < kLdsAhead; ++n) ring[n] = operand(n);
+      if (n + kLdsAhead < 32) ring[n % kLdsAhead] = stream_operand(ks, vts, n + kLdsAhead);
+      // staging last: the loads issued at the end of the previous matrix step have had
+      // almost a whole iteration (~2 us) to arrive before their registers are stored
+      if (n >= 20 && n < 28) store_piece(group, store_lo, store_hi, n - 20);
+      if (n >= 28 && n < 32) load_piece(kt + 2, n - 28);
       __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-      for (int n = 0; n < 32; ++n) {
-        const int i = n >> 1;
-        if (n & 1)
-          qk_mfma(i, ring[n % kLdsAhead]);
-        else
-          oacc[i & 3] = Mfma<T>::m32x32x16(ring[n % kLdsAhead], pk[i >> 2], oacc[i & 3]);
-        if (n + kLdsAhead < 32) ring[n % kLdsAhead] = operand(n + kLdsAhead);
-        // staging last: the loads issued at the end of the previous matrix step have had
-        // almost a whole iteration (~2 us) to arrive before their registers are stored
-        if (n >= 20 && n < 28) store_piece(grp ? (int)(kt & 1) : (int)((kt + 1) & 1), n - 20);
-        if (n >= 28 && n < 32) load_piece(kt + ahead_u, n - 28);
-        __builtin_amdgcn_sched_barrier(0);
-      }
-      return;
     }
-    if (do_pv) {
-#pragma unroll
-      for (int i = 0; i < 16; ++i)
-        oacc[i & 3] = Mfma<T>::m32x32x16(vt_operand(i), pk[i >> 2], oacc[i & 3]);
-    }
-    if (do_qk) {
-#pragma unroll
-      for (int i = 0; i < 16; ++i) qk_mfma(i, k_operand(i));
-    }
-    if (grp == 0) {
-      if (kt + 1 < n_tiles) store_tile((kt + 1) & 1);
-      if (kt + 2 < n_tiles) load_tile(kt + 2);
-    } else {
-      if (kt < n_tiles) store_tile(kt & 1);
-      if (kt + 1 < n_tiles) load_tile(kt + 1);
-    }
+    // the barrier that follows carries no wait of its own: wait here for the LDS stores
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
   };
 
   // Vector step kt = soft-max of tile kt: mask on the diagonal, row max, lazy
@@ -653,31 +671,39 @@ __global__ __launch_bounds__(kPpThreads, 2) void prefill_pingpong_kernel(Prefill
     l_run += psum;
   };
 
-  auto matrix_any = [&](uint32_t kt) __attribute__((always_inline)) {
-    if (kt >= 1 && kt + 2 < n_tiles)
-      matrix_step(std::true_type{}, kt);
-    else
-      matrix_step(std::false_type{}, kt);
-  };
-
   // Phases, one workgroup barrier apart: group 0 runs matrix(0) | vector(0) |
   // matrix(1) | vector(1) ... matrix(n_tiles); group 1 runs the same sequence one
-  // phase later.
-  if (grp == 0) matrix_any(0);
-  __syncthreads();
-  for (uint32_t kt = 0; kt < n_tiles; ++kt) {
-    if (grp == 0)
+  // phase later.  One loop per group behind a scalar branch (the wave number goes
+  // through readfirstlane so that the compiler knows a wave runs one of them
+  // only; in a shared loop body it keeps the two groups' values apart and
+  // runs out of registers).  A vector step has no LDS traffic, so it leaves the
+  // operand requests for the next matrix step in flight across the barrier.
+  constexpr std::integral_constant<int, 0> kGroup0;
+  constexpr std::integral_constant<int, 1> kGroup1;
+  if (__builtin_amdgcn_readfirstlane(grp) == 0) {
+    prefetch_ring(0);
+    matrix_step(kGroup0, 0);
+    __builtin_amdgcn_s_barrier();
+    for (uint32_t kt = 0; kt < n_tiles; ++kt) {
       vector_step(kt);
-    else
-      matrix_any(kt);
-    __syncthreads();
-    if (grp == 0)
-      matrix_any(kt + 1);
-    else
+      prefetch_ring(kt + 1);
+      __builtin_amdgcn_s_barrier();
+      matrix_step(kGroup0, kt + 1);
+      __builtin_amdgcn_s_barrier();
+    }
+  } else {
+    prefetch_ring(0);
+    __builtin_amdgcn_s_barrier();
+    for (uint32_t kt = 0; kt < n_tiles; ++kt) {
+      matrix_step(kGroup1, kt);
+      __builtin_amdgcn_s_barrier();
       vector_step(kt);
-    __syncthreads();
+      prefetch_ring(kt + 1);
+      __builtin_amdgcn_s_barrier();
+    }
+    matrix_step(kGroup1, n_tiles);
   }
-  if (grp == 1) matrix_any(n_tiles);
+
 
   {
     const float l = sum_with_partner_half(l_run);
