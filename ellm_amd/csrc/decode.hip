@@ -75,6 +75,24 @@ __device__ __forceinline__ void store_coherent64(float* p, float lo, float hi) {
                         ((uint64_t)__builtin_bit_cast(uint32_t, hi) << 32);
   __hip_atomic_store((uint64_t*)p, bits, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
+// Agent-scope load of four floats.  The compiler has no 16-byte atomic load, so the
+// instruction is written out (sc1 = agent scope, as its own 8-byte atomic loads carry)
+// and the caller waits for it with wait_loaded() before touching the result.
+__device__ __forceinline__ f32x4 load_coherent128_nowait(const float* p) {
+  f32x4 v;
+  asm volatile("global_load_dwordx4 %0, %1, off sc1" : "=v"(v) : "v"(p) : "memory");
+  return v;
+}
+// Wait for every outstanding vector-memory operation; the registers go through the
+// statement so that no use of them can be scheduled ahead of the wait.
+__device__ __forceinline__ void wait_loaded(f32x4 (&v)[16]) {
+  asm volatile("s_waitcnt vmcnt(0)"
+               : "+v"(v[0]), "+v"(v[1]), "+v"(v[2]), "+v"(v[3]), "+v"(v[4]), "+v"(v[5]), "+v"(v[6]),
+                 "+v"(v[7]));
+  asm volatile(""
+               : "+v"(v[8]), "+v"(v[9]), "+v"(v[10]), "+v"(v[11]), "+v"(v[12]), "+v"(v[13]),
+                 "+v"(v[14]), "+v"(v[15]));
+}
 // Block until every vector-memory operation this wave has issued is complete
 // (s_waitcnt vmcnt(0); expcnt and lgkmcnt left at their maxima).
 __device__ __forceinline__ void wait_vm_done() { __builtin_amdgcn_s_waitcnt(0x0F70); }
@@ -321,11 +339,12 @@ __global__ __launch_bounds__(kDecWaves* kWave, DEPTH == 1 ? 4 : 3) void decode_s
     return s_last != 0;
   };
   // Fold `count` (<= 16) partials of every head of this group, starting at
-  // partial `first` of a table with `pitch` partials per row.  Every load a
-  // thread needs is issued before anything is waited for, so a fold costs one
-  // trip to memory: an 8-byte (max, sum) pair per thread, shared through LDS,
-  // and 8-byte accumulator pairs for the thread's (head, d pair) items.
-  // emit(h, dp, a0, a1, sum, max) receives columns 2 dp and 2 dp + 1.
+  // partial `first` of a table with `pitch` partials per row.  A thread owns four
+  // consecutive columns of one head (one item; eight heads make 256 items, one per
+  // thread) and issues every load it needs before it waits for any: a fold costs
+  // one trip to memory, an 8-byte (max, sum) pair per thread, shared through LDS,
+  // and one 16-byte accumulator quad per partial.
+  // emit(h, dq, a[4], sum, max) receives columns 4 dq .. 4 dq + 3.
   auto fold = [&](const float* acc_tab, const float* ml_tab, uint32_t pitch, uint32_t first,
                   uint32_t count, auto emit) {
     float* sm = (float*)smem;  // [head][kMergeFan][2]; the staging buffers are idle by now
@@ -335,21 +354,22 @@ __global__ __launch_bounds__(kDecWaves* kWave, DEPTH == 1 ? 4 : 3) void decode_s
     if ((uint32_t)tid < n_ml)
       ml_bits = load_coherent64(
           ml_tab + (((size_t)seq * p.n_q_heads + head0 + h_e) * pitch + first + s_e) * 2);
-    const uint32_t items = heads_here * (kHeadDim / 2);
+    const uint32_t items = heads_here * (kHeadDim / 4);
     bool published = false;
     for (uint32_t item = tid; item < (items + kDecWaves * kWave - 1) / (kDecWaves * kWave) *
                                          (kDecWaves * kWave);
          item += kDecWaves * kWave) {  // same trip count for every thread: the loop holds a barrier
       const bool mine = item < items;
-      const uint32_t h = mine ? item / (kHeadDim / 2) : 0, dp = item % (kHeadDim / 2);
+      const uint32_t h = mine ? item / (kHeadDim / 4) : 0, dq = item % (kHeadDim / 4);
       const float* ac =
-          acc_tab + (((size_t)seq * p.n_q_heads + head0 + h) * pitch + first) * kHeadDim + 2 * dp;
-      uint64_t av[kMergeFan];
+          acc_tab + (((size_t)seq * p.n_q_heads + head0 + h) * pitch + first) * kHeadDim + 4 * dq;
+      f32x4 av[kMergeFan];
 #pragma unroll
       for (int i = 0; i < kMergeFan; ++i) {
-        const uint32_t sidx = min((uint32_t)i, count - 1);
-        av[i] = mine ? load_coherent64(ac + (size_t)sidx * kHeadDim) : 0;
+        av[i] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+        if ((uint32_t)i < count) av[i] = load_coherent128_nowait(ac + (size_t)i * kHeadDim);
       }
+      wait_loaded(av);  // (also covers ml_bits: the compiler's own wait for it comes no later)
       if (!published) {
         if ((uint32_t)tid < n_ml) *(uint64_t*)(sm + (h_e * kMergeFan + s_e) * 2) = ml_bits;
         __syncthreads();
@@ -359,24 +379,27 @@ __global__ __launch_bounds__(kDecWaves* kWave, DEPTH == 1 ? 4 : 3) void decode_s
       const float* hm = sm + h * kMergeFan * 2;
       float m_new = hm[0];
       for (uint32_t i = 1; i < count; ++i) m_new = fmaxf(m_new, hm[2 * i]);
-      float l_acc = 0.0f, a0 = 0.0f, a1 = 0.0f;
+      float l_acc = 0.0f;
+      f32x4 a = {0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
       for (int i = 0; i < kMergeFan; ++i) {
         if ((uint32_t)i < count) {
           const float wgt = fast_exp2(hm[2 * i] - m_new);
           l_acc += wgt * hm[2 * i + 1];
-          a0 += wgt * __builtin_bit_cast(float, (uint32_t)av[i]);
-          a1 += wgt * __builtin_bit_cast(float, (uint32_t)(av[i] >> 32));
+          a += wgt * av[i];
         }
       }
-      emit(h, dp, a0, a1, l_acc, m_new);
+      emit(h, dq, a, l_acc, m_new);
     }
   };
-  auto emit_final = [&](uint32_t h, uint32_t dp, float a0, float a1, float l, float m) {
+  auto emit_final = [&](uint32_t h, uint32_t dq, const f32x4& a, float l, float m) {
     const size_t row = (size_t)seq * p.n_q_heads + head0 + h;
     const float inv = 1.0f / l;
-    *(uint32_t*)(p.out + row * kHeadDim + 2 * dp) = Mfma<T>::pack2(a0 * inv, a1 * inv);
-    if (p.lse && dp == 0) p.lse[row] = (m + fast_log2(l)) * kLn2;
+    u32x2 w;
+    w[0] = Mfma<T>::pack2(a[0] * inv, a[1] * inv);
+    w[1] = Mfma<T>::pack2(a[2] * inv, a[3] * inv);
+    *(u32x2*)(p.out + row * kHeadDim + 4 * dq) = w;
+    if (p.lse && dq == 0) p.lse[row] = (m + fast_log2(l)) * kLn2;
   };
 
   if (!arrive(ctr + 1 + cluster, in_cluster)) return;
@@ -385,10 +408,11 @@ __global__ __launch_bounds__(kDecWaves* kWave, DEPTH == 1 ? 4 : 3) void decode_s
     return;
   }
   fold(p.ws_acc, p.ws_ml, p.n_split, cluster * kMergeFan, in_cluster,
-       [&](uint32_t h, uint32_t dp, float a0, float a1, float l, float m) {
+       [&](uint32_t h, uint32_t dq, const f32x4& a, float l, float m) {
          const size_t crow = ((size_t)seq * p.n_q_heads + head0 + h) * p.n_cluster_max + cluster;
-         store_coherent64(p.ws2_acc + crow * kHeadDim + 2 * dp, a0, a1);
-         if (dp == 0) store_coherent64(p.ws2_ml + crow * 2, m, l);
+         store_coherent64(p.ws2_acc + crow * kHeadDim + 4 * dq, a[0], a[1]);
+         store_coherent64(p.ws2_acc + crow * kHeadDim + 4 * dq + 2, a[2], a[3]);
+         if (dq == 0) store_coherent64(p.ws2_ml + crow * 2, m, l);
        });
   if (!arrive(ctr, n_clusters)) return;
   fold(p.ws2_acc, p.ws2_ml, p.n_cluster_max, 0, n_clusters, emit_final);
