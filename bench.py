@@ -32,9 +32,9 @@ HBM_PEAK_GBS = 8000.0       # MI355X HBM3E, published
 # copy of known size; summaries and commands under profiles/).  Not measurable from inside
 # this script; null for workloads without a counter run.
 TRAFFIC_BYTES = {
-    "decode": (264960 + 2459) * 1024,          # 16 x 8192 and 1 x 131072 dispatches averaged
-    "decode128k": (264960 + 2459) * 1024,
-    "prefill": (1363420 + 362270) * 1024,
+    "decode": (264959 + 2523) * 1024,          # 16 x 8192 and 1 x 131072 dispatches averaged
+    "decode128k": (264959 + 2523) * 1024,
+    "prefill": (1363516 + 319881) * 1024,
 }
 MFMA_F16_PEAK_TFLOPS = 2500.0  # MI355X dense fp16/bf16 MFMA, published
 D = 128
