@@ -145,6 +145,40 @@ def bench_prefill(seq, steps, warmup, hq=32, hkv=4, dtype_name="f16", p0=0):
     }
 
 
+def bench_ragged_decode(batch, lo, hi, steps, warmup, hq=32, hkv=4, seed=7):
+    """One single-token step over `batch` sequences whose cache lengths are drawn
+    uniformly from [lo, hi] (per-sequence positions on the device)."""
+    import numpy as np
+    import torch
+
+    import ellm_amd
+
+    rng = np.random.default_rng(seed)
+    lengths = rng.integers(lo, hi + 1, size=batch)
+    cap = int(hi)
+    scale = 1.0 / D ** 0.5
+    k = torch.empty((batch, hkv, cap, D), dtype=torch.float16, device="cuda").normal_()
+    v = torch.empty((batch, hkv, cap, D), dtype=torch.float16, device="cuda").normal_()
+    q = _dev_normal((1, batch, hq, D), torch.float16, 301)
+    out = torch.zeros_like(q)
+    pos = torch.tensor((lengths - 1).astype(np.int32), dtype=torch.int32, device="cuda")
+    op = ellm_amd.Attention(q, k, v, out, batch, hq, hkv, D, [hkv * cap * D, cap * D, D, 1], scale,
+                            sequence_capacity=cap, max_position_interval=1)
+    max_pos = int(lengths.max() - 1)
+    per, step_ms = _time_steps(lambda i: op.run_ragged(pos, max_pos, batch), steps, warmup)
+    alg_bytes = int(2 * hkv * D * 2 * lengths.sum() + 2 * batch * hq * D * 2)
+    kern_ms = sum(per) / len(per)
+    op.close()
+    return {
+        "alg_bytes": alg_bytes,
+        "ms_per_step": step_ms,
+        "kernel_ms": kern_ms,
+        "gbs": alg_bytes / (step_ms * 1e-3) / 1e9,
+        "kernel_gbs": alg_bytes / (kern_ms * 1e-3) / 1e9,
+        "tokens": int(lengths.sum()),
+    }
+
+
 def cpu_baseline_decode(batch, length, hq=32, hkv=4, budget_s=20.0):
     """The CPU oracle on the full single-token workload (all host cores)."""
     import numpy as np
@@ -178,7 +212,7 @@ def main():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--skip-cpu", action="store_true")
-    ap.add_argument("--only", default="", help="decode | prefill | decode128k")
+    ap.add_argument("--only", default="", help="decode | prefill | decode128k | chunk | mixed")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="first run one plain 256 MiB device copy (a known-traffic dispatch "
                          "for scaling rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE readings)")
@@ -231,6 +265,39 @@ def main():
                          "peak": HBM_PEAK_GBS, "unit": "GB/s",
                          "frac": round(d128["kernel_gbs"] / HBM_PEAK_GBS, 4),
                          "traffic": TRAFFIC_BYTES["decode128k"]},
+        })
+
+    if args.only in ("", "chunk"):
+        ck_steps = max(3, min(args.steps, 5))
+        ck = bench_prefill(8192, ck_steps, min(args.warmup, 1), hq=64, hkv=8, dtype_name="bf16",
+                           p0=120000)
+        also.append({
+            "workload": "chunked prefill: 8192 new tokens on a 120000-token cache, 64q/8kv heads, "
+                        "bf16 (BASELINE configs[3])",
+            "metric": "prefill attn TFLOP/s", "value": round(ck["tflops"], 2), "unit": "TFLOP/s",
+            "ms_per_step": round(ck["ms_per_step"], 4), "steps": ck_steps,
+            "roofline": {"bound": "mfma", "achieved": round(ck["kernel_tflops"], 2),
+                         "peak": MFMA_F16_PEAK_TFLOPS, "unit": "TFLOP/s",
+                         "frac": round(ck["kernel_tflops"] / MFMA_F16_PEAK_TFLOPS, 4),
+                         "traffic": None},
+        })
+    if args.only in ("", "mixed"):
+        # one layer of BASELINE configs[4]: a 16384-token prefill and a single-token step over 32
+        # sequences with cache lengths U{1024..131072}; the configuration runs this 48 times a step
+        mx_steps = max(3, min(args.steps, 10))
+        mp = bench_prefill(16384, mx_steps, min(args.warmup, 2))
+        md = bench_ragged_decode(32, 1024, 131072, mx_steps, min(args.warmup, 2))
+        also.append({
+            "workload": "mixed step, one of 48 layers (BASELINE configs[4]): prefill 16384 tokens + "
+                        "single-token step over 32 sequences, cache lengths U{1024..131072} (seed 7)",
+            "metric": "attention ms per layer",
+            "value": round(mp["ms_per_step"] + md["ms_per_step"], 4), "unit": "ms",
+            "prefill_ms": round(mp["ms_per_step"], 4), "prefill_tflops": round(mp["tflops"], 1),
+            "decode_ms": round(md["ms_per_step"], 4), "decode_gbs": round(md["gbs"], 1),
+            "decode_cached_tokens": md["tokens"], "steps": mx_steps,
+            "roofline": {"bound": "hbm", "achieved": round(md["kernel_gbs"], 1),
+                         "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                         "frac": round(md["kernel_gbs"] / HBM_PEAK_GBS, 4), "traffic": None},
         })
 
     cpu = None
