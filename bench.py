@@ -179,6 +179,33 @@ def bench_ragged_decode(batch, lo, hi, steps, warmup, hq=32, hkv=4, seed=7):
     }
 
 
+def bench_kv_write(n_tokens, steps, warmup, hkv=4, seqs=1):
+    """Key rows RMS-normalised and rotated, value rows copied, both written to their
+    token coordinates of the cache (the step before attention in a layer)."""
+    import torch
+
+    import ellm_amd
+
+    cap = n_tokens
+    copies = 6   # sources and cache layers rotate (6 x 128 MiB) so that no step finds its rows cached
+    cache = ellm_amd.KVCache(copies, seqs, hkv, cap, ellm_amd.DTYPE_F16)
+    ks = [_dev_normal((n_tokens, seqs, hkv, D), torch.float16, 21 + c) for c in range(copies)]
+    vs = [_dev_normal((n_tokens, seqs, hkv, D), torch.float16, 41 + c) for c in range(copies)]
+    j = torch.arange(D // 2, device="cuda", dtype=torch.float64)
+    ang = torch.arange(cap, device="cuda", dtype=torch.float64)[:, None] * (1.0e6 ** (-2.0 * j / D))[None, :]
+    rope = torch.stack((torch.cos(ang), torch.sin(ang)), dim=-1).reshape(cap, D).to(torch.float16)
+    per, step_ms = _time_steps(
+        lambda i: cache.append_norm_rope(i % copies, 0, ks[i % copies], vs[i % copies], rope),
+        steps, warmup)
+    rows = n_tokens * seqs * hkv
+    alg_bytes = rows * D * 2 * 4 + cap * D * 2          # K, V read and written; the table read once
+    kern_ms = sum(per) / len(per)
+    cache.close()
+    return {"alg_bytes": alg_bytes, "ms_per_step": step_ms, "kernel_ms": kern_ms,
+            "gbs": alg_bytes / (step_ms * 1e-3) / 1e9,
+            "kernel_gbs": alg_bytes / (kern_ms * 1e-3) / 1e9}
+
+
 def cpu_baseline_decode(batch, length, hq=32, hkv=4, budget_s=20.0):
     """The CPU oracle on the full single-token workload (all host cores)."""
     import numpy as np
@@ -212,7 +239,7 @@ def main():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--skip-cpu", action="store_true")
-    ap.add_argument("--only", default="", help="decode | prefill | decode128k | chunk | mixed")
+    ap.add_argument("--only", default="", help="decode | prefill | decode128k | chunk | mixed | kvwrite")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="first run one plain 256 MiB device copy (a known-traffic dispatch "
                          "for scaling rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE readings)")
@@ -298,6 +325,18 @@ def main():
             "roofline": {"bound": "hbm", "achieved": round(md["kernel_gbs"], 1),
                          "peak": HBM_PEAK_GBS, "unit": "GB/s",
                          "frac": round(md["kernel_gbs"] / HBM_PEAK_GBS, 4), "traffic": None},
+        })
+
+    if args.only in ("", "kvwrite"):
+        kw = bench_kv_write(32768, args.steps, args.warmup)
+        also.append({
+            "workload": "cache write with key RMS norm + rotary rotation: 32768 tokens x 4 kv heads, "
+                        "fp16 (the K/V rows of the 32k prefill)",
+            "metric": "kv write HBM GB/s", "value": round(kw["gbs"], 1), "unit": "GB/s",
+            "ms_per_step": round(kw["ms_per_step"], 5), "steps": args.steps,
+            "roofline": {"bound": "hbm", "achieved": round(kw["kernel_gbs"], 1),
+                         "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                         "frac": round(kw["kernel_gbs"] / HBM_PEAK_GBS, 4), "traffic": None},
         })
 
     cpu = None

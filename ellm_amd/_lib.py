@@ -70,6 +70,8 @@ ABI_SYMBOLS = {
     "ellm_kv_destroy": (ctypes.c_int, [_vp]),
     "ellm_kv_layer": (ctypes.c_int, [_vp, _sz, _pvp, _pvp, ctypes.POINTER(_sz * 4)]),
     "ellm_kv_append": (ctypes.c_int, [_vp, _sz, _sz, _sz, _sz, _vp, _vp, _sz, _vp]),
+    "ellm_kv_append_norm_rope": (ctypes.c_int, [_vp, _sz, _sz, _sz, _sz, _vp, _vp, _sz, _vp, _sz,
+                                                ctypes.c_float, _vp, _sz, _vp]),
 }
 
 _lib = None

@@ -135,6 +135,22 @@ class KVCache:
                                        ctypes.c_void_p(v_src.data_ptr()), pitch,
                                        _stream_ptr(stream)))
 
+    def append_norm_rope(self, layer, position_index, k_src, v_src, rope, eps=1e-6, batch_size=None,
+                         positions=None, max_position=0, stream=None):
+        """append() with the key rows RMS-normalised and rotated by the rotary-table row of
+        their position (rope: [positions, 128] device tensor, (cos, sin) interleaved).
+        positions: optional uint32/int32 device tensor of per-sequence start positions,
+        bounded by max_position."""
+        n_tokens, pitch = k_src.shape[0], k_src.shape[1]
+        if batch_size is None:
+            batch_size = pitch
+        pos_ptr = ctypes.c_void_p(positions.data_ptr()) if positions is not None else None
+        check(self._lib.ellm_kv_append_norm_rope(
+            self._handle, layer, position_index, n_tokens, batch_size,
+            ctypes.c_void_p(k_src.data_ptr()), ctypes.c_void_p(v_src.data_ptr()), pitch,
+            ctypes.c_void_p(rope.data_ptr()), rope.shape[0], ctypes.c_float(eps), pos_ptr,
+            int(max_position), _stream_ptr(stream)))
+
     def close(self):
         if self._handle:
             check(self._lib.ellm_kv_destroy(self._handle))

@@ -349,4 +349,40 @@ int ellm_kv_append(ellm_kv_cache* c, size_t layer, size_t position_index, size_t
   return ELLM_OK;
 }
 
+int ellm_kv_append_norm_rope(ellm_kv_cache* c, size_t layer, size_t position_index, size_t n_tokens,
+                             size_t batch_size, const void* k_src, const void* v_src,
+                             size_t src_batch_pitch, const void* rope, size_t rope_positions,
+                             float eps, const uint32_t* positions, size_t max_position,
+                             void* stream) {
+  if (!c) return fail(ELLM_ERR_INVALID_ARGUMENT, "null cache");
+  if (n_tokens == 0 || batch_size == 0) return ELLM_OK;
+  if (!k_src || !v_src || !rope) return fail(ELLM_ERR_INVALID_ARGUMENT, "null source or rotary table");
+  if (!aligned16(k_src) || !aligned16(v_src) || !aligned16(rope))
+    return fail(ELLM_ERR_INVALID_ARGUMENT, "sources and rotary table must be 16-byte aligned");
+  if (!(eps >= 0.0f)) return fail(ELLM_ERR_INVALID_ARGUMENT, "eps must be >= 0");
+  if (layer >= c->desc.layers)
+    return fail(ELLM_ERR_OUT_OF_RANGE, "layer %zu of %zu", layer, c->desc.layers);
+  if (batch_size > c->desc.sequences || src_batch_pitch < batch_size)
+    return fail(ELLM_ERR_OUT_OF_RANGE, "batch_size %zu exceeds the cache's %zu sequences or the source pitch %zu",
+                batch_size, c->desc.sequences, src_batch_pitch);
+  // with per-sequence positions the highest start is max_position (entries above it are clamped)
+  const size_t first = positions ? max_position : position_index;
+  if (first >= c->desc.capacity || n_tokens > c->desc.capacity - first)
+    return fail(ELLM_ERR_OUT_OF_RANGE, "positions [%zu, %zu) do not fit the capacity %zu", first,
+                first + n_tokens, c->desc.capacity);
+  if (first + n_tokens > rope_positions)
+    return fail(ELLM_ERR_OUT_OF_RANGE, "positions [%zu, %zu) are beyond the %zu rows of the rotary table",
+                first, first + n_tokens, rope_positions);
+  if (n_tokens > 0xffffffffu / 2 || src_batch_pitch > 65535)
+    return fail(ELLM_ERR_UNSUPPORTED, "n_tokens or src_batch_pitch too large");
+  void* k = (char*)c->k + layer * c->layer_elems * 2;
+  void* v = (char*)c->v + layer * c->layer_elems * 2;
+  hipError_t e = ellm::launch_kv_append_norm_rope(
+      k, v, k_src, v_src, rope, positions, (uint32_t)n_tokens, (uint32_t)batch_size,
+      (uint32_t)src_batch_pitch, (uint32_t)c->desc.kv_head_num, (uint32_t)c->desc.capacity,
+      (uint32_t)position_index, (uint32_t)max_position, eps, c->desc.dtype, (hipStream_t)stream);
+  if (e != hipSuccess) return fail_hip(e, "kv append (norm + rope) launch");
+  return ELLM_OK;
+}
+
 }  // extern "C"

@@ -67,4 +67,15 @@ hipError_t launch_kv_append(void* k_dst, void* v_dst, const void* k_src, const v
                             uint32_t n_kv_heads, uint32_t capacity, uint32_t position_index,
                             hipStream_t stream);
 
+// Same, with RMS norm and rotary rotation of the key rows; rope: [positions][128] of
+// the cache's type, (cos, sin) interleaved; positions (may be null): per-sequence start
+// positions on the device, each clamped to max_start.
+hipError_t launch_kv_append_norm_rope(void* k_dst, void* v_dst, const void* k_src,
+                                      const void* v_src, const void* rope,
+                                      const uint32_t* positions, uint32_t n_tokens, uint32_t batch,
+                                      uint32_t src_batch_pitch, uint32_t n_kv_heads,
+                                      uint32_t capacity, uint32_t position_index,
+                                      uint32_t max_start, float eps, int dtype,
+                                      hipStream_t stream);
+
 }  // namespace ellm

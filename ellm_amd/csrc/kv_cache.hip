@@ -31,7 +31,108 @@ __global__ __launch_bounds__(256) void kv_append_kernel(
   }
 }
 
+// The same write with the key rows normalised and rotated on the way in (what the
+// reference's fused projection does to a finished 128-wide head column,
+// src/kernel/x86_64/f16_512/matmul_rms_complex.rs:76-96, generic forms
+// src/kernel/generic/rms_norm.rs:6-26 and complex_mul.rs:3-20):
+//   y = x / (sqrt(mean(x^2)) + eps);  (e, f) = (a c - b d, a d + b c) for the
+//   interleaved pairs (a, b) of y and (c, d) = (cos, sin) of the rotary row of
+//   the token's position.
+// Sixteen lanes own one row (8 elements each).  All arithmetic is binary32 with
+// one rounding per operation, in the order of the reference's scalar code: the
+// sum of squares runs through the 128 elements from first to last (the sixteen
+// lanes take turns, each adding its eight squares to the running sum it is
+// handed), so the result is the same bits a sequential CPU loop produces.  The
+// extra instructions (about 150 a row) stay well under what the HBM transfer of
+// the row allows.
+template <typename T>
+__global__ __launch_bounds__(256) void kv_append_norm_rope_kernel(
+    uint16_t* __restrict__ k_dst, uint16_t* __restrict__ v_dst, const uint16_t* __restrict__ k_src,
+    const uint16_t* __restrict__ v_src, const uint16_t* __restrict__ rope,
+    const uint32_t* __restrict__ positions, uint32_t n_tokens, uint32_t batch,
+    uint32_t src_batch_pitch, uint32_t n_kv_heads, uint32_t capacity, uint32_t position_index,
+    uint32_t max_start, float eps) {
+#pragma clang fp contract(off)
+  const uint32_t c = threadIdx.x & 15;
+  const size_t rows = (size_t)n_tokens * batch * n_kv_heads;
+  // every lane of a wave runs the same number of trips: the loop holds cross-lane reads
+  const size_t rows_per_pass = (size_t)gridDim.x * (blockDim.x >> 4);
+  const size_t passes = (rows + rows_per_pass - 1) / rows_per_pass;
+  for (size_t pass = 0; pass < passes; ++pass) {
+    const size_t row = pass * rows_per_pass + (size_t)blockIdx.x * (blockDim.x >> 4) + (threadIdx.x >> 4);
+    const bool live = row < rows;
+    size_t r = live ? row : 0;
+    const uint32_t h = r % n_kv_heads;
+    r /= n_kv_heads;
+    const uint32_t b = r % batch;
+    const uint32_t t = r / batch;
+    const uint32_t start = positions ? min(positions[b], max_start) : position_index;
+    const uint32_t pos = start + t;
+    const size_t src = (((size_t)t * src_batch_pitch + b) * n_kv_heads + h) * kHeadDim + 8 * c;
+    const size_t dst = (((size_t)b * n_kv_heads + h) * capacity + pos) * kHeadDim + 8 * c;
+    const u32x4 kraw = load16(k_src + src);
+    const u32x4 vraw = load16(v_src + src);
+    const u32x4 rraw = load16(rope + (size_t)pos * kHeadDim + 8 * c);
+    float x[8], sq[8];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      x[2 * e] = T::to_float((uint16_t)(kraw[e] & 0xffffu));
+      x[2 * e + 1] = T::to_float((uint16_t)(kraw[e] >> 16));
+    }
+#pragma unroll
+    for (int e = 0; e < 8; ++e) sq[e] = x[e] * x[e];
+    float sum = 0.0f;  // sum of squares of all elements before this lane's
+#pragma unroll
+    for (int l = 0; l < 16; ++l) {
+      float mine = sum;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) mine = mine + sq[e];
+      sum = __shfl(mine, l, 16);  // lane l's total moves on to everybody
+    }
+    const float variance = sum / (float)kHeadDim;
+    const float rrms = 1.0f / (sqrtf(variance) + eps);
+    u32x4 out;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      const float a = x[2 * e] * rrms, bb = x[2 * e + 1] * rrms;
+      const float cs = T::to_float((uint16_t)(rraw[e] & 0xffffu));
+      const float sn = T::to_float((uint16_t)(rraw[e] >> 16));
+      const float re = a * cs - bb * sn;
+      const float im = a * sn + bb * cs;
+      out[e] = T::pack2(re, im);
+    }
+    if (live) {
+      store16(k_dst + dst, out);
+      store16(v_dst + dst, vraw);
+    }
+  }
+}
+
 }  // namespace
+
+hipError_t launch_kv_append_norm_rope(void* k_dst, void* v_dst, const void* k_src,
+                                      const void* v_src, const void* rope,
+                                      const uint32_t* positions, uint32_t n_tokens, uint32_t batch,
+                                      uint32_t src_batch_pitch, uint32_t n_kv_heads,
+                                      uint32_t capacity, uint32_t position_index,
+                                      uint32_t max_start, float eps, int dtype,
+                                      hipStream_t stream) {
+  const size_t rows = (size_t)n_tokens * batch * n_kv_heads;
+  if (rows == 0) return hipSuccess;
+  size_t blocks = (rows + 15) / 16;
+  if (blocks > 16384) blocks = 16384;
+  auto go = [&](auto kernel) {
+    hipLaunchKernelGGL(kernel, dim3((uint32_t)blocks), dim3(256), 0, stream, (uint16_t*)k_dst,
+                       (uint16_t*)v_dst, (const uint16_t*)k_src, (const uint16_t*)v_src,
+                       (const uint16_t*)rope, positions, n_tokens, batch, src_batch_pitch,
+                       n_kv_heads, capacity, position_index, max_start, eps);
+  };
+  if (dtype == 0)
+    go(kv_append_norm_rope_kernel<Mfma<F16>>);
+  else
+    go(kv_append_norm_rope_kernel<Mfma<BF16>>);
+  return hipGetLastError();
+}
 
 hipError_t launch_kv_append(void* k_dst, void* v_dst, const void* k_src, const void* v_src,
                             uint32_t n_tokens, uint32_t batch, uint32_t src_batch_pitch,

@@ -162,6 +162,39 @@ int ellm_kv_append(ellm_kv_cache* cache, size_t layer, size_t position_index, si
                    size_t batch_size, const void* k_src, const void* v_src,
                    size_t src_batch_pitch, void* stream);
 
+/*
+ * ellm_kv_append with the key rows normalised and rotated on the way into the
+ * cache; value rows are copied as they are.  Per 128-wide key row x of a token
+ * at position p:
+ *     y = x / (sqrt(mean(x^2)) + eps)                 (RMS norm, weight 1: eps is
+ *                                                     added to the root mean square,
+ *                                                     src/kernel/generic/rms_norm.rs:6-26)
+ *     (k[2j], k[2j+1]) = (y[2j] c - y[2j+1] s, y[2j] s + y[2j+1] c),
+ *                        (c, s) = (rope[p][2j], rope[p][2j+1])
+ *                                                    (src/kernel/generic/complex_mul.rs:3-20)
+ * which is what the reference's fused projection applies to every finished
+ * head column (matmul_finalize_rmsnorm_rope_inplace_3x128,
+ * src/kernel/x86_64/f16_512/matmul_rms_complex.rs:76-96, called from
+ * src/compiler/mul/matmul3.rs:243-254 with eps = 1e-6, :436-451), written
+ * straight to token coordinates as the reference's output_to_kv flag intends
+ * (src/compiler/zip_map/complex_zip.rs:92-100: destination moved by the
+ * position, rotary row advanced one head_size per position).  Arithmetic is
+ * binary32, rounded to the storage type once.
+ *
+ * rope: device, [rope_positions][128] in the cache's dtype, (cos, sin)
+ * interleaved — the reference's "model.position_embedding.weight",
+ * [max_position_embeddings][1][1][head_size] (src/qwen3_moe/attention.rs:258-262).
+ * positions: NULL (every sequence starts at position_index) or device
+ * uint32[batch_size] start positions, one per sequence, for single-token steps
+ * over sequences of different lengths; max_position bounds them (larger
+ * entries are clamped to it) and is what the range checks use.
+ */
+int ellm_kv_append_norm_rope(ellm_kv_cache* cache, size_t layer, size_t position_index,
+                             size_t n_tokens, size_t batch_size, const void* k_src,
+                             const void* v_src, size_t src_batch_pitch, const void* rope,
+                             size_t rope_positions, float eps, const uint32_t* positions,
+                             size_t max_position, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

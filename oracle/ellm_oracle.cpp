@@ -28,11 +28,27 @@
 //   oracle_attention_run_threads    src/serving/start.rs:59-77 (one thread per core,
 //                                   every thread calls run, then the barrier)
 //   oracle_scale_softmax            known answer held in src/kernel/test.rs:605-629
+//   oracle_rms_norm                 src/kernel/generic/rms_norm.rs:6-26 (weight 1; eps is
+//                                   added to the root mean square, not under the root)
+//   oracle_complex_mul              src/kernel/generic/complex_mul.rs:3-20 (interleaved
+//                                   (re, im) pairs; rotary table rows are (cos, sin) pairs)
+//   oracle_norm_rope_row            src/kernel/x86_64/f16_512/matmul_rms_complex.rs:76-96 and
+//                                   src/compiler/mul/matmul3.rs:482-491 (RMS norm then rotation
+//                                   of one 128-wide head row, in place)
+//   oracle_kv_append_norm_rope      the cache write the reference only hints at
+//                                   (output_to_kv, src/compiler/zip_map/complex_zip.rs:92-100:
+//                                   destination advanced by the position, rotary row advanced
+//                                   by one head_size per position): key rows normalised and
+//                                   rotated with the row of their position, value rows copied
 //
 // Pins (checked in tests/test_oracle_*.py): the all-ones known answer, the 1*1+2*2
 // literal, dot products 32 / 128 / 38, the 18-value scale_softmax literal, the
 // assign literals, closed forms (position 0, equal scores, constant V, shift
-// invariance), chunk invariance, a float64 two-pass brute force and torch SDPA.
+// invariance), chunk invariance, a float64 two-pass brute force and torch SDPA;
+// for the key-row path the 18-value rms_norm literal (rms_norm.rs:54-86), the
+// 34-value complex_mul literal (complex_mul.rs:33-49), fused == separate calls
+// (matmul_rms_complex.rs:215-322), closed forms (unit output RMS, zero row stays
+// zero, rotations keep pair norms) and a float64 restatement.
 
 #include <atomic>
 #include <chrono>
@@ -212,6 +228,27 @@ inline float dot_product(const float* a, const float* b, size_t n) {
 // src/kernel/generic/flash_attention.rs:39-47 — o[i] = s1*o[i] + s2*v[i].
 inline void scalar_vector_mul_and_acc(float s1, float* o, float s2, const float* v, size_t n) {
   for (size_t i = 0; i < n; ++i) o[i] = s1 * o[i] + s2 * v[i];
+}
+
+// src/kernel/generic/rms_norm.rs:6-26 — sequential sum of squares, mean, then
+// 1 / (sqrt(mean) + eps); no weight vector.
+inline void rms_norm(const float* in, float* out, size_t n, float eps) {
+  float sum = in[0] * in[0];
+  for (size_t i = 1; i < n; ++i) sum = sum + in[i] * in[i];
+  const float variance = sum / (float)n;
+  const float rrms = 1.0f / (std::sqrt(variance) + eps);
+  for (size_t i = 0; i < n; ++i) out[i] = in[i] * rrms;
+}
+
+// src/kernel/generic/complex_mul.rs:3-20 — (a + ib)(c + id) on interleaved pairs.
+inline void complex_mul(const float* x, const float* y, float* out, size_t n) {
+  for (size_t i = 0; i + 1 < n; i += 2) {
+    const float a = x[i], b = x[i + 1], c = y[i], d = y[i + 1];
+    const float e = a * c - b * d;
+    const float f = a * d + b * c;
+    out[i] = e;
+    out[i + 1] = f;
+  }
 }
 
 // One query row against keys 0..=position of one K/V plane.
@@ -453,6 +490,55 @@ double ellm_oracle_attention_rows_threads(const ellm_oracle_attn* op, size_t pos
   for (auto& t : pool) t.join();
   const auto t1 = std::chrono::steady_clock::now();
   return std::chrono::duration<double>(t1 - t0).count();
+}
+
+void ellm_oracle_rms_norm_f32(const float* in, float* out, size_t n, float eps) {
+  rms_norm(in, out, n, eps);
+}
+void ellm_oracle_complex_mul_f32(const float* x, const float* y, float* out, size_t n) {
+  complex_mul(x, y, out, n);
+}
+
+// RMS norm then rotation of one stored row, both in binary32, rounded to the
+// storage type once at the end (the reference's all-f16 path rounds after every
+// operation; like its accumulation order that is outside the contract).
+void ellm_oracle_norm_rope_row(const void* row, const void* rope_row, void* out, size_t n,
+                               float eps, int dtype) {
+  std::vector<float> x(n), r(n), y(n);
+  load_row(row, 0, dtype, x.data(), n);
+  load_row(rope_row, 0, dtype, r.data(), n);
+  rms_norm(x.data(), y.data(), n, eps);
+  complex_mul(y.data(), r.data(), x.data(), n);
+  for (size_t i = 0; i < n; ++i) store_elem(out, i, dtype, x[i]);
+}
+
+// Cache write with the key rows normalised and rotated.  Sources are
+// [n_tokens][src_batch_pitch][kv_heads][head_size]; the cache layer is
+// [sequences][kv_heads][capacity][head_size]; rope is [positions][head_size].
+// Token t of sequence b lands at position (positions ? positions[b] : position_index) + t
+// and its key is rotated with that position's row.  Returns 0, or 1 when a
+// position falls outside the cache or the table (nothing is written then).
+int ellm_oracle_kv_append_norm_rope(void* k_cache, void* v_cache, size_t kv_heads, size_t capacity,
+                                    size_t head_size, size_t position_index, size_t n_tokens,
+                                    size_t batch_size, const void* k_src, const void* v_src,
+                                    size_t src_batch_pitch, const void* rope, size_t rope_positions,
+                                    float eps, const uint32_t* positions, int dtype) {
+  for (size_t b = 0; b < batch_size; ++b) {
+    const size_t p0 = positions ? positions[b] : position_index;
+    if (p0 + n_tokens > capacity || p0 + n_tokens > rope_positions) return 1;
+  }
+  const size_t esz = dtype_size(dtype);
+  for (size_t t = 0; t < n_tokens; ++t)
+    for (size_t b = 0; b < batch_size; ++b)
+      for (size_t h = 0; h < kv_heads; ++h) {
+        const size_t pos = (positions ? positions[b] : position_index) + t;
+        const size_t src = ((t * src_batch_pitch + b) * kv_heads + h) * head_size;
+        const size_t dst = ((b * kv_heads + h) * capacity + pos) * head_size;
+        ellm_oracle_norm_rope_row(elem_ptr(k_src, src, dtype), elem_ptr(rope, pos * head_size, dtype),
+                                  elem_ptr(k_cache, dst, dtype), head_size, eps, dtype);
+        std::memcpy(elem_ptr(v_cache, dst, dtype), elem_ptr(v_src, src, dtype), head_size * esz);
+      }
+  return 0;
 }
 
 // Storage conversions exposed so tests can check them against numpy.

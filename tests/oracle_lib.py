@@ -72,6 +72,15 @@ def load():
     lib.ellm_oracle_bf16_to_f32.argtypes = [ctypes.c_uint16]
     lib.ellm_oracle_barrier_selftest.restype = ctypes.c_int
     lib.ellm_oracle_barrier_selftest.argtypes = [sz, sz]
+    lib.ellm_oracle_rms_norm_f32.restype = None
+    lib.ellm_oracle_rms_norm_f32.argtypes = [vp, vp, sz, f]
+    lib.ellm_oracle_complex_mul_f32.restype = None
+    lib.ellm_oracle_complex_mul_f32.argtypes = [vp, vp, vp, sz]
+    lib.ellm_oracle_norm_rope_row.restype = None
+    lib.ellm_oracle_norm_rope_row.argtypes = [vp, vp, vp, sz, f, ctypes.c_int]
+    lib.ellm_oracle_kv_append_norm_rope.restype = ctypes.c_int
+    lib.ellm_oracle_kv_append_norm_rope.argtypes = [vp, vp, sz, sz, sz, sz, sz, sz, vp, vp, sz, vp,
+                                                    sz, f, vp, ctypes.c_int]
     _lib = lib
     return lib
 
@@ -104,6 +113,49 @@ def from_storage(a, dtype):
 
 def storage_np_dtype(dtype):
     return {F16: np.float16, BF16: np.uint16, F32: np.float32}[dtype]
+
+
+def rms_norm(x, eps):
+    """src/kernel/generic/rms_norm.rs restated; x: float32 vector."""
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    out = np.zeros_like(x)
+    load().ellm_oracle_rms_norm_f32(_ptr(x), _ptr(out), x.size, ctypes.c_float(eps))
+    return out
+
+
+def complex_mul(x, y):
+    """src/kernel/generic/complex_mul.rs restated; interleaved (re, im) float32 vectors."""
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    y = np.ascontiguousarray(y, dtype=np.float32)
+    out = np.zeros_like(x)
+    load().ellm_oracle_complex_mul_f32(_ptr(x), _ptr(y), _ptr(out), x.size)
+    return out
+
+
+def norm_rope_row(row, rope_row, eps, dtype):
+    """One stored head row: RMS norm, rotation by one rotary-table row, stored again."""
+    out = np.zeros_like(row)
+    load().ellm_oracle_norm_rope_row(_ptr(row), _ptr(rope_row), _ptr(out), row.size,
+                                     ctypes.c_float(eps), dtype)
+    return out
+
+
+def kv_append_norm_rope(k_cache, v_cache, position_index, k_src, v_src, rope, eps, dtype,
+                        batch_size=None, positions=None):
+    """k_cache / v_cache: [sequence, kv_head, capacity, D] storage arrays, written in place;
+    k_src / v_src: [n_tokens, src_batch_pitch, kv_head, D]; rope: [positions, D].
+    Returns the oracle's status (0 ok, 1 a position outside the cache or the table)."""
+    _, kv_heads, capacity, d = k_cache.shape
+    n_tokens, pitch = k_src.shape[0], k_src.shape[1]
+    if batch_size is None:
+        batch_size = pitch
+    pos = None
+    if positions is not None:
+        pos = np.ascontiguousarray(positions, dtype=np.uint32)
+    return load().ellm_oracle_kv_append_norm_rope(
+        _ptr(k_cache), _ptr(v_cache), kv_heads, capacity, d, position_index, n_tokens, batch_size,
+        _ptr(k_src), _ptr(v_src), pitch, _ptr(rope), rope.shape[0], ctypes.c_float(eps),
+        _ptr(pos), dtype)
 
 
 def assign(length, num, idx):
