@@ -35,6 +35,7 @@ TRAFFIC_BYTES = {
     "decode": (264959 + 2523) * 1024,          # 16 x 8192 and 1 x 131072 dispatches averaged
     "decode128k": (264959 + 2523) * 1024,
     "prefill": (1363516 + 319881) * 1024,
+    "kvwrite": (73808 + 65536) * 1024,
 }
 MFMA_F16_PEAK_TFLOPS = 2500.0  # MI355X dense fp16/bf16 MFMA, published
 D = 128
@@ -336,7 +337,8 @@ def main():
             "ms_per_step": round(kw["ms_per_step"], 5), "steps": args.steps,
             "roofline": {"bound": "hbm", "achieved": round(kw["kernel_gbs"], 1),
                          "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                         "frac": round(kw["kernel_gbs"] / HBM_PEAK_GBS, 4), "traffic": None},
+                         "frac": round(kw["kernel_gbs"] / HBM_PEAK_GBS, 4),
+                         "traffic": TRAFFIC_BYTES["kvwrite"]},
         })
 
     cpu = None
