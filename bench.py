@@ -207,6 +207,50 @@ def bench_kv_write(n_tokens, steps, warmup, hkv=4, seqs=1):
             "kernel_gbs": alg_bytes / (kern_ms * 1e-3) / 1e9}
 
 
+def bench_mixed_step(layers, prefill_tokens, batch, lo, hi, steps, warmup, hq=32, hkv=4, seed=7):
+    """One step of the mixed configuration end to end: for each layer a prefill of
+    `prefill_tokens` tokens of one sequence and a single-token step over `batch` other
+    sequences with cache lengths U{lo..hi}, all launches on one stream.  The layers use the
+    same device buffers (a full set of 48 caches at this capacity does not fit; the work per
+    layer is the same and nothing stays in a cache between layers: one layer's K/V is 8.6 GB)."""
+    import numpy as np
+    import torch
+
+    import ellm_amd
+
+    rng = np.random.default_rng(seed)
+    lengths = rng.integers(lo, hi + 1, size=batch)
+    cap = int(hi)
+    scale = 1.0 / D ** 0.5
+    k = torch.empty((batch, hkv, cap, D), dtype=torch.float16, device="cuda").normal_()
+    v = torch.empty((batch, hkv, cap, D), dtype=torch.float16, device="cuda").normal_()
+    q = _dev_normal((1, batch, hq, D), torch.float16, 301)
+    out = torch.zeros_like(q)
+    pos = torch.tensor((lengths - 1).astype(np.int32), dtype=torch.int32, device="cuda")
+    dec = ellm_amd.Attention(q, k, v, out, batch, hq, hkv, D, [hkv * cap * D, cap * D, D, 1], scale,
+                             sequence_capacity=cap, max_position_interval=1)
+    max_pos = int(lengths.max() - 1)
+    pq = _dev_normal((prefill_tokens, 1, hq, D), torch.float16, 311)
+    pk = _dev_normal((1, hkv, prefill_tokens, D), torch.float16, 312)
+    pv = _dev_normal((1, hkv, prefill_tokens, D), torch.float16, 313)
+    pout = torch.zeros_like(pq)
+    pre = ellm_amd.Attention(pq, pk, pv, pout, 1, hq, hkv, D,
+                             [hkv * prefill_tokens * D, prefill_tokens * D, D, 1], scale,
+                             sequence_capacity=prefill_tokens, max_position_interval=prefill_tokens)
+
+    def step(_):
+        for _layer in range(layers):
+            pre.run(0, prefill_tokens, 1)
+            dec.run_ragged(pos, max_pos, batch)
+
+    _, step_ms = _time_steps(step, steps, warmup)
+    flops = layers * 4 * D * hq * (prefill_tokens * (prefill_tokens + 1) // 2)
+    nbytes = layers * int(2 * hkv * D * 2 * lengths.sum() + 2 * batch * hq * D * 2)
+    pre.close()
+    dec.close()
+    return {"ms_per_step": step_ms, "flops": flops, "bytes": nbytes, "tokens": int(lengths.sum())}
+
+
 def cpu_baseline_decode(batch, length, hq=32, hkv=4, budget_s=20.0):
     """The CPU oracle on the full single-token workload (all host cores)."""
     import numpy as np
@@ -240,7 +284,7 @@ def main():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--skip-cpu", action="store_true")
-    ap.add_argument("--only", default="", help="decode | prefill | decode128k | chunk | mixed | kvwrite")
+    ap.add_argument("--only", default="", help="decode | prefill | decode128k | chunk | mixed | mixed48 | kvwrite")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="first run one plain 256 MiB device copy (a known-traffic dispatch "
                          "for scaling rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE readings)")
@@ -328,6 +372,16 @@ def main():
                          "frac": round(md["kernel_gbs"] / HBM_PEAK_GBS, 4), "traffic": None},
         })
 
+    if args.only in ("", "mixed48"):
+        ms = bench_mixed_step(48, 16384, 32, 1024, 131072, 3, 1)
+        also.append({
+            "workload": "mixed step end to end (BASELINE configs[4]): 48 layers x (prefill 16384 tokens + "
+                        "single-token step over 32 sequences, cache lengths U{1024..131072}, seed 7), "
+                        "Q/K/V drawn directly (no projections), one stream",
+            "metric": "attention ms per step", "value": round(ms["ms_per_step"], 3), "unit": "ms",
+            "steps": 3, "prefill_tflop_per_step": round(ms["flops"] / 1e12, 2),
+            "decode_gb_per_step": round(ms["bytes"] / 1e9, 1),
+        })
     if args.only in ("", "kvwrite"):
         kw = bench_kv_write(32768, args.steps, args.warmup)
         also.append({
