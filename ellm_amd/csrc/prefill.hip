@@ -10,18 +10,16 @@
 //
 // Formulation (everything transposed so that one lane owns one query row):
 //   S^T[key][row] = K . Q^T     32x32x16 MFMA, A = K tile from LDS, B = Q in registers
-//   O^T[d][row]  += V^T . P^T   32x32x16 MFMA, A = V^T tile from LDS, B = P^T in registers
+//   O^T[d][row]  += V^T . P^T   32x32x16 MFMA, A = V^T from LDS (transposing read), B = P^T in registers
 // The C layout of S^T (lane = row, registers = keys) is, up to a fixed
 // permutation of keys inside each 16-key group, the B layout the second MFMA
-// wants; V^T is written to LDS with the same permutation, so P never leaves the
+// wants; the V^T operand is read with the same permutation, so P never leaves the
 // lane that produced it and row max / row sum need one cross-lane exchange.
 //
-// A workgroup (4 waves) owns 4*NB blocks of 32 query rows that all read the
-// same K/V plane: up to 8 query heads of one GQA group x consecutive token
-// blocks.  Stacking the group's heads makes each LDS tile feed 4*NB times more
-// MFMA work and keeps the token span (and so the masked part of the diagonal
-// tile) short.
-#include <cstdlib>
+// A workgroup (8 waves) owns 8 blocks of 32 query rows that all read the same
+// K/V plane: up to 8 query heads of one GQA group x consecutive token blocks.
+// Stacking the group's heads makes each LDS tile feed 8 times more MFMA work
+// and keeps the token span (and so the masked part of the diagonal tile) short.
 #include <type_traits>
 
 #include "common.hpp"
@@ -30,13 +28,9 @@
 namespace ellm {
 namespace {
 
-constexpr int kPfWaves = 4;
-constexpr int kPfThreads = kPfWaves * kWave;
 constexpr int kBK = 64;                     // keys per tile
 constexpr int kKsPitch = kHeadDim + 8;      // halves per K row (272 B)
-constexpr int kVtsPitch = kBK + 8;          // halves per V^T row (144 B)
 constexpr int kKsHalves = kBK * kKsPitch;
-constexpr int kVtsHalves = kHeadDim * kVtsPitch;
 constexpr float kRescaleStep = 8.0f;        // log2 units
 
 struct PrefillKernelArgs {
@@ -60,314 +54,8 @@ struct PrefillKernelArgs {
   float c;                   // |scale| * log2(e), > 0
 };
 
-template <typename T, int NB>
-__global__ __launch_bounds__(kPfThreads, NB == 1 ? 2 : 1) void prefill_kernel(PrefillKernelArgs p) {
-  // K tiles [2][64][kKsPitch] then V^T tiles [2][128][kVtsPitch]
-  __shared__ __attribute__((aligned(16))) uint16_t smem[2 * kKsHalves + 2 * kVtsHalves];
-
-  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
-  const int j = lane & 31, g = lane >> 5;
-
-  // ---- which (plane, token block) this workgroup owns ----------------------
-  // Workgroups are dealt to the 8 XCDs round-robin by id.  When the planes
-  // divide 8, id % 8 picks the plane, so each XCD's L2 only ever holds one K/V
-  // plane; in every case long rows (late tokens) come first so the tail of the
-  // launch is made of short work items.
-  uint32_t combo, order;
-  if (p.xcd_mode) {
-    const uint32_t xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
-    const uint32_t per = 8 / p.combos;
-    combo = xcd % p.combos;
-    order = slot * per + xcd / p.combos;
-  } else {
-    combo = blockIdx.x % p.combos;
-    order = blockIdx.x / p.combos;
-  }
-  if (order >= p.n_wg_tokens) return;
-  const uint32_t wg_tok = p.n_wg_tokens - 1 - order;
-  const uint32_t seq = combo / (p.n_kv_heads * p.head_groups);
-  const uint32_t kvh = (combo / p.head_groups) % p.n_kv_heads;
-  const uint32_t hgrp = combo % p.head_groups;
-  const uint32_t t_base = wg_tok * 32 * p.tblocks_per_wg;
-  const uint32_t S = p.interval, P0 = p.position_index;
-
-  const uint32_t wg_last_tok = min(S, t_base + 32 * p.tblocks_per_wg) - 1;
-  const uint32_t kmax = P0 + wg_last_tok;  // last key any row here may see
-  const uint32_t n_tiles = kmax / kBK + 1;
-  // tiles whose 64 keys are visible to every row of this workgroup: no mask needed
-  const uint32_t n_plain = min(n_tiles, (P0 + t_base + 1) / kBK);
-
-  // ---- per row-block bookkeeping -------------------------------------------
-  uint32_t head[NB], tok[NB];
-  bool row_valid[NB];
-#pragma unroll
-  for (int n = 0; n < NB; ++n) {
-    const uint32_t rb = wave * NB + n;
-    const uint32_t hg = rb % p.heads_per_wg, tb = rb / p.heads_per_wg;
-    head[n] = kvh * p.group + hgrp * p.heads_per_wg + hg;
-    const uint32_t tok0 = t_base + 32 * tb;
-    tok[n] = min(tok0 + j, S - 1);  // clamped rows compute a valid row and are not stored
-    row_valid[n] = tok0 + j < S;
-  }
-
-  // ---- Q as the B operand: lane (row j, half g) holds q[row][16 s + 8 g + 0..7] -------
-  u32x4 qreg[NB][8];
-#pragma unroll
-  for (int n = 0; n < NB; ++n) {
-    const uint16_t* qrow =
-        p.q + (size_t)tok[n] * p.q_token_stride + ((size_t)seq * p.n_q_heads + head[n]) * kHeadDim;
-#pragma unroll
-    for (int s = 0; s < 8; ++s) {
-      qreg[n][s] = load16(qrow + 16 * s + 8 * g);
-      if (p.negate_q) qreg[n][s] ^= 0x80008000u;
-    }
-  }
-  const float c = p.c;
-
-  const uint16_t* kplane = p.k + seq * p.kv_stride_seq + kvh * p.kv_stride_head;
-  const uint16_t* vplane = p.v + seq * p.kv_stride_seq + kvh * p.kv_stride_head;
-
-  // ---- tile staging: HBM -> registers -> LDS -------------------------------
-  const int ld_c = tid & 15;    // 8-element column chunk
-  const int ld_r = tid >> 4;    // 0..15
-  // V^T column position of the 4-key group this thread transposes: the two low
-  // bits of the group index are swapped (see the layout note above).
-  const int vt_grp = (ld_r & ~3) | ((ld_r & 1) << 1) | ((ld_r >> 1) & 1);
-  // 16-byte chunks of a V^T row are XOR-swizzled with bits 4..6 of the row (d)
-  // index: the transposing 8-byte writes (rows 8 apart across lanes) and the
-  // 16-byte operand reads (consecutive rows across lanes) are then both free
-  // of LDS bank conflicts.
-  const int vt_swz = (ld_c >> 1) & 7;
-  u32x4 kreg[4], vreg[4];
-  // rows past kmax are clamped onto it: in bounds, initialised, and masked later
-  auto load_k = [&](uint32_t kt) {
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const uint32_t row = min(kt * kBK + ld_r + 16 * i, kmax);
-      kreg[i] = load16(kplane + (size_t)row * p.kv_stride_pos + 8 * ld_c);
-    }
-  };
-  auto load_v = [&](uint32_t kt) {
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const uint32_t row = min(kt * kBK + 4 * ld_r + i, kmax);
-      vreg[i] = load16(vplane + (size_t)row * p.kv_stride_pos + 8 * ld_c);
-    }
-  };
-  auto store_k = [&](int buf) {
-    uint16_t* ks = smem + buf * kKsHalves;
-#pragma unroll
-    for (int i = 0; i < 4; ++i) store16(ks + (ld_r + 16 * i) * kKsPitch + 8 * ld_c, kreg[i]);
-  };
-  auto store_v = [&](int buf) {
-    uint16_t* vts = smem + 2 * kKsHalves + buf * kVtsHalves;
-#pragma unroll
-    for (int e = 0; e < 8; ++e) {
-      u32x2 col = gather_column(vreg[0][e >> 1], vreg[1][e >> 1], vreg[2][e >> 1],
-                                vreg[3][e >> 1], (e & 1) != 0);
-      *(u32x2*)(vts + (8 * ld_c + e) * kVtsPitch + 8 * ((vt_grp >> 1) ^ vt_swz) +
-                4 * (vt_grp & 1)) = col;
-    }
-  };
-
-  float m_run[NB], l_run[NB];
-  f32x16 oacc[NB][4];
-#pragma unroll
-  for (int n = 0; n < NB; ++n) {
-    m_run[n] = -INFINITY;
-    l_run[n] = 0.0f;
-#pragma unroll
-    for (int db = 0; db < 4; ++db)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) oacc[n][db][r] = 0.0f;
-  }
-
-  // S^T of one tile: K tile (LDS) times Q (registers)
-  auto qk_tile = [&](int kbuf, f32x16 (&st)[NB][2]) {
-    const uint16_t* ks = smem + kbuf * kKsHalves;
-#pragma unroll
-    for (int s = 0; s < 8; ++s) {
-#pragma unroll
-      for (int mb = 0; mb < 2; ++mb) {
-        const u32x4 a = load16(ks + (32 * mb + j) * kKsPitch + 16 * s + 8 * g);
-#pragma unroll
-        for (int n = 0; n < NB; ++n) {
-          if (s == 0) {
-            f32x16 z;
-#pragma unroll
-            for (int r = 0; r < 16; ++r) z[r] = 0.0f;
-            st[n][mb] = Mfma<T>::m32x32x16(a, qreg[n][s], z);
-          } else {
-            st[n][mb] = Mfma<T>::m32x32x16(a, qreg[n][s], st[n][mb]);
-          }
-        }
-      }
-    }
-  };
-
-  // One tile of the software pipeline.  On entry `sc` holds the raw scores of
-  // tile kt, LDS holds K(kt+1) and V(kt), and K(kt+2) / V(kt+1) are on their way
-  // into the staging registers.  The scores of tile kt+1 (MFMA) are computed
-  // next to the row maxima of tile kt (VALU), and the exponentials of tile kt
-  // (VALU) next to its P.V products (MFMA), so that both pipes have work in the
-  // same stretch of straight-line code.
-  auto pipeline_step = [&](auto masked, auto has_next_static, f32x16 (&sc)[NB][2],
-                           f32x16 (&sn)[NB][2], uint32_t kt) {
-    constexpr bool kMasked = decltype(masked)::value;
-    constexpr bool kNextStatic = decltype(has_next_static)::value;
-    const uint32_t kb = kt * kBK;
-    const bool has_next = kNextStatic || (kt + 1 < n_tiles);
-
-    if (kMasked) {
-#pragma unroll
-      for (int n = 0; n < NB; ++n) {
-        const uint32_t rowpos = P0 + tok[n];
-#pragma unroll
-        for (int mb = 0; mb < 2; ++mb)
-#pragma unroll
-          for (int r = 0; r < 16; ++r) {
-            const uint32_t key = kb + 32 * mb + 8 * (r >> 2) + 4 * g + (r & 3);
-            sc[n][mb][r] = (key <= rowpos) ? sc[n][mb][r] : -INFINITY;
-          }
-      }
-    }
-    if (has_next) qk_tile((kt + 1) & 1, sn);
-
-    // Scores stay unscaled; scale*log2(e) (c > 0) is folded into the exponent's
-    // FMA.  The reference max m is only moved when the tile's max exceeds it by
-    // more than kRescaleStep (log2 units), so most tiles skip the rescale of
-    // O^T; probabilities are then at most 2^kRescaleStep, well inside binary16
-    // and bfloat16 range.
-    float neg_m[NB];
-    bool grow_any = false;
-    float tmax[NB];
-#pragma unroll
-    for (int n = 0; n < NB; ++n) {
-      float rmax = sc[n][0][0];
-#pragma unroll
-      for (int mb = 0; mb < 2; ++mb)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) rmax = fmaxf(rmax, sc[n][mb][r]);
-      rmax = fmaxf(rmax, xor_shuffle(rmax, 32));
-      tmax[n] = rmax * c;
-      grow_any |= tmax[n] > m_run[n] + kRescaleStep;
-    }
-    if (__any(grow_any)) {
-#pragma unroll
-      for (int n = 0; n < NB; ++n) {
-        const bool grow = tmax[n] > m_run[n] + kRescaleStep;
-        const float m_new = grow ? tmax[n] : m_run[n];
-        const float alpha = grow ? fast_exp2(m_run[n] - m_new) : 1.0f;
-        m_run[n] = m_new;
-        l_run[n] *= alpha;
-#pragma unroll
-        for (int db = 0; db < 4; ++db) oacc[n][db] *= alpha;
-      }
-    }
-#pragma unroll
-    for (int n = 0; n < NB; ++n)  // finite from tile 0 on; the guard keeps -inf - -inf out
-      neg_m[n] = (m_run[n] == -INFINITY) ? 0.0f : -m_run[n];
-
-    // exponentials of 16-key chunk cc, then that chunk's four P.V products.  The
-    // row sum adds the unrounded binary32 probabilities: summing the rounded ones
-    // would move the log-sum-exp by up to half a storage ulp, beyond 1e-4.
-    const uint16_t* vts = smem + 2 * kKsHalves + (kt & 1) * kVtsHalves;
-    float psum[NB];
-#pragma unroll
-    for (int n = 0; n < NB; ++n) psum[n] = 0.0f;
-#pragma unroll
-    for (int cc = 0; cc < 4; ++cc) {
-      const int mb = cc >> 1, r0 = 8 * (cc & 1);
-      u32x4 pk[NB];
-#pragma unroll
-      for (int n = 0; n < NB; ++n)
-#pragma unroll
-        for (int w = 0; w < 4; ++w) {
-          const float p0 = fast_exp2(__builtin_fmaf(sc[n][mb][r0 + 2 * w], c, neg_m[n]));
-          const float p1 = fast_exp2(__builtin_fmaf(sc[n][mb][r0 + 2 * w + 1], c, neg_m[n]));
-          pk[n][w] = Mfma<T>::pack2(p0, p1);
-          psum[n] += p0 + p1;
-        }
-#pragma unroll
-      for (int db = 0; db < 4; ++db) {
-        const int chunk = (2 * cc + g) ^ ((2 * db + (j >> 4)) & 7);
-        const u32x4 a = load16(vts + (32 * db + j) * kVtsPitch + 8 * chunk);
-#pragma unroll
-        for (int n = 0; n < NB; ++n) oacc[n][db] = Mfma<T>::m32x32x16(a, pk[n], oacc[n][db]);
-      }
-    }
-#pragma unroll
-    for (int n = 0; n < NB; ++n) l_run[n] += psum[n];
-
-    // K(kt+2) -> the K buffer tile kt lived in, V(kt+1) -> the other V buffer;
-    // then start the next pair of loads into the same registers.
-    if (kt + 2 < n_tiles) store_k(kt & 1);
-    if (kt + 1 < n_tiles) store_v((kt + 1) & 1);
-    if (kt + 3 < n_tiles) load_k(kt + 3);
-    if (kt + 2 < n_tiles) load_v(kt + 2);
-    __syncthreads();
-  };
-
-  // ---- prologue -----------------------------------------------------------------
-  f32x16 sa[NB][2], sb[NB][2];
-  load_k(0);
-  load_v(0);
-  store_k(0);
-  store_v(0);
-  if (n_tiles > 1) {
-    load_k(1);
-    store_k(1);
-  }
-  if (n_tiles > 2) load_k(2);
-  if (n_tiles > 1) load_v(1);
-  __syncthreads();
-  qk_tile(0, sa);
-  __syncthreads();  // tile 0 of K is overwritten at the end of the first step
-
-  // ---- main loop: plain tiles with a successor, two per trip so that the two
-  // score buffers swap roles without register copies ------------------------------
-  const uint32_t n_main = min(n_plain, n_tiles - 1);
-  uint32_t kt = 0;
-  using yes = std::true_type;
-  using no = std::false_type;
-  for (; kt + 2 <= n_main; kt += 2) {
-    pipeline_step(no{}, yes{}, sa, sb, kt);
-    pipeline_step(no{}, yes{}, sb, sa, kt + 1);
-  }
-  // ---- remaining tiles (odd one out, tiles crossing the diagonal, last tile) -------
-  for (; kt < n_tiles; ++kt) {
-    pipeline_step(yes{}, no{}, sa, sb, kt);
-#pragma unroll
-    for (int n = 0; n < NB; ++n)
-#pragma unroll
-      for (int mb = 0; mb < 2; ++mb) sa[n][mb] = sb[n][mb];
-  }
-
-  // ---- epilogue: normalise, convert, store ----------------------------------
-#pragma unroll
-  for (int n = 0; n < NB; ++n) {
-    float l = l_run[n] + xor_shuffle(l_run[n], 32);
-    if (!row_valid[n]) continue;
-    const float inv = 1.0f / l;
-    uint16_t* orow =
-        p.out + (size_t)tok[n] * p.q_token_stride + ((size_t)seq * p.n_q_heads + head[n]) * kHeadDim;
-#pragma unroll
-    for (int db = 0; db < 4; ++db)
-#pragma unroll
-      for (int q4 = 0; q4 < 4; ++q4) {
-        u32x2 w;
-        w[0] = Mfma<T>::pack2(oacc[n][db][4 * q4] * inv, oacc[n][db][4 * q4 + 1] * inv);
-        w[1] = Mfma<T>::pack2(oacc[n][db][4 * q4 + 2] * inv, oacc[n][db][4 * q4 + 3] * inv);
-        *(u32x2*)(orow + 32 * db + 8 * q4 + 4 * g) = w;
-      }
-    if (p.lse && g == 0)
-      p.lse[((size_t)tok[n] * p.batch_pitch + seq) * p.n_q_heads + head[n]] =
-          (m_run[n] + fast_log2(l)) * kLn2;
-  }
-}
-
 // ---------------------------------------------------------------------------
-// Ping-pong variant: 8 waves, two per SIMD.  Waves 0-3 and waves 4-7 run the
+// Ping-pong kernel: 8 waves, two per SIMD.  Waves 0-3 and waves 4-7 run the
 // same per-tile sequence  S^T = K.Q^T -> soft-max -> O^T += V^T.P^T  half a
 // step apart: while one group is in its matrix phase (P.V of the previous tile,
 // then Q.K of the next one, plus moving the following K or V tile into LDS) the
@@ -377,7 +65,7 @@ __global__ __launch_bounds__(kPfThreads, NB == 1 ? 2 : 1) void prefill_kernel(Pr
 // ALU work at the same time; left to themselves, two identical workgroups on a
 // compute unit run in lockstep and the two pipes take turns instead.
 // Rows: wave w owns row block w (32 rows) of 8; all 256 rows read the same K/V
-// tiles.  Waves 0-3 stage the K tiles, waves 4-7 the (transposed) V tiles.
+// tiles.  Waves 0-3 stage the K tiles, waves 4-7 the V tiles.
 // ---------------------------------------------------------------------------
 typedef __attribute__((address_space(3))) uint16_t LdsHalf;
 typedef __attribute__((address_space(3))) u32x4 LdsU32x4;
@@ -724,9 +412,9 @@ uint32_t gcd_u32(uint32_t a, uint32_t b) {
   return a;
 }
 
-template <typename T, int NB, bool PP>
-hipError_t launch_nb(const AttnArgs& a, hipStream_t stream) {
-  constexpr uint32_t kRowBlocks = PP ? kPpWaves : kPfWaves * NB;
+template <typename T>
+hipError_t launch_pingpong(const AttnArgs& a, hipStream_t stream) {
+  constexpr uint32_t kRowBlocks = kPpWaves;
   PrefillKernelArgs p;
   p.q = (const uint16_t*)a.q;
   p.k = (const uint16_t*)a.k;
@@ -763,30 +451,15 @@ hipError_t launch_nb(const AttnArgs& a, hipStream_t stream) {
   } else {
     n_wg = p.combos * p.n_wg_tokens;
   }
-  if (PP)
-    hipLaunchKernelGGL((prefill_pingpong_kernel<T>), dim3(n_wg), dim3(kPpThreads), 0, stream, p);
-  else
-    hipLaunchKernelGGL((prefill_kernel<T, NB>), dim3(n_wg), dim3(kPfThreads), 0, stream, p);
+  hipLaunchKernelGGL((prefill_pingpong_kernel<T>), dim3(n_wg), dim3(kPpThreads), 0, stream, p);
   return hipGetLastError();
 }
 
 }  // namespace
 
 hipError_t launch_prefill(const AttnArgs& a, hipStream_t stream) {
-  static const int mode = [] {
-    const char* e = getenv("ELLM_PREFILL_MODE");  // tuning override: 0 ping-pong, 1 / 2 = NB
-    return e ? atoi(e) : 0;
-  }();
-  if (mode == 1) {
-    if (a.dtype == 0) return launch_nb<F16, 1, false>(a, stream);
-    return launch_nb<BF16, 1, false>(a, stream);
-  }
-  if (mode == 2) {
-    if (a.dtype == 0) return launch_nb<F16, 2, false>(a, stream);
-    return launch_nb<BF16, 2, false>(a, stream);
-  }
-  if (a.dtype == 0) return launch_nb<F16, 1, true>(a, stream);
-  return launch_nb<BF16, 1, true>(a, stream);
+  if (a.dtype == 0) return launch_pingpong<F16>(a, stream);
+  return launch_pingpong<BF16>(a, stream);
 }
 
 }  // namespace ellm
