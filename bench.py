@@ -251,6 +251,58 @@ def bench_mixed_step(layers, prefill_tokens, batch, lo, hi, steps, warmup, hq=32
     return {"ms_per_step": step_ms, "flops": flops, "bytes": nbytes, "tokens": int(lengths.sum())}
 
 
+def bench_token_step(layers, batch, length, steps, warmup, hq=32, hkv=4):
+    """One single-token step of a whole model's attention: per layer the fused cache write of
+    the new key / value rows (key RMS norm + rotation) and the attention over the cache, the
+    per-sequence positions advanced on the device at the end; launched eagerly (2 launches a
+    layer + 1) and replayed from a graph recorded once through the library."""
+    import torch
+
+    import ellm_amd
+
+    cap = length + 2 * (steps + warmup) + 8
+    scale = 1.0 / D ** 0.5
+    stream = torch.cuda.Stream()
+    cache = ellm_amd.KVCache(layers, batch, hkv, cap, ellm_amd.DTYPE_F16)
+    j = torch.arange(D // 2, device="cuda", dtype=torch.float64)
+    ang = torch.arange(cap, device="cuda", dtype=torch.float64)[:, None] * (1.0e6 ** (-2.0 * j / D))[None, :]
+    rope = torch.stack((torch.cos(ang), torch.sin(ang)), dim=-1).reshape(cap, D).to(torch.float16)
+    q = _dev_normal((1, batch, hq, D), torch.float16, 401)
+    k1 = _dev_normal((1, batch, hkv, D), torch.float16, 402)
+    v1 = _dev_normal((1, batch, hkv, D), torch.float16, 403)
+    out = torch.zeros_like(q)
+    ops = []
+    for layer in range(layers):
+        kt, vt = cache.layer_tensors(layer, torch.float16)
+        kt.normal_()
+        vt.normal_()
+        _, _, strides = cache.layer(layer)
+        ops.append(ellm_amd.Attention(q, kt, vt, out, batch, hq, hkv, D, strides, scale,
+                                      sequence_capacity=cap, max_position_interval=1))
+    pos = torch.full((batch,), length - 1, dtype=torch.int32, device="cuda")
+    torch.cuda.synchronize()
+
+    def step(_=None):
+        for layer in range(layers):
+            cache.append_norm_rope(layer, 0, k1, v1, rope, positions=pos, max_position=cap - 1)
+            ops[layer].run_ragged(pos, cap - 1, batch)
+        ellm_amd.positions_advance(pos, 1)
+
+    with torch.cuda.stream(stream):
+        _, eager_ms = _time_steps(step, steps, warmup)
+        pos.fill_(length - 1)
+        stream.synchronize()
+        with ellm_amd.StepGraph(stream) as graph:
+            step()
+        _, graph_ms = _time_steps(lambda _i: graph.launch(), steps, warmup)
+    graph.close()
+    for op in ops:
+        op.close()
+    cache.close()
+    nbytes = layers * (2 * batch * hkv * length * D * 2 + 2 * batch * hq * D * 2)
+    return {"eager_ms": eager_ms, "graph_ms": graph_ms, "bytes": nbytes}
+
+
 def cpu_baseline_decode(batch, length, hq=32, hkv=4, budget_s=20.0):
     """The CPU oracle on the full single-token workload (all host cores)."""
     import numpy as np
@@ -284,7 +336,7 @@ def main():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--skip-cpu", action="store_true")
-    ap.add_argument("--only", default="", help="decode | prefill | decode128k | chunk | mixed | mixed48 | kvwrite")
+    ap.add_argument("--only", default="", help="decode | prefill | decode128k | chunk | mixed | mixed48 | kvwrite | tokenstep")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="first run one plain 256 MiB device copy (a known-traffic dispatch "
                          "for scaling rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE readings)")
@@ -394,6 +446,19 @@ def main():
                          "frac": round(kw["kernel_gbs"] / HBM_PEAK_GBS, 4),
                          "traffic": TRAFFIC_BYTES["kvwrite"]},
         })
+
+    if args.only in ("", "tokenstep"):
+        for (tb, tl) in ((16, 8192), (4, 1024)):
+            ts = bench_token_step(48, tb, tl, min(args.steps, 20), min(args.warmup, 3))
+            also.append({
+                "workload": f"single-token step over 48 layers: per layer the fused cache write of {tb} new "
+                            f"K/V rows x 4 heads + attention over {tb} seq x {tl} cached tokens, positions "
+                            "advanced on the device; 97 launches issued one by one vs one recorded graph",
+                "metric": "attention ms per token step", "value": round(ts["graph_ms"], 4), "unit": "ms",
+                "eager_ms": round(ts["eager_ms"], 4), "graph_ms": round(ts["graph_ms"], 4),
+                "steps": min(args.steps, 20),
+                "gbs": round(ts["bytes"] / (ts["graph_ms"] * 1e-3) / 1e9, 1),
+            })
 
     cpu = None
     if not args.skip_cpu and dec is not None:

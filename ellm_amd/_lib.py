@@ -72,6 +72,12 @@ ABI_SYMBOLS = {
     "ellm_kv_append": (ctypes.c_int, [_vp, _sz, _sz, _sz, _sz, _vp, _vp, _sz, _vp]),
     "ellm_kv_append_norm_rope": (ctypes.c_int, [_vp, _sz, _sz, _sz, _sz, _vp, _vp, _sz, _vp, _sz,
                                                 ctypes.c_float, _vp, _sz, _vp]),
+    "ellm_schedule_calls": (ctypes.c_int, [_sz, _sz, _sz, _sz, _vp, _sz, ctypes.POINTER(_sz)]),
+    "ellm_graph_begin": (ctypes.c_int, [_vp]),
+    "ellm_graph_end": (ctypes.c_int, [_vp, _pvp]),
+    "ellm_graph_launch": (ctypes.c_int, [_vp, _vp]),
+    "ellm_graph_destroy": (ctypes.c_int, [_vp]),
+    "ellm_positions_advance": (ctypes.c_int, [_vp, _sz, ctypes.c_uint32, _vp]),
 }
 
 _lib = None

@@ -159,7 +159,7 @@ int ellm_attn_create(const ellm_attn_desc* d, ellm_attn** out_handle) {
   if (e == hipSuccess) e = hipMalloc((void**)&h->counters, h->ws.counters * sizeof(uint32_t));
   if (e == hipSuccess) e = hipMemset(h->counters, 0, h->ws.counters * sizeof(uint32_t));
   if (e != hipSuccess) {
-    free_workspace(h);
+    (void)free_workspace(h);
     delete h;
     return fail_hip(e, "hipMalloc(workspace)");
   }
@@ -382,6 +382,93 @@ int ellm_kv_append_norm_rope(ellm_kv_cache* c, size_t layer, size_t position_ind
       (uint32_t)src_batch_pitch, (uint32_t)c->desc.kv_head_num, (uint32_t)c->desc.capacity,
       (uint32_t)position_index, (uint32_t)max_position, eps, c->desc.dtype, (hipStream_t)stream);
   if (e != hipSuccess) return fail_hip(e, "kv append (norm + rope) launch");
+  return ELLM_OK;
+}
+
+int ellm_schedule_calls(size_t prompt_begin, size_t prompt_end, size_t chunk, size_t generation_end,
+                        ellm_call* calls, size_t capacity, size_t* n_calls) {
+  if (!n_calls) return fail(ELLM_ERR_INVALID_ARGUMENT, "null n_calls");
+  if (chunk == 0) return fail(ELLM_ERR_INVALID_ARGUMENT, "chunk must be positive");
+  if (prompt_end < prompt_begin)
+    return fail(ELLM_ERR_INVALID_ARGUMENT, "prompt_end %zu before prompt_begin %zu", prompt_end,
+                prompt_begin);
+  if (capacity && !calls) return fail(ELLM_ERR_INVALID_ARGUMENT, "null calls");
+  size_t n = 0;
+  auto push = [&](size_t pos, size_t interval) {
+    if (n < capacity) calls[n] = ellm_call{pos, interval};
+    ++n;
+  };
+  const size_t prompt = prompt_end - prompt_begin;
+  if (prompt) {
+    const size_t full = (prompt - 1) / chunk;  // chunks before the last one
+    for (size_t i = 0; i < full; ++i) push(prompt_begin + i * chunk, chunk);
+    push(prompt_begin + full * chunk, prompt - full * chunk);
+  }
+  for (size_t pos = prompt_end; pos < generation_end; ++pos) push(pos, 1);
+  *n_calls = n;
+  if (n > capacity) return fail(ELLM_ERR_OUT_OF_RANGE, "%zu calls, room for %zu", n, capacity);
+  return ELLM_OK;
+}
+
+struct ellm_graph {
+  hipGraph_t graph;
+  hipGraphExec_t exec;
+};
+
+int ellm_graph_begin(void* stream) {
+  if (!stream) return fail(ELLM_ERR_INVALID_ARGUMENT, "the null stream cannot be recorded");
+  // relaxed mode: other host threads may keep calling into the runtime meanwhile
+  hipError_t e = hipStreamBeginCapture((hipStream_t)stream, hipStreamCaptureModeRelaxed);
+  if (e != hipSuccess) return fail_hip(e, "hipStreamBeginCapture");
+  return ELLM_OK;
+}
+
+int ellm_graph_end(void* stream, ellm_graph** out_graph) {
+  if (!stream || !out_graph) return fail(ELLM_ERR_INVALID_ARGUMENT, "null stream or output");
+  *out_graph = nullptr;
+  hipGraph_t g = nullptr;
+  hipError_t e = hipStreamEndCapture((hipStream_t)stream, &g);
+  if (e != hipSuccess) return fail_hip(e, "hipStreamEndCapture");
+  hipGraphExec_t x = nullptr;
+  e = hipGraphInstantiate(&x, g, nullptr, nullptr, 0);
+  if (e != hipSuccess) {
+    (void)hipGraphDestroy(g);
+    return fail_hip(e, "hipGraphInstantiate");
+  }
+  ellm_graph* h = new (std::nothrow) ellm_graph{g, x};
+  if (!h) {
+    (void)hipGraphExecDestroy(x);
+    (void)hipGraphDestroy(g);
+    return fail(ELLM_ERR_HIP, "out of host memory");
+  }
+  *out_graph = h;
+  return ELLM_OK;
+}
+
+int ellm_graph_launch(ellm_graph* graph, void* stream) {
+  if (!graph) return fail(ELLM_ERR_INVALID_ARGUMENT, "null graph");
+  hipError_t e = hipGraphLaunch(graph->exec, (hipStream_t)stream);
+  if (e != hipSuccess) return fail_hip(e, "hipGraphLaunch");
+  return ELLM_OK;
+}
+
+int ellm_graph_destroy(ellm_graph* graph) {
+  if (!graph) return ELLM_OK;
+  hipError_t e1 = hipGraphExecDestroy(graph->exec);
+  hipError_t e2 = hipGraphDestroy(graph->graph);
+  delete graph;
+  if (e1 != hipSuccess) return fail_hip(e1, "hipGraphExecDestroy");
+  if (e2 != hipSuccess) return fail_hip(e2, "hipGraphDestroy");
+  return ELLM_OK;
+}
+
+int ellm_positions_advance(uint32_t* positions, size_t batch_size, uint32_t by, void* stream) {
+  if (batch_size == 0) return ELLM_OK;
+  if (!positions) return fail(ELLM_ERR_INVALID_ARGUMENT, "null positions");
+  if (batch_size > 0xffffffffu) return fail(ELLM_ERR_UNSUPPORTED, "batch_size too large");
+  hipError_t e =
+      ellm::launch_positions_advance(positions, (uint32_t)batch_size, by, (hipStream_t)stream);
+  if (e != hipSuccess) return fail_hip(e, "positions advance launch");
   return ELLM_OK;
 }
 

@@ -78,4 +78,7 @@ hipError_t launch_kv_append_norm_rope(void* k_dst, void* v_dst, const void* k_sr
                                       uint32_t max_start, float eps, int dtype,
                                       hipStream_t stream);
 
+hipError_t launch_positions_advance(uint32_t* positions, uint32_t n, uint32_t by,
+                                    hipStream_t stream);
+
 }  // namespace ellm

@@ -108,7 +108,20 @@ __global__ __launch_bounds__(256) void kv_append_norm_rope_kernel(
   }
 }
 
+__global__ void positions_advance_kernel(uint32_t* positions, uint32_t n, uint32_t by) {
+  const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) positions[i] += by;
+}
+
 }  // namespace
+
+hipError_t launch_positions_advance(uint32_t* positions, uint32_t n, uint32_t by,
+                                    hipStream_t stream) {
+  if (n == 0) return hipSuccess;
+  hipLaunchKernelGGL(positions_advance_kernel, dim3((n + 255) / 256), dim3(256), 0, stream,
+                     positions, n, by);
+  return hipGetLastError();
+}
 
 hipError_t launch_kv_append_norm_rope(void* k_dst, void* v_dst, const void* k_src,
                                       const void* v_src, const void* rope,

@@ -195,6 +195,49 @@ int ellm_kv_append_norm_rope(ellm_kv_cache* cache, size_t layer, size_t position
                              size_t rope_positions, float eps, const uint32_t* positions,
                              size_t max_position, void* stream);
 
+/* ------------------------------------------------------------------------ *
+ * Position / chunk schedule and a recorded single-token step.
+ * ------------------------------------------------------------------------ */
+
+/* One run of every operator of the graph: positions
+ * [position_index, position_index + position_interval). */
+typedef struct ellm_call {
+  size_t position_index;
+  size_t position_interval;
+} ellm_call;
+
+/*
+ * The calls for one request: the prompt [prompt_begin, prompt_end) in chunks of
+ * `chunk` positions with a shorter last chunk, then one position at a time up
+ * to generation_end (exclusive).  Restates the loop of the reference's serving
+ * thread, src/serving/start copy.rs:71-113 (last chunk at
+ * prompt_end - (remainder ? remainder : chunk)), without its repetition of the
+ * last chunk.  Writes at most `capacity` calls; *n_calls receives the number
+ * the schedule has (ELLM_ERR_OUT_OF_RANGE when it exceeds capacity).
+ */
+int ellm_schedule_calls(size_t prompt_begin, size_t prompt_end, size_t chunk, size_t generation_end,
+                        ellm_call* calls, size_t capacity, size_t* n_calls);
+
+/*
+ * A recorded sequence of launches (a HIP graph), for the single-token loop in
+ * which the host would otherwise issue two launches per layer per token: the
+ * reference runs its operator queue once per token behind a spin barrier
+ * (src/serving/start.rs:59-77).  Between begin and end, calls of
+ * ellm_kv_append_norm_rope / ellm_kv_append / ellm_attn_run_ragged /
+ * ellm_positions_advance on `stream` are recorded instead of executed; the
+ * per-sequence positions live in device memory, so one recording serves every
+ * step.  `stream` must be a created stream, not the null stream.  A handle
+ * recorded into a graph must outlive it.
+ */
+typedef struct ellm_graph ellm_graph;
+int ellm_graph_begin(void* stream);
+int ellm_graph_end(void* stream, ellm_graph** out_graph);
+int ellm_graph_launch(ellm_graph* graph, void* stream);
+int ellm_graph_destroy(ellm_graph* graph);
+
+/* positions[i] += by for i < batch_size (device array), in stream order. */
+int ellm_positions_advance(uint32_t* positions, size_t batch_size, uint32_t by, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

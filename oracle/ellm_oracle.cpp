@@ -28,6 +28,11 @@
 //   oracle_attention_run_threads    src/serving/start.rs:59-77 (one thread per core,
 //                                   every thread calls run, then the barrier)
 //   oracle_scale_softmax            known answer held in src/kernel/test.rs:605-629
+//   oracle_schedule_calls           src/serving/start copy.rs:71-111 (the prompt in chunks of
+//                                   sequence_chunk_size, a shorter last chunk, then one token
+//                                   at a time); the prototype's loop runs the last chunk
+//                                   twice and underflows on an empty prompt, which is not
+//                                   followed
 //   oracle_rms_norm                 src/kernel/generic/rms_norm.rs:6-26 (weight 1; eps is
 //                                   added to the root mean square, not under the root)
 //   oracle_complex_mul              src/kernel/generic/complex_mul.rs:3-20 (interleaved
@@ -539,6 +544,36 @@ int ellm_oracle_kv_append_norm_rope(void* k_cache, void* v_cache, size_t kv_head
         std::memcpy(elem_ptr(v_cache, dst, dtype), elem_ptr(v_src, src, dtype), head_size * esz);
       }
   return 0;
+}
+
+// The (position_index, position_interval) pairs every operator of the graph is run with
+// for one request.  src/serving/start copy.rs:71-86 computes the last chunk as
+//   remainder = prompt_end % chunk;  last_interval = remainder ? remainder : chunk;
+//   last_position = prompt_end - last_interval
+// (stated there for prompt_begin = 0; lengths are taken from prompt_begin here), runs full
+// chunks before it (:89-95), the last chunk (:97-101), then single tokens (:102-113).
+// Returns the number of calls, or -1 when `capacity` pairs do not hold them.
+long ellm_oracle_schedule_calls(size_t prompt_begin, size_t prompt_end, size_t chunk,
+                                size_t generation_end, size_t* positions, size_t* intervals,
+                                size_t capacity) {
+  if (chunk == 0 || prompt_end < prompt_begin) return -1;
+  size_t n = 0;
+  auto push = [&](size_t pos, size_t interval) {
+    if (n < capacity) {
+      positions[n] = pos;
+      intervals[n] = interval;
+    }
+    ++n;
+  };
+  if (prompt_end > prompt_begin) {
+    const size_t remainder = (prompt_end - prompt_begin) % chunk;
+    const size_t last_interval = remainder ? remainder : chunk;
+    const size_t last_position = prompt_end - last_interval;
+    for (size_t pos = prompt_begin; pos < last_position; pos += chunk) push(pos, chunk);
+    push(last_position, last_interval);
+  }
+  for (size_t pos = prompt_end; pos < generation_end; ++pos) push(pos, 1);
+  return n <= capacity ? (long)n : -1;
 }
 
 // Storage conversions exposed so tests can check them against numpy.

@@ -72,6 +72,8 @@ def load():
     lib.ellm_oracle_bf16_to_f32.argtypes = [ctypes.c_uint16]
     lib.ellm_oracle_barrier_selftest.restype = ctypes.c_int
     lib.ellm_oracle_barrier_selftest.argtypes = [sz, sz]
+    lib.ellm_oracle_schedule_calls.restype = ctypes.c_long
+    lib.ellm_oracle_schedule_calls.argtypes = [sz, sz, sz, sz, vp, vp, sz]
     lib.ellm_oracle_rms_norm_f32.restype = None
     lib.ellm_oracle_rms_norm_f32.argtypes = [vp, vp, sz, f]
     lib.ellm_oracle_complex_mul_f32.restype = None
@@ -113,6 +115,19 @@ def from_storage(a, dtype):
 
 def storage_np_dtype(dtype):
     return {F16: np.float16, BF16: np.uint16, F32: np.float32}[dtype]
+
+
+def schedule_calls(prompt_begin, prompt_end, chunk, generation_end, capacity=None):
+    """The oracle's (position_index, position_interval) list, or None when it does not fit."""
+    if capacity is None:
+        capacity = max(prompt_end - prompt_begin, 0) + max(generation_end - prompt_end, 0) + 2
+    pos = np.zeros(max(capacity, 1), dtype=np.uintp)
+    itv = np.zeros(max(capacity, 1), dtype=np.uintp)
+    n = load().ellm_oracle_schedule_calls(prompt_begin, prompt_end, chunk, generation_end,
+                                          _ptr(pos), _ptr(itv), capacity)
+    if n < 0:
+        return None
+    return [(int(pos[i]), int(itv[i])) for i in range(n)]
 
 
 def rms_norm(x, eps):
