@@ -303,6 +303,58 @@ def bench_token_step(layers, batch, length, steps, warmup, hq=32, hkv=4):
     return {"eager_ms": eager_ms, "graph_ms": graph_ms, "bytes": nbytes}
 
 
+def bench_qkv_projection(tokens, steps, warmup, hidden=2048, hq=32, hkv=4, dtype_name="f16", batch=1):
+    """Fused Q/K/V projection of `tokens` token rows (x `batch` sequences): C = X . [Wq; Wk; Wv]^T
+    with RMS norm + rotary rotation of the query and key heads, query rows to the Q scratch,
+    key / value rows to their token coordinates of the cache."""
+    import torch
+
+    import ellm_amd
+
+    dt = torch.float16 if dtype_name == "f16" else torch.bfloat16
+    cap = tokens
+    x = _dev_normal((tokens, batch, hidden), dt, 71)
+    wq = _dev_normal((hq * D, hidden), dt, 72, scale=hidden ** -0.5)
+    wk = _dev_normal((hkv * D, hidden), dt, 73, scale=hidden ** -0.5)
+    wv = _dev_normal((hkv * D, hidden), dt, 74, scale=hidden ** -0.5)
+    j = torch.arange(D // 2, device="cuda", dtype=torch.float64)
+    ang = torch.arange(cap, device="cuda", dtype=torch.float64)[:, None] * (1.0e6 ** (-2.0 * j / D))[None, :]
+    rope = torch.stack((torch.cos(ang), torch.sin(ang)), dim=-1).reshape(cap, D).to(dt)
+    q = torch.zeros((tokens, batch, hq, D), dtype=dt, device="cuda")
+    cache = ellm_amd.KVCache(1, batch, hkv, cap,
+                             ellm_amd.DTYPE_F16 if dtype_name == "f16" else ellm_amd.DTYPE_BF16)
+    kt, vt = cache.layer_tensors(0, dt)
+    _, _, strides = cache.layer(0)
+    op = ellm_amd.MatMul3(x, wq, q, wk, kt, wv, vt, rope, D, batch, hq, hkv, strides, cap)
+    per, step_ms = _time_steps(lambda i: op.run(0, tokens, batch), steps, warmup)
+    flops = 2 * tokens * batch * hidden * (hq + 2 * hkv) * D
+    kern_ms = sum(per) / len(per)
+    op.close()
+    cache.close()
+    return {"flops": flops, "ms_per_step": step_ms, "kernel_ms": kern_ms,
+            "tflops": flops / (step_ms * 1e-3) / 1e12, "kernel_tflops": flops / (kern_ms * 1e-3) / 1e12}
+
+
+def bench_output_projection(tokens, steps, warmup, hidden=2048, hq=32, dtype_name="f16"):
+    """Output projection with residual: Y = R + A . Wo^T, A = the attention output rows."""
+    import torch
+
+    import ellm_amd
+
+    dt = torch.float16 if dtype_name == "f16" else torch.bfloat16
+    a = _dev_normal((tokens, 1, hq * D), dt, 81)
+    w = _dev_normal((hidden, hq * D), dt, 82, scale=(hq * D) ** -0.5)
+    r = _dev_normal((tokens, 1, hidden), dt, 83)
+    out = torch.zeros_like(r)
+    op = ellm_amd.MatMulAdd(a, w, r, out)
+    per, step_ms = _time_steps(lambda i: op.run(0, tokens, 1), steps, warmup)
+    flops = 2 * tokens * hidden * hq * D
+    kern_ms = sum(per) / len(per)
+    op.close()
+    return {"flops": flops, "ms_per_step": step_ms, "kernel_ms": kern_ms,
+            "tflops": flops / (step_ms * 1e-3) / 1e12, "kernel_tflops": flops / (kern_ms * 1e-3) / 1e12}
+
+
 def cpu_baseline_decode(batch, length, hq=32, hkv=4, budget_s=20.0):
     """The CPU oracle on the full single-token workload (all host cores)."""
     import numpy as np
@@ -336,7 +388,7 @@ def main():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--skip-cpu", action="store_true")
-    ap.add_argument("--only", default="", help="decode | prefill | decode128k | chunk | mixed | mixed48 | kvwrite | tokenstep")
+    ap.add_argument("--only", default="", help="decode | prefill | decode128k | chunk | mixed | mixed48 | kvwrite | tokenstep | qkv | oproj")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="first run one plain 256 MiB device copy (a known-traffic dispatch "
                          "for scaling rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE readings)")
@@ -459,6 +511,30 @@ def main():
                 "steps": min(args.steps, 20),
                 "gbs": round(ts["bytes"] / (ts["graph_ms"] * 1e-3) / 1e9, 1),
             })
+
+    if args.only in ("", "qkv"):
+        pj_steps = max(3, min(args.steps, 20))
+        pj = bench_qkv_projection(32768, pj_steps, min(args.warmup, 3))
+        also.append({
+            "workload": "fused Q/K/V projection: 32768 tokens x hidden 2048 -> 32q + 4k + 4v heads x 128, fp16, "
+                        "RMS norm + rotary rotation of Q and K heads, K/V written to the cache",
+            "metric": "projection TFLOP/s", "value": round(pj["tflops"], 2), "unit": "TFLOP/s",
+            "ms_per_step": round(pj["ms_per_step"], 4), "steps": pj_steps,
+            "roofline": {"bound": "mfma", "achieved": round(pj["kernel_tflops"], 2),
+                         "peak": MFMA_F16_PEAK_TFLOPS, "unit": "TFLOP/s",
+                         "frac": round(pj["kernel_tflops"] / MFMA_F16_PEAK_TFLOPS, 4), "traffic": None},
+        })
+    if args.only in ("", "oproj"):
+        pj_steps = max(3, min(args.steps, 20))
+        po = bench_output_projection(32768, pj_steps, min(args.warmup, 3))
+        also.append({
+            "workload": "output projection + residual: 32768 tokens x 4096 -> 2048, fp16",
+            "metric": "projection TFLOP/s", "value": round(po["tflops"], 2), "unit": "TFLOP/s",
+            "ms_per_step": round(po["ms_per_step"], 4), "steps": pj_steps,
+            "roofline": {"bound": "mfma", "achieved": round(po["kernel_tflops"], 2),
+                         "peak": MFMA_F16_PEAK_TFLOPS, "unit": "TFLOP/s",
+                         "frac": round(po["kernel_tflops"] / MFMA_F16_PEAK_TFLOPS, 4), "traffic": None},
+        })
 
     cpu = None
     if not args.skip_cpu and dec is not None:

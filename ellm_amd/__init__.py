@@ -16,4 +16,5 @@ from ._lib import (  # noqa: F401
     load_library,
 )
 from .attention import Attention, KVCache  # noqa: F401
+from .projection import MatMul3, MatMulAdd  # noqa: F401
 from .schedule import StepGraph, positions_advance, schedule_calls  # noqa: F401

@@ -53,6 +53,46 @@ class KvDesc(ctypes.Structure):
     ]
 
 
+class MatMul3Desc(ctypes.Structure):
+    _fields_ = [
+        ("hidden", ctypes.c_void_p),
+        ("q_weight", ctypes.c_void_p),
+        ("k_weight", ctypes.c_void_p),
+        ("v_weight", ctypes.c_void_p),
+        ("q_state", ctypes.c_void_p),
+        ("k_state", ctypes.c_void_p),
+        ("v_state", ctypes.c_void_p),
+        ("rope", ctypes.c_void_p),
+        ("rope_position_stride", ctypes.c_size_t),
+        ("rope_head_stride", ctypes.c_size_t),
+        ("rope_elems", ctypes.c_size_t),
+        ("hidden_size", ctypes.c_size_t),
+        ("batch_size", ctypes.c_size_t),
+        ("attention_head_num", ctypes.c_size_t),
+        ("kv_head_num", ctypes.c_size_t),
+        ("head_size", ctypes.c_size_t),
+        ("kv_strides", ctypes.c_size_t * 4),
+        ("sequence_capacity", ctypes.c_size_t),
+        ("max_position_interval", ctypes.c_size_t),
+        ("eps", ctypes.c_float),
+        ("dtype", ctypes.c_int),
+    ]
+
+
+class MatMulAddDesc(ctypes.Structure):
+    _fields_ = [
+        ("a", ctypes.c_void_p),
+        ("b_nt", ctypes.c_void_p),
+        ("residual", ctypes.c_void_p),
+        ("output", ctypes.c_void_p),
+        ("batch_size", ctypes.c_size_t),
+        ("n", ctypes.c_size_t),
+        ("k", ctypes.c_size_t),
+        ("max_position_interval", ctypes.c_size_t),
+        ("dtype", ctypes.c_int),
+    ]
+
+
 _sz = ctypes.c_size_t
 _vp = ctypes.c_void_p
 _pvp = ctypes.POINTER(ctypes.c_void_p)
@@ -78,6 +118,13 @@ ABI_SYMBOLS = {
     "ellm_graph_launch": (ctypes.c_int, [_vp, _vp]),
     "ellm_graph_destroy": (ctypes.c_int, [_vp]),
     "ellm_positions_advance": (ctypes.c_int, [_vp, _sz, ctypes.c_uint32, _vp]),
+    "ellm_matmul3_create": (ctypes.c_int, [ctypes.POINTER(MatMul3Desc), _pvp]),
+    "ellm_matmul3_run": (ctypes.c_int, [_vp, _sz, _sz, _sz, _vp]),
+    "ellm_matmul3_run_ragged": (ctypes.c_int, [_vp, _vp, _sz, _sz, _vp]),
+    "ellm_matmul3_destroy": (ctypes.c_int, [_vp]),
+    "ellm_matmul_add_create": (ctypes.c_int, [ctypes.POINTER(MatMulAddDesc), _pvp]),
+    "ellm_matmul_add_run": (ctypes.c_int, [_vp, _sz, _sz, _sz, _vp]),
+    "ellm_matmul_add_destroy": (ctypes.c_int, [_vp]),
 }
 
 _lib = None

@@ -81,4 +81,33 @@ hipError_t launch_kv_append_norm_rope(void* k_dst, void* v_dst, const void* k_sr
 hipError_t launch_positions_advance(uint32_t* positions, uint32_t n, uint32_t by,
                                     hipStream_t stream);
 
+// Projection C = X . W^T on MFMA with the per-head epilogue (see project.hip).
+// Column segment 0 (heads0 heads, weights w0) goes row-major to out0 [rows][heads0 * 128],
+// optionally normalised + rotated (finalize0) and with `residual` added; segments 1 and 2
+// (heads_kv heads each, weights wk / wv) go to token coordinates of k_out / v_out through
+// the three strides, the key rows normalised + rotated.  Row r of X is token r / batch_pitch
+// of sequence r % batch_pitch; sequences >= batch are skipped.
+struct ProjectArgs {
+  const void* x;
+  const void* w0;
+  const void* wk;
+  const void* wv;
+  void* out0;
+  const void* residual;
+  void* k_out;
+  void* v_out;
+  const void* rope;
+  const uint32_t* positions;
+  size_t kv_stride_seq, kv_stride_head, kv_stride_pos;
+  uint32_t rope_pos_stride, rope_head_stride;
+  uint32_t K, rows, batch_pitch, batch, heads0, heads_kv;
+  uint32_t position_index, max_start, finalize0;
+  float eps;
+  int dtype;
+};
+hipError_t launch_project(const ProjectArgs& a, hipStream_t stream);
+
+// Records the message ellm_last_error_string() returns on this thread; returns status.
+int set_error(int status, const char* fmt, ...) __attribute__((format(printf, 2, 3)));
+
 }  // namespace ellm

@@ -1,0 +1,399 @@
+// Projections around the attention operator on gfx950 MFMA:
+//   fused Q/K/V projection   C = X . [Wq; Wk; Wv]^T  with, per finished 128-wide head
+//   row, RMS norm (weight 1) and rotary rotation for the query and key heads, the
+//   query rows written to the Q scratch, key and value rows written straight to their
+//   token coordinates of the cache; replaces MatMul3::run (reference:
+//   src/compiler/mul/matmul3.rs:289-385, finalize :243-254 and :436-451);
+//   output projection + residual   Y = A . Wo^T + R; replaces MatMulAdd::run
+//   (src/compiler/mul/matmul_add.rs:128-232).
+// Weights are row-major [N][K] as the reference keeps them ("W_nt"), activations are
+// row-major [rows][K]; both operands are K-contiguous, which is what MFMA wants.
+//
+// Formulation: the product is computed transposed, C^T[n][token] = W . X^T, so that a
+// lane of the 32x32 accumulator block owns one token and 16 of 32 output columns: a
+// head row (128 columns) of a token then sits in two lanes (l and l ^ 32), the sum of
+// squares needs one cross-lane exchange and the (even, odd) rotation pairs are
+// register neighbours.
+//
+// A workgroup of 4 waves (one per SIMD, 512 registers each) owns a tile of 256 tokens x
+// 256 output columns (two heads); wave (wn, wm) owns head wn and tokens 128 wm..+127 as
+// 4 x 4 accumulator blocks (256 accumulator registers).  K runs in chunks of 32
+// through a three-stage LDS ring: chunk c is read while chunk c+2 is written, chunk
+// c+1 is already complete, so the first operands of the next chunk are requested
+// before the barrier that ends the current one and the MFMA stream never drains.
+#include <type_traits>
+
+#include "common.hpp"
+#include "kernels.hpp"
+
+namespace ellm {
+namespace {
+
+constexpr int kTile = 256;                          // tokens, and output columns, per workgroup
+constexpr int kKc = 32;                             // K elements per chunk
+constexpr int kRowPitch = (kKc + 8) * 2;            // 80 B: 16 consecutive rows' 16-byte pieces tile all 64 banks
+constexpr int kStageBytes = 2 * kTile * kRowPitch;  // X rows then W rows
+constexpr int kStages = 3;
+constexpr int kEpPitch = kHeadDim * 2 + 16;         // output row in LDS
+constexpr int kEpWaveBytes = 32 * kEpPitch + 32 * 8;  // 32 rows and their destinations, per wave
+constexpr int kProjThreads = 256;
+constexpr int kProjLdsBytes = kStages * kStageBytes;
+static_assert(4 * kEpWaveBytes <= kProjLdsBytes, "the epilogue reuses the stages");
+constexpr int kGroupM = 4;                          // token tiles that take turns on one column tile
+constexpr int kBufFlags = 0x00020000;               // raw buffer of 32-bit data, no swizzle
+
+typedef __attribute__((address_space(3))) u32x4 LdsVec4;
+typedef __attribute__((address_space(3))) u32x2 LdsVec2;
+typedef __attribute__((address_space(3))) uint64_t LdsU64;
+
+struct ProjectKernelArgs {
+  const uint16_t* x;         // [rows][K]
+  const uint16_t* w[3];      // column segments 0 (query / plain), 1 (key), 2 (value): [heads * 128][K]
+  uint16_t* out0;            // segment 0 destination, row-major [rows][ld0]
+  const uint16_t* residual;  // added to segment 0 (same layout), may be null
+  uint16_t* k_out;
+  uint16_t* v_out;
+  const uint16_t* rope;
+  const uint32_t* positions;
+  size_t kv_stride_seq, kv_stride_head, kv_stride_pos;  // elements
+  uint32_t ld0;
+  uint32_t rope_pos_stride, rope_head_stride;           // elements
+  uint32_t K, rows, batch_pitch, batch;
+  uint32_t heads0, heads_kv;
+  uint32_t tiles_m, tiles_n;
+  uint32_t position_index, max_start;
+  uint32_t finalize0;        // segment 0 rows are normalised and rotated
+  float eps;
+};
+
+template <int N, typename F>
+__device__ __forceinline__ void static_for(F&& f) {
+  if constexpr (N > 0) {
+    static_for<N - 1>(f);
+    f(std::integral_constant<int, N - 1>{});
+  }
+}
+
+__device__ __forceinline__ uint64_t uniform64(const void* p) {
+  const uint32_t lo = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(uint64_t)p);
+  const uint32_t hi = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)((uint64_t)p >> 32));
+  return ((uint64_t)hi << 32) | (uint64_t)lo;
+}
+
+constexpr int kModeQkv = 0;  // heads normalised + rotated (or passed through), K/V to token coordinates
+constexpr int kModeAdd = 1;  // plain product plus a residual of the output's layout
+
+template <typename S, int MODE>
+__global__ __launch_bounds__(kProjThreads) void project_kernel(ProjectKernelArgs p) {
+  using M = Mfma<S>;
+  extern __shared__ __attribute__((aligned(16))) uint8_t proj_smem[];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int j = lane & 31, g = lane >> 5;
+  const int wn = wave & 1, wm = wave >> 1;
+
+  // workgroup -> tile: ids that share id % 8 (one XCD, one L2) are made consecutive,
+  // then kGroupM token tiles x all column tiles form a band that is walked token-first
+  uint32_t tm, tn;
+  {
+    const uint32_t total = p.tiles_m * p.tiles_n;
+    const uint32_t q = total >> 3, r = total & 7, xcd = blockIdx.x & 7, idx = blockIdx.x >> 3;
+    const uint32_t pid = xcd * q + min(xcd, r) + idx;
+    const uint32_t per_band = kGroupM * p.tiles_n;
+    const uint32_t band = pid / per_band, in_band = pid % per_band;
+    const uint32_t first_m = band * kGroupM;
+    const uint32_t band_m = min(p.tiles_m - first_m, (uint32_t)kGroupM);
+    tm = first_m + in_band % band_m;
+    tn = in_band / band_m;
+  }
+  const uint32_t heads_total = p.heads0 + 2 * p.heads_kv;
+  const uint32_t K = p.K;
+  const uint32_t n_chunks = K / kKc;
+
+  // operand sources: one descriptor for the token rows, one per head of the tile
+  const uint32_t row0 = tm * kTile;
+  const uint32_t rows_here = min(p.rows - row0, (uint32_t)kTile);
+  const __amdgpu_buffer_rsrc_t x_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+      (void*)(uniform64(p.x) + (uint64_t)row0 * K * 2), 0, rows_here * K * 2, kBufFlags);
+  auto head_rsrc = [&](uint32_t hh) {
+    const uint16_t* base = p.w[0];
+    uint32_t hs = hh, bytes = kHeadDim * K * 2;
+    if (hh >= p.heads0 + p.heads_kv) {
+      base = p.w[2];
+      hs = hh - p.heads0 - p.heads_kv;
+    } else if (hh >= p.heads0) {
+      base = p.w[1];
+      hs = hh - p.heads0;
+    }
+    if (hh >= heads_total) {  // odd head count: the tile's second half reads zeros
+      base = p.w[0];
+      hs = 0;
+      bytes = 0;
+    }
+    return __builtin_amdgcn_make_buffer_rsrc((void*)(uniform64(base) + (uint64_t)hs * kHeadDim * K * 2),
+                                             0, bytes, kBufFlags);
+  };
+  const __amdgpu_buffer_rsrc_t w_rsrc0 = head_rsrc(2 * tn), w_rsrc1 = head_rsrc(2 * tn + 1);
+
+  // staging: thread -> row tid / 4 (+ 64 i), 16-byte piece tid % 4 of the chunk's 64 B
+  const uint32_t st_row = tid >> 2, st_piece = tid & 3;
+  uint32_t src_off[4];  // rows st_row + 64 i of a 256-row (X) or, i & 1, 128-row (W head) source
+#pragma unroll
+  for (int i = 0; i < 4; ++i) src_off[i] = (st_row + 64 * i) * K * 2 + st_piece * 16;
+  const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t*)proj_smem;
+  auto pin = [](uint32_t addr) {
+    asm volatile("" : "+v"(addr));
+    return addr;
+  };
+  const uint32_t st_store = lds0 + st_row * kRowPitch + st_piece * 16;
+  // Two sets of staging registers: a chunk is requested two iterations (about 1.2 us)
+  // before it is stored to LDS, which is what a fetch from HBM can take under load.
+  u32x4 stg[2][8];
+  // (a chunk past the last one fetches bytes of the next row, or zeros past the end of
+  // the buffer, into a stage nobody reads)
+  auto load_piece = [&](auto set, uint32_t chunk, int i) {
+    const uint32_t soff = chunk * (kKc * 2);
+    if (i < 4)
+      stg[set][i] = __builtin_amdgcn_raw_buffer_load_b128(x_rsrc, src_off[i], soff, 0);
+    else
+      stg[set][i] = __builtin_amdgcn_raw_buffer_load_b128((i < 6) ? w_rsrc0 : w_rsrc1, src_off[i & 1], soff, 0);
+  };
+  auto store_piece = [&](auto set, uint32_t base, int i) {
+    *(LdsVec4*)(base + 64 * i * kRowPitch) = stg[set][i];
+  };
+
+  f32x16 acc[4][4];  // [column block nb][token block mb]
+#pragma unroll
+  for (int nb = 0; nb < 4; ++nb)
+#pragma unroll
+    for (int mb = 0; mb < 4; ++mb)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[nb][mb][r] = 0.0f;
+
+  // operand reads: lane (j, g) takes row j of a 32-row block, K piece g of the 16-wide step
+  const uint32_t x_read = lds0 + (wm * 128 + j) * kRowPitch + g * 16;
+  const uint32_t w_read = lds0 + (kTile + wn * 128 + j) * kRowPitch + g * 16;
+  // operand o of a step: 0..3 = W blocks, 4..7 = X blocks
+  auto read_operand = [&](uint32_t xb, uint32_t wb, int step, int o) {
+    const uint32_t at = (o < 4 ? wb + 32 * o * kRowPitch : xb + 32 * (o - 4) * kRowPitch) + 32 * step;
+    return (u32x4) * (const LdsVec4*)at;
+  };
+
+  // prologue: chunks 0 and 1 into stages 0 and 1, chunks 2 and 3 into the staging registers
+  constexpr std::integral_constant<int, 0> kSet0{};
+  constexpr std::integral_constant<int, 1> kSet1{};
+#pragma unroll
+  for (int i = 0; i < 8; ++i) load_piece(kSet0, 0, i);
+#pragma unroll
+  for (int i = 0; i < 8; ++i) load_piece(kSet1, 1, i);
+  {
+    const uint32_t base = pin(st_store);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) store_piece(kSet0, base, i);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) load_piece(kSet0, 2, i);
+    const uint32_t base1 = pin(st_store + kStageBytes);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) store_piece(kSet1, base1, i);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) load_piece(kSet1, 3, i);
+  }
+  __syncthreads();
+
+  u32x4 opa[8], opb[8];
+  {
+    const uint32_t xb = pin(x_read), wb = pin(w_read);
+#pragma unroll
+    for (int o = 0; o < 8; ++o) opa[o] = read_operand(xb, wb, 0, o);
+  }
+
+  // One iteration = one chunk (two 16-wide steps, 32 MFMAs).  Chunk c sits in stage
+  // c % 3; during it the staging set c % 2 (chunk c + 2) is stored to stage (c + 2) % 3
+  // and refilled with chunk c + 4.
+  uint32_t stage = 0;
+  auto iteration = [&](auto set, uint32_t c) __attribute__((always_inline)) {
+    const uint32_t stage1 = (stage == 2) ? 0 : stage + 1;   // chunk c + 1
+    const uint32_t stage2 = (stage1 == 2) ? 0 : stage1 + 1;  // chunk c + 2 goes here
+    const uint32_t xb = pin(x_read + stage * kStageBytes), wb = pin(w_read + stage * kStageBytes);
+    const uint32_t xb1 = pin(x_read + stage1 * kStageBytes), wb1 = pin(w_read + stage1 * kStageBytes);
+    const uint32_t store_at = pin(st_store + stage2 * kStageBytes);
+    __builtin_amdgcn_sched_barrier(0);
+    // step 0: operands opa, fetch step 1 into opb
+    static_for<16>([&](auto n_) {
+      constexpr int n = decltype(n_)::value;
+      acc[n >> 2][n & 3] = M::m32x32x16(opa[n >> 2], opa[4 + (n & 3)], acc[n >> 2][n & 3]);
+      if constexpr (n < 8) opb[n] = read_operand(xb, wb, 1, n);
+      __builtin_amdgcn_sched_barrier(0);
+    });
+    // step 1: operands opb, fetch step 0 of chunk c + 1 into opa; staging
+    static_for<16>([&](auto n_) {
+      constexpr int n = decltype(n_)::value;
+      acc[n >> 2][n & 3] = M::m32x32x16(opb[n >> 2], opb[4 + (n & 3)], acc[n >> 2][n & 3]);
+      if constexpr (n < 8) opa[n] = read_operand(xb1, wb1, 0, n);
+      if constexpr (n >= 8) {
+        store_piece(set, store_at, n - 8);
+        load_piece(set, c + 4, n - 8);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    });
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+    __builtin_amdgcn_s_barrier();
+    stage = stage1;
+  };
+  for (uint32_t c = 0; c < n_chunks; c += 2) {  // K is a multiple of 64: chunks come in pairs
+    iteration(kSet0, c);
+    iteration(kSet1, c + 1);
+  }
+  // (the reads into opa after the last chunk fetched a stage nobody wrote: discarded)
+
+  // ---- epilogue: per wave one head x 128 tokens ------------------------------------
+  const uint32_t hh = 2 * tn + wn;
+  if (hh >= heads_total) return;
+  const uint32_t seg = (hh < p.heads0) ? 0u : (hh < p.heads0 + p.heads_kv ? 1u : 2u);
+  const uint32_t hs = hh - (seg == 0 ? 0u : (seg == 1 ? p.heads0 : p.heads0 + p.heads_kv));
+  const bool finalize = MODE == kModeQkv && ((seg == 1) || (seg == 0 && p.finalize0));
+  uint16_t* const dst = (seg == 0) ? p.out0 : (seg == 1 ? p.k_out : p.v_out);
+  // In the accumulator layout lane (j, g) holds, for token 32 mb + j, the
+  // columns 32 nb + 8 b + 4 g + (0..3) of the head: four consecutive columns = two rotation
+  // pairs = one 8-byte piece of the rotary row, of the residual row and of the output
+  // row; lanes l and l ^ 32 together own the token's 128 columns.  The extra operand
+  // (table or residual) of token block mb + 1 is requested before block mb is worked on.
+  // One code path: a head that is not normalised and rotated runs the same arithmetic
+  // with scale 1 and the rotation (cos, sin) = (1, 0), which leaves every value as it is.
+  uint16_t* out_row[4];
+  const uint16_t* ext_row[4];
+  bool live[4];
+#pragma unroll
+  for (int mb = 0; mb < 4; ++mb) {
+    const uint32_t R = row0 + wm * 128 + 32 * mb + j;
+    const uint32_t t = R / p.batch_pitch, b = R % p.batch_pitch;
+    live[mb] = R < p.rows && b < p.batch;
+    uint32_t pos = t;
+    if (p.positions)
+      pos += live[mb] ? min(p.positions[b], p.max_start) : 0u;
+    else
+      pos += p.position_index;
+    const size_t col = hs * kHeadDim;
+    if (seg == 0)
+      out_row[mb] = dst + (size_t)R * p.ld0 + col;
+    else
+      out_row[mb] = dst + (size_t)b * p.kv_stride_seq + (size_t)hs * p.kv_stride_head +
+                    (size_t)pos * p.kv_stride_pos;
+    if (MODE == kModeQkv)
+      ext_row[mb] = p.rope + (size_t)pos * p.rope_pos_stride + (size_t)hs * p.rope_head_stride + 4 * g;
+    else
+      ext_row[mb] = p.residual + (size_t)R * p.ld0 + col + 4 * g;
+  }
+  const uint32_t ep_rows = lds0 + wave * kEpWaveBytes, ep_table = ep_rows + 32 * kEpPitch;
+  const uint32_t one_zero = M::pack2(1.0f, 0.0f);
+  u32x2 ext[2][16];
+  auto fetch_ext = [&](auto set, int mb) {
+    if ((MODE == kModeAdd || finalize) && live[mb]) {
+#pragma unroll
+      for (int i = 0; i < 16; ++i) ext[set][i] = *(const u32x2*)(ext_row[mb] + 32 * (i >> 2) + 8 * (i & 3));
+    } else {
+#pragma unroll
+      for (int i = 0; i < 16; ++i) ext[set][i] = u32x2{one_zero, one_zero};
+    }
+  };
+  fetch_ext(kSet0, 0);
+  static_for<4>([&](auto mb_) {
+    constexpr int mb = decltype(mb_)::value;
+    constexpr int set = mb & 1;
+    __builtin_amdgcn_sched_barrier(0);  // one token block's accumulators at a time leave the AGPRs
+    if constexpr (mb + 1 < 4) fetch_ext(std::integral_constant<int, 1 - set>{}, mb + 1);
+    float inv = 1.0f;
+    if (MODE == kModeQkv) {
+      float ss = 0.0f;
+#pragma unroll
+      for (int nb = 0; nb < 4; ++nb)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) ss = fmaf(acc[nb][mb][r], acc[nb][mb][r], ss);
+      ss = sum_with_partner_half(ss);
+      inv = finalize ? 1.0f / (sqrtf(ss / (float)kHeadDim) + p.eps) : 1.0f;
+    }
+    u32x2 packed[16];
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      const int nb = i >> 2, b4 = i & 3;
+      float o0 = acc[nb][mb][4 * b4], o1 = acc[nb][mb][4 * b4 + 1];
+      float o2 = acc[nb][mb][4 * b4 + 2], o3 = acc[nb][mb][4 * b4 + 3];
+      const u32x2 rr = ext[set][i];
+      const float e0 = M::to_float((uint16_t)(rr[0] & 0xffffu)), e1 = M::to_float((uint16_t)(rr[0] >> 16));
+      const float e2 = M::to_float((uint16_t)(rr[1] & 0xffffu)), e3 = M::to_float((uint16_t)(rr[1] >> 16));
+      if (MODE == kModeQkv) {
+        const float y0 = o0 * inv, y1 = o1 * inv, y2 = o2 * inv, y3 = o3 * inv;
+        o0 = y0 * e0 - y1 * e1;
+        o1 = y0 * e1 + y1 * e0;
+        o2 = y2 * e2 - y3 * e3;
+        o3 = y2 * e3 + y3 * e2;
+      } else {
+        o0 += e0;
+        o1 += e1;
+        o2 += e2;
+        o3 += e3;
+      }
+      packed[i] = u32x2{M::pack2(o0, o1), M::pack2(o2, o3)};
+    }
+    // out through LDS so that a store instruction covers whole 256-byte rows: the lane
+    // that owns token j also leaves the row's destination (0: nothing to write)
+    if (g == 0) *(LdsU64*)(ep_table + 8 * j) = live[mb] ? (uint64_t)out_row[mb] : 0ull;
+#pragma unroll
+    for (int i = 0; i < 16; ++i)
+      *(LdsVec2*)(ep_rows + j * kEpPitch + 2 * (32 * (i >> 2) + 8 * (i & 3) + 4 * g)) = packed[i];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const uint32_t row = 4 * i + (lane >> 4);
+      uint16_t* const to = (uint16_t*)*(const LdsU64*)(ep_table + 8 * row);
+      const u32x4 v = *(const LdsVec4*)(ep_rows + row * kEpPitch + 16 * (lane & 15));
+      if (to) store16(to + 8 * (lane & 15), v);
+    }
+  });
+}
+
+}  // namespace
+
+hipError_t launch_project(const ProjectArgs& a, hipStream_t stream) {
+  if (a.rows == 0) return hipSuccess;
+  ProjectKernelArgs p;
+  p.x = (const uint16_t*)a.x;
+  p.w[0] = (const uint16_t*)a.w0;
+  p.w[1] = (const uint16_t*)a.wk;
+  p.w[2] = (const uint16_t*)a.wv;
+  p.out0 = (uint16_t*)a.out0;
+  p.residual = (const uint16_t*)a.residual;
+  p.k_out = (uint16_t*)a.k_out;
+  p.v_out = (uint16_t*)a.v_out;
+  p.rope = (const uint16_t*)a.rope;
+  p.positions = a.positions;
+  p.kv_stride_seq = a.kv_stride_seq;
+  p.kv_stride_head = a.kv_stride_head;
+  p.kv_stride_pos = a.kv_stride_pos;
+  p.ld0 = a.heads0 * kHeadDim;
+  p.rope_pos_stride = a.rope_pos_stride;
+  p.rope_head_stride = a.rope_head_stride;
+  p.K = a.K;
+  p.rows = a.rows;
+  p.batch_pitch = a.batch_pitch;
+  p.batch = a.batch;
+  p.heads0 = a.heads0;
+  p.heads_kv = a.heads_kv;
+  p.tiles_m = (a.rows + kTile - 1) / kTile;
+  p.tiles_n = (a.heads0 + 2 * a.heads_kv + 1) / 2;
+  p.position_index = a.position_index;
+  p.max_start = a.max_start;
+  p.finalize0 = a.finalize0;
+  p.eps = a.eps;
+  const uint32_t blocks = p.tiles_m * p.tiles_n;
+  auto go = [&](auto kernel) {
+    hipError_t e = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                       kProjLdsBytes);
+    if (e != hipSuccess) return e;
+    hipLaunchKernelGGL(kernel, dim3(blocks), dim3(kProjThreads), kProjLdsBytes, stream, p);
+    return hipGetLastError();
+  };
+  if (a.residual)
+    return a.dtype == 0 ? go(project_kernel<F16, kModeAdd>) : go(project_kernel<BF16, kModeAdd>);
+  return a.dtype == 0 ? go(project_kernel<F16, kModeQkv>) : go(project_kernel<BF16, kModeQkv>);
+}
+
+}  // namespace ellm

@@ -1,0 +1,120 @@
+"""Host-side mirrors of the reference's projection operators either side of attention:
+``MatMul3`` (fused Q/K/V projection with RMS norm + rotary rotation of the query and
+key heads, src/compiler/mul/matmul3.rs) and ``MatMulAdd`` (output projection plus
+residual, src/compiler/mul/matmul_add.rs).  torch tensors are device buffers only."""
+import ctypes
+
+from ._lib import MatMul3Desc, MatMulAddDesc, check, load_library
+from .attention import _dtype_code, _stream_ptr
+
+
+class MatMul3:
+    """MatMul3::new / run over device buffers.
+
+    hidden:  [max_position_interval, batch_capacity, hidden_size]
+    weights: [heads * 128, hidden_size] (row-major N x K, as the reference keeps them)
+    q_state: [max_position_interval, batch_capacity, attention_head_num, 128]
+    k_state, v_state: any buffers addressed by kv_strides = (sequence, kv head, position, 1)
+    rope: (cos, sin) interleaved; row of head h at position p starts at
+          p * rope_position_stride + h * rope_head_stride elements
+    """
+
+    def __init__(self, hidden, q_weight, q_state, k_weight, k_state, v_weight, v_state, rope,
+                 head_dim, batch_size, attention_head_num, kv_head_num, kv_strides,
+                 sequence_capacity, rope_position_stride=128, rope_head_stride=0, eps=1e-6,
+                 max_position_interval=None):
+        self._lib = load_library()
+        self._keep = (hidden, q_weight, q_state, k_weight, k_state, v_weight, v_state, rope)
+        d = MatMul3Desc()
+        d.hidden, d.q_weight, d.k_weight, d.v_weight = (hidden.data_ptr(), q_weight.data_ptr(),
+                                                        k_weight.data_ptr(), v_weight.data_ptr())
+        d.q_state, d.k_state, d.v_state = q_state.data_ptr(), k_state.data_ptr(), v_state.data_ptr()
+        d.rope = rope.data_ptr()
+        d.rope_position_stride, d.rope_head_stride = int(rope_position_stride), int(rope_head_stride)
+        d.rope_elems = rope.numel()
+        d.hidden_size = hidden.shape[-1]
+        d.batch_size = batch_size
+        d.attention_head_num, d.kv_head_num, d.head_size = attention_head_num, kv_head_num, head_dim
+        for i in range(4):
+            d.kv_strides[i] = int(kv_strides[i])
+        d.sequence_capacity = int(sequence_capacity)
+        d.max_position_interval = int(
+            max_position_interval if max_position_interval is not None else hidden.shape[0])
+        d.eps = float(eps)
+        d.dtype = _dtype_code(hidden)
+        self.desc = d
+        self._handle = ctypes.c_void_p()
+        check(self._lib.ellm_matmul3_create(ctypes.byref(d), ctypes.byref(self._handle)))
+
+    @classmethod
+    def new(cls, *args, **kwargs):
+        return cls(*args, **kwargs)
+
+    def run(self, position_index, position_interval, batch_size, cpu_num=1, thread_id=0,
+            stream=None):
+        if thread_id != 0:
+            return
+        check(self._lib.ellm_matmul3_run(self._handle, position_index, position_interval,
+                                         batch_size, _stream_ptr(stream)))
+
+    def run_ragged(self, positions, max_position, batch_size, stream=None):
+        check(self._lib.ellm_matmul3_run_ragged(self._handle, ctypes.c_void_p(positions.data_ptr()),
+                                                int(max_position), batch_size, _stream_ptr(stream)))
+
+    def close(self):
+        if self._handle:
+            check(self._lib.ellm_matmul3_destroy(self._handle))
+            self._handle = ctypes.c_void_p()
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+
+class MatMulAdd:
+    """MatMulAdd::new / run: output = residual + a . b_nt^T.
+
+    a: [max_position_interval, batch_capacity, k]; b_nt: [n, k];
+    residual, output: [max_position_interval, batch_capacity, n]
+    """
+
+    def __init__(self, a, b_nt, residual, output, m_max=None, n_max=None, k_max=None,
+                 max_position_interval=None):
+        self._lib = load_library()
+        self._keep = (a, b_nt, residual, output)
+        d = MatMulAddDesc()
+        d.a, d.b_nt, d.residual, d.output = (a.data_ptr(), b_nt.data_ptr(), residual.data_ptr(),
+                                             output.data_ptr())
+        d.batch_size = int(m_max if m_max is not None else a.shape[1])
+        d.n = int(n_max if n_max is not None else b_nt.shape[0])
+        d.k = int(k_max if k_max is not None else b_nt.shape[1])
+        d.max_position_interval = int(
+            max_position_interval if max_position_interval is not None else a.shape[0])
+        d.dtype = _dtype_code(a)
+        self.desc = d
+        self._handle = ctypes.c_void_p()
+        check(self._lib.ellm_matmul_add_create(ctypes.byref(d), ctypes.byref(self._handle)))
+
+    @classmethod
+    def new(cls, *args, **kwargs):
+        return cls(*args, **kwargs)
+
+    def run(self, position_index, position_interval, batch_size, cpu_num=1, thread_id=0,
+            stream=None):
+        if thread_id != 0:
+            return
+        check(self._lib.ellm_matmul_add_run(self._handle, position_index, position_interval,
+                                            batch_size, _stream_ptr(stream)))
+
+    def close(self):
+        if self._handle:
+            check(self._lib.ellm_matmul_add_destroy(self._handle))
+            self._handle = ctypes.c_void_p()
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass

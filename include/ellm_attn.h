@@ -238,6 +238,98 @@ int ellm_graph_destroy(ellm_graph* graph);
 /* positions[i] += by for i < batch_size (device array), in stream order. */
 int ellm_positions_advance(uint32_t* positions, size_t batch_size, uint32_t by, void* stream);
 
+/* ------------------------------------------------------------------------ *
+ * Projections either side of the attention operator.
+ * ------------------------------------------------------------------------ */
+
+/*
+ * Fused Q/K/V projection: replaces MatMul3::new / run
+ * (src/compiler/mul/matmul3.rs:63-120, 289-385; built by Tensor::matmul3,
+ * src/ptensor/tensor.rs:439-498; used by src/qwen3_moe/attention.rs:121-136).
+ *     [Cq | Ck | Cv] = hidden . [Wq; Wk; Wv]^T          (binary32 accumulation)
+ * Weights are row-major [N][hidden_size] ("W_nt", matmul3.rs:21-29).  Every
+ * finished 128-wide head row of Cq and Ck is RMS-normalised (weight 1, eps
+ * added to the root mean square) and rotated with a rotary row, as the
+ * reference's finalize does (matmul3.rs:243-254, 436-451;
+ * src/kernel/x86_64/f16_512/matmul_rms_complex.rs:76-96); arithmetic is
+ * binary32 from the sums to the single rounding to the storage type.
+ * Row r of `hidden` is token r / batch_size (capacity) of sequence
+ * r % batch_size, at position position_index + token (or positions[sequence] +
+ * token).  Query rows go to q_state in the same row order; key and value rows go
+ * to  state + sequence * kv_strides[0] + head * kv_strides[1] + position *
+ * kv_strides[2], which covers both the reference's own k_state layout
+ * [position][sequence][kv_head][128] (strides {H*128, 128, B*H*128, 1}, the
+ * permuted view of src/qwen3_moe/attention.rs:152-166) and the dimension-first
+ * cache of ellm_kv_layer.
+ * The rotary row of head h at position p starts at
+ *     rope + p * rope_position_stride + h * rope_head_stride    (elements);
+ * the reference indexes the table by output column only
+ * (rope_base.add(head_col0), matmul3.rs:243-251: position stride 0, head stride
+ * 128), a rotary table proper has position stride 128 and head stride 0.
+ * Unlike the reference's run, which takes M = batch_size rows and ignores
+ * position_interval (matmul3.rs:296-306), all position_interval token rows are
+ * projected.
+ */
+typedef struct ellm_matmul3_desc {
+  const void* hidden;   /* device, [max_position_interval][batch_size][hidden_size] */
+  const void* q_weight; /* device, [attention_head_num * 128][hidden_size] */
+  const void* k_weight; /* device, [kv_head_num * 128][hidden_size] */
+  const void* v_weight; /* device, [kv_head_num * 128][hidden_size] */
+  void* q_state;        /* device, [max_position_interval][batch_size][attention_head_num][128] */
+  void* k_state;        /* device, addressed through kv_strides */
+  void* v_state;
+  const void* rope;     /* device, (cos, sin) interleaved */
+  size_t rope_position_stride; /* elements, multiple of 4 */
+  size_t rope_head_stride;     /* elements, multiple of 4 */
+  size_t rope_elems;           /* elements in the table (bounds) */
+  size_t hidden_size;          /* K: multiple of 64 */
+  size_t batch_size;           /* sequence capacity of a token row */
+  size_t attention_head_num;
+  size_t kv_head_num;
+  size_t head_size;            /* 128 */
+  size_t kv_strides[4];        /* elements: sequence, kv head, position, 1 */
+  size_t sequence_capacity;    /* positions per K/V plane */
+  size_t max_position_interval;
+  float eps;                   /* the reference passes 1e-6 */
+  int dtype;
+} ellm_matmul3_desc;
+typedef struct ellm_matmul3 ellm_matmul3;
+int ellm_matmul3_create(const ellm_matmul3_desc* desc, ellm_matmul3** out_handle);
+/* MatMul3::run(position_index, position_interval, batch_size, cpu_num, thread_id) */
+int ellm_matmul3_run(ellm_matmul3* handle, size_t position_index, size_t position_interval,
+                     size_t batch_size, void* stream);
+/* One token per sequence at positions[sequence] (device uint32, clamped to max_position). */
+int ellm_matmul3_run_ragged(ellm_matmul3* handle, const uint32_t* positions, size_t max_position,
+                            size_t batch_size, void* stream);
+int ellm_matmul3_destroy(ellm_matmul3* handle);
+
+/*
+ * Output projection with residual: replaces MatMulAdd::new / run
+ * (src/compiler/mul/matmul_add.rs:45-75, 128-232; built by Tensor::matmul_add,
+ * src/ptensor/tensor.rs:402-437; used by src/qwen3_moe/attention.rs:176-196 on
+ * the [token][sequence][heads * 128] view of the attention output).
+ *     output = residual + a . b_nt^T     (binary32, rounded once)
+ * a: [max_position_interval][batch_size][k]; b_nt: [n][k]; residual, output:
+ * [max_position_interval][batch_size][n]; output may alias residual.
+ */
+typedef struct ellm_matmul_add_desc {
+  const void* a;
+  const void* b_nt;
+  const void* residual;
+  void* output;
+  size_t batch_size; /* m_max: sequence capacity of a token row */
+  size_t n;          /* multiple of 128 */
+  size_t k;          /* multiple of 64 */
+  size_t max_position_interval;
+  int dtype;
+} ellm_matmul_add_desc;
+typedef struct ellm_matmul_add ellm_matmul_add;
+int ellm_matmul_add_create(const ellm_matmul_add_desc* desc, ellm_matmul_add** out_handle);
+/* MatMulAdd::run(position_index, position_interval, batch_size, cpu_num, thread_id) */
+int ellm_matmul_add_run(ellm_matmul_add* handle, size_t position_index, size_t position_interval,
+                        size_t batch_size, void* stream);
+int ellm_matmul_add_destroy(ellm_matmul_add* handle);
+
 #ifdef __cplusplus
 }
 #endif

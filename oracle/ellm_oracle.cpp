@@ -46,6 +46,11 @@
 //                                   by one head_size per position): key rows normalised and
 //                                   rotated with the row of their position, value rows copied
 //
+//   oracle_matmul_nt / matmul3 /    src/compiler/mul/matmul3.rs:289-385 (three products, finalize
+//   matmul_add                      of Q and K heads :243-254), src/compiler/mul/matmul_add.rs:
+//                                   128-232 (residual + product); binary32 accumulation as in the
+//                                   reference's own checks (matmul3.rs:553-570)
+//
 // Pins (checked in tests/test_oracle_*.py): the all-ones known answer, the 1*1+2*2
 // literal, dot products 32 / 128 / 38, the 18-value scale_softmax literal, the
 // assign literals, closed forms (position 0, equal scores, constant V, shift
@@ -53,7 +58,11 @@
 // for the key-row path the 18-value rms_norm literal (rms_norm.rs:54-86), the
 // 34-value complex_mul literal (complex_mul.rs:33-49), fused == separate calls
 // (matmul_rms_complex.rs:215-322), closed forms (unit output RMS, zero row stays
-// zero, rotations keep pair norms) and a float64 restatement.
+// zero, rotations keep pair norms) and a float64 restatement; for the
+// projections the input formulas of the reference's tests (src/ptensor/tensor.rs:1079-1230,
+// src/compiler/mul/matmul3.rs:620-700) against a float64 numpy product, identity
+// weights (the projection returns its input), linearity and the finalize of the pinned
+// rms_norm / complex_mul.
 
 #include <atomic>
 #include <chrono>
@@ -544,6 +553,105 @@ int ellm_oracle_kv_append_norm_rope(void* k_cache, void* v_cache, size_t kv_head
         std::memcpy(elem_ptr(v_cache, dst, dtype), elem_ptr(v_src, src, dtype), head_size * esz);
       }
   return 0;
+}
+
+// ---- projections either side of attention ----------------------------------------
+// C[m][n] = sum_k a[m][k] * b_nt[n][k], binary32 accumulation in ascending k: the
+// arithmetic of the reference's own checks (gemm_ref_f16_acc_f32_from_wnt,
+// src/compiler/mul/matmul3.rs:553-570; verify_matmul_nt, src/ptensor/tensor.rs:1202-1228).
+// The reference's AVX-512 micro-kernel accumulates in binary16 per 3x32 tile
+// (src/kernel/x86_64/f16_512/matmul_rms_complex.rs:24-66), which is outside the contract.
+void ellm_oracle_matmul_nt(const void* a, const void* b_nt, float* c, size_t m, size_t n, size_t k,
+                           int dtype) {
+  std::vector<float> arow(k), brow(k);
+  for (size_t i = 0; i < m; ++i) {
+    load_row(a, i * k, dtype, arow.data(), k);
+    for (size_t jn = 0; jn < n; ++jn) {
+      load_row(b_nt, jn * k, dtype, brow.data(), k);
+      float sum = 0.0f;
+      for (size_t kk = 0; kk < k; ++kk) sum += arow[kk] * brow[kk];
+      c[i * n + jn] = sum;
+    }
+  }
+}
+
+// MatMul3::run (src/compiler/mul/matmul3.rs:289-385) over position_interval token rows:
+// the three products, then per finished 128-wide head row of Q and K the finalize of
+// :243-254 (rms_norm then complex_mul with a rotary row, eps from :436-451 passed in),
+// all in binary32, one rounding at the end.  hidden: [interval][batch_pitch][k];
+// q_state: [interval][batch_pitch][q_heads * head]; K/V rows go to
+// state + sequence * kv_strides[0] + head * kv_strides[1] + position * kv_strides[2];
+// rotary row of head h at position p: rope + p * rope_pos_stride + h * rope_head_stride
+// (the reference: position stride 0, head stride head_size, :243-251).
+// Returns 0, or 1 when a position falls outside capacity or the table.
+int ellm_oracle_matmul3(const void* hidden, const void* wq, const void* wk, const void* wv,
+                        void* q_state, void* k_state, void* v_state, const void* rope,
+                        size_t rope_pos_stride, size_t rope_head_stride, size_t rope_elems,
+                        size_t k, size_t batch_pitch, size_t batch_size, size_t q_heads,
+                        size_t kv_heads, size_t head, const size_t* kv_strides, size_t capacity,
+                        size_t position_index, size_t interval, const uint32_t* positions,
+                        float eps, int dtype) {
+  const size_t heads_max = q_heads > kv_heads ? q_heads : kv_heads;
+  for (size_t b = 0; b < batch_size; ++b) {
+    const size_t last = (positions ? positions[b] : position_index) + interval - 1;
+    if (last >= capacity) return 1;
+    if (last * rope_pos_stride + (heads_max - 1) * rope_head_stride + head > rope_elems) return 1;
+  }
+  std::vector<float> x(k), w(k), c(head), y(head), r(head), o(head);
+  auto head_row = [&](const void* weights, size_t h) {
+    for (size_t jn = 0; jn < head; ++jn) {
+      load_row(weights, (h * head + jn) * k, dtype, w.data(), k);
+      float sum = 0.0f;
+      for (size_t kk = 0; kk < k; ++kk) sum += x[kk] * w[kk];
+      c[jn] = sum;
+    }
+  };
+  auto finalize = [&](size_t h, size_t pos) {
+    load_row(rope, pos * rope_pos_stride + h * rope_head_stride, dtype, r.data(), head);
+    rms_norm(c.data(), y.data(), head, eps);
+    complex_mul(y.data(), r.data(), o.data(), head);
+  };
+  for (size_t t = 0; t < interval; ++t)
+    for (size_t b = 0; b < batch_size; ++b) {
+      const size_t row = t * batch_pitch + b;
+      const size_t pos = (positions ? positions[b] : position_index) + t;
+      load_row(hidden, row * k, dtype, x.data(), k);
+      for (size_t h = 0; h < q_heads; ++h) {
+        head_row(wq, h);
+        finalize(h, pos);
+        for (size_t i = 0; i < head; ++i) store_elem(q_state, (row * q_heads + h) * head + i, dtype, o[i]);
+      }
+      for (size_t h = 0; h < kv_heads; ++h) {
+        const size_t dst = b * kv_strides[0] + h * kv_strides[1] + pos * kv_strides[2];
+        head_row(wk, h);
+        finalize(h, pos);
+        for (size_t i = 0; i < head; ++i) store_elem(k_state, dst + i, dtype, o[i]);
+        head_row(wv, h);
+        for (size_t i = 0; i < head; ++i) store_elem(v_state, dst + i, dtype, c[i]);
+      }
+    }
+  return 0;
+}
+
+// MatMulAdd::run (src/compiler/mul/matmul_add.rs:128-232): output = residual + a . b_nt^T
+// (the reference copies the residual tile into the output and accumulates the product on
+// top, :176-215), binary32, one rounding.  a: [interval][batch_pitch][k]; residual,
+// output: [interval][batch_pitch][n].
+void ellm_oracle_matmul_add(const void* a, const void* b_nt, const void* residual, void* output,
+                            size_t n, size_t k, size_t batch_pitch, size_t batch_size,
+                            size_t interval, int dtype) {
+  std::vector<float> x(k), w(k);
+  for (size_t t = 0; t < interval; ++t)
+    for (size_t b = 0; b < batch_size; ++b) {
+      const size_t row = t * batch_pitch + b;
+      load_row(a, row * k, dtype, x.data(), k);
+      for (size_t jn = 0; jn < n; ++jn) {
+        load_row(b_nt, jn * k, dtype, w.data(), k);
+        float sum = 0.0f;
+        for (size_t kk = 0; kk < k; ++kk) sum += x[kk] * w[kk];
+        store_elem(output, row * n + jn, dtype, load_elem(residual, row * n + jn, dtype) + sum);
+      }
+    }
 }
 
 // The (position_index, position_interval) pairs every operator of the graph is run with

@@ -107,3 +107,13 @@ def gpu_attention(q, k, v, scale, dtype, position_index=0, batch=None, positions
 def rand_storage(shape, seed, dtype, scale=1.0):
     rng = np.random.default_rng(seed)
     return orc.to_storage(rng.standard_normal(shape, dtype=np.float32) * np.float32(scale), dtype)
+
+
+def compare_ulps(got, want, dtype, ulps=1.0, floor=2.0 ** -3):
+    """Projection outputs: both sides accumulate in binary32 (in different orders) and round
+    once, so they may land on adjacent storage values: |got - want| <= `ulps` units in the
+    last place of the storage type at max(|want|, floor)."""
+    err = np.abs(got - want)
+    bound = ulps * storage_ulp(np.maximum(np.abs(want), floor), dtype)
+    return {"max_abs": float(err.max()), "worst_ulps": float((err / bound * ulps).max()),
+            "ok": bool((err <= bound).all()) and not np.isnan(got).any()}

@@ -83,6 +83,14 @@ def load():
     lib.ellm_oracle_kv_append_norm_rope.restype = ctypes.c_int
     lib.ellm_oracle_kv_append_norm_rope.argtypes = [vp, vp, sz, sz, sz, sz, sz, sz, vp, vp, sz, vp,
                                                     sz, f, vp, ctypes.c_int]
+    lib.ellm_oracle_matmul_nt.restype = None
+    lib.ellm_oracle_matmul_nt.argtypes = [vp, vp, vp, sz, sz, sz, ctypes.c_int]
+    lib.ellm_oracle_matmul3.restype = ctypes.c_int
+    lib.ellm_oracle_matmul3.argtypes = [vp, vp, vp, vp, vp, vp, vp, vp, sz, sz, sz, sz, sz, sz, sz,
+                                        sz, sz, ctypes.POINTER(sz * 4), sz, sz, sz, vp, f,
+                                        ctypes.c_int]
+    lib.ellm_oracle_matmul_add.restype = None
+    lib.ellm_oracle_matmul_add.argtypes = [vp, vp, vp, vp, sz, sz, sz, sz, sz, ctypes.c_int]
     _lib = lib
     return lib
 
@@ -171,6 +179,44 @@ def kv_append_norm_rope(k_cache, v_cache, position_index, k_src, v_src, rope, ep
         _ptr(k_cache), _ptr(v_cache), kv_heads, capacity, d, position_index, n_tokens, batch_size,
         _ptr(k_src), _ptr(v_src), pitch, _ptr(rope), rope.shape[0], ctypes.c_float(eps),
         _ptr(pos), dtype)
+
+
+def matmul_nt(a, b_nt, dtype):
+    """a: [m, k], b_nt: [n, k] storage arrays -> float32 [m, n], binary32 accumulation."""
+    m, k = a.shape
+    n = b_nt.shape[0]
+    c = np.zeros((m, n), dtype=np.float32)
+    load().ellm_oracle_matmul_nt(_ptr(a), _ptr(b_nt), _ptr(c), m, n, k, dtype)
+    return c
+
+
+def matmul3(hidden, wq, wk, wv, q_state, k_state, v_state, rope, kv_strides, capacity, position_index,
+            interval, dtype, batch_size=None, positions=None, eps=1e-6, rope_position_stride=128,
+            rope_head_stride=0, head=128):
+    """hidden: [interval_capacity, batch_pitch, k]; weights: [heads * head, k]; q_state:
+    [interval_capacity, batch_pitch, q_heads, head]; k_state / v_state: storage arrays addressed
+    through kv_strides (elements), all written in place.  Returns the oracle's status."""
+    pitch, k = hidden.shape[1], hidden.shape[2]
+    if batch_size is None:
+        batch_size = pitch
+    pos = np.ascontiguousarray(positions, dtype=np.uint32) if positions is not None else None
+    strides = (ctypes.c_size_t * 4)(*[int(x) for x in kv_strides])
+    return load().ellm_oracle_matmul3(
+        _ptr(hidden), _ptr(wq), _ptr(wk), _ptr(wv), _ptr(q_state), _ptr(k_state), _ptr(v_state),
+        _ptr(rope), rope_position_stride, rope_head_stride, rope.size, k, pitch, batch_size,
+        wq.shape[0] // head, wk.shape[0] // head, head, ctypes.byref(strides), capacity,
+        position_index, interval, _ptr(pos), ctypes.c_float(eps), dtype)
+
+
+def matmul_add(a, b_nt, residual, dtype, interval=None, batch_size=None):
+    """a: [interval_capacity, batch_pitch, k]; b_nt: [n, k]; residual: [.., .., n] -> output."""
+    pitch, k = a.shape[1], a.shape[2]
+    n = b_nt.shape[0]
+    out = np.zeros_like(residual)
+    load().ellm_oracle_matmul_add(_ptr(a), _ptr(b_nt), _ptr(residual), _ptr(out), n, k, pitch,
+                                  batch_size if batch_size is not None else pitch,
+                                  interval if interval is not None else a.shape[0], dtype)
+    return out
 
 
 def assign(length, num, idx):
