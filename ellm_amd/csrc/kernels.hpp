@@ -104,8 +104,14 @@ struct ProjectArgs {
   uint32_t position_index, max_start, finalize0;
   float eps;
   int dtype;
+  // workspace of the few-rows kernel (may be null: the tile kernel runs whatever the row count)
+  float* ws;
+  uint32_t* counters;
 };
 hipError_t launch_project(const ProjectArgs& a, hipStream_t stream);
+// Few-rows kernel: rows it handles at most, floats of partial sums and counters it needs.
+constexpr uint32_t kProjectSmallRows = 64;
+size_t project_workspace_floats(uint32_t heads, uint32_t K);
 
 // Records the message ellm_last_error_string() returns on this thread; returns status.
 int set_error(int status, const char* fmt, ...) __attribute__((format(printf, 2, 3)));

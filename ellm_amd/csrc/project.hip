@@ -21,12 +21,10 @@
 // through a three-stage LDS ring: chunk c is read while chunk c+2 is written, chunk
 // c+1 is already complete, so the first operands of the next chunk are requested
 // before the barrier that ends the current one and the MFMA stream never drains.
-#include <type_traits>
-
-#include "common.hpp"
-#include "kernels.hpp"
+#include "project_common.hpp"
 
 namespace ellm {
+using namespace proj;
 namespace {
 
 constexpr int kTile = 256;                          // tokens, and output columns, per workgroup
@@ -40,48 +38,10 @@ constexpr int kProjThreads = 256;
 constexpr int kProjLdsBytes = kStages * kStageBytes;
 static_assert(4 * kEpWaveBytes <= kProjLdsBytes, "the epilogue reuses the stages");
 constexpr int kGroupM = 4;                          // token tiles that take turns on one column tile
-constexpr int kBufFlags = 0x00020000;               // raw buffer of 32-bit data, no swizzle
 
 typedef __attribute__((address_space(3))) u32x4 LdsVec4;
 typedef __attribute__((address_space(3))) u32x2 LdsVec2;
 typedef __attribute__((address_space(3))) uint64_t LdsU64;
-
-struct ProjectKernelArgs {
-  const uint16_t* x;         // [rows][K]
-  const uint16_t* w[3];      // column segments 0 (query / plain), 1 (key), 2 (value): [heads * 128][K]
-  uint16_t* out0;            // segment 0 destination, row-major [rows][ld0]
-  const uint16_t* residual;  // added to segment 0 (same layout), may be null
-  uint16_t* k_out;
-  uint16_t* v_out;
-  const uint16_t* rope;
-  const uint32_t* positions;
-  size_t kv_stride_seq, kv_stride_head, kv_stride_pos;  // elements
-  uint32_t ld0;
-  uint32_t rope_pos_stride, rope_head_stride;           // elements
-  uint32_t K, rows, batch_pitch, batch;
-  uint32_t heads0, heads_kv;
-  uint32_t tiles_m, tiles_n;
-  uint32_t position_index, max_start;
-  uint32_t finalize0;        // segment 0 rows are normalised and rotated
-  float eps;
-};
-
-template <int N, typename F>
-__device__ __forceinline__ void static_for(F&& f) {
-  if constexpr (N > 0) {
-    static_for<N - 1>(f);
-    f(std::integral_constant<int, N - 1>{});
-  }
-}
-
-__device__ __forceinline__ uint64_t uniform64(const void* p) {
-  const uint32_t lo = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(uint64_t)p);
-  const uint32_t hi = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)((uint64_t)p >> 32));
-  return ((uint64_t)hi << 32) | (uint64_t)lo;
-}
-
-constexpr int kModeQkv = 0;  // heads normalised + rotated (or passed through), K/V to token coordinates
-constexpr int kModeAdd = 1;  // plain product plus a residual of the output's layout
 
 template <typename S, int MODE>
 __global__ __launch_bounds__(kProjThreads) void project_kernel(ProjectKernelArgs p) {
@@ -383,6 +343,8 @@ hipError_t launch_project(const ProjectArgs& a, hipStream_t stream) {
   p.max_start = a.max_start;
   p.finalize0 = a.finalize0;
   p.eps = a.eps;
+  if (a.ws && a.counters && a.rows <= kSmallRowsMax)
+    return launch_project_small(p, a.ws, a.counters, a.dtype, a.residual != nullptr, stream);
   const uint32_t blocks = p.tiles_m * p.tiles_n;
   auto go = [&](auto kernel) {
     hipError_t e = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -394,6 +356,10 @@ hipError_t launch_project(const ProjectArgs& a, hipStream_t stream) {
   if (a.residual)
     return a.dtype == 0 ? go(project_kernel<F16, kModeAdd>) : go(project_kernel<BF16, kModeAdd>);
   return a.dtype == 0 ? go(project_kernel<F16, kModeQkv>) : go(project_kernel<BF16, kModeQkv>);
+}
+
+size_t project_workspace_floats(uint32_t heads, uint32_t K) {
+  return small_workspace_floats(heads, K);
 }
 
 }  // namespace ellm

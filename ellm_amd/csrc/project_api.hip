@@ -16,10 +16,47 @@ constexpr size_t kMaxK = 1u << 16;
 
 struct ellm_matmul3 {
   ellm_matmul3_desc d;
+  float* ws;
+  uint32_t* counters;
 };
 struct ellm_matmul_add {
   ellm_matmul_add_desc d;
+  float* ws;
+  uint32_t* counters;
 };
+
+namespace {
+// Partial sums and arrival counters of the few-rows kernel; left null (the tile kernel then
+// runs every call) when they would take more than 64 MiB.
+int alloc_small_workspace(uint32_t heads, uint32_t K, float** ws, uint32_t** counters) {
+  *ws = nullptr;
+  *counters = nullptr;
+  int n_dev = 0;
+  if (hipGetDeviceCount(&n_dev) != hipSuccess || n_dev == 0) {
+    (void)hipGetLastError();
+    return ellm::set_error(ELLM_ERR_NO_DEVICE, "no HIP device visible");
+  }
+  const size_t floats = ellm::project_workspace_floats(heads, K);
+  if (floats * sizeof(float) > (size_t)64 << 20) return ELLM_OK;
+  hipError_t e = hipMalloc((void**)ws, floats * sizeof(float));
+  if (e == hipSuccess) e = hipMalloc((void**)counters, heads * sizeof(uint32_t));
+  if (e == hipSuccess) e = hipMemset(*counters, 0, heads * sizeof(uint32_t));
+  if (e != hipSuccess) {
+    (void)hipFree(*ws);
+    (void)hipFree(*counters);
+    *ws = nullptr;
+    *counters = nullptr;
+    return ellm::set_error(ELLM_ERR_HIP, "projection workspace: %s", hipGetErrorString(e));
+  }
+  return ELLM_OK;
+}
+int free_small_workspace(float* ws, uint32_t* counters) {
+  hipError_t e1 = ws ? hipFree(ws) : hipSuccess, e2 = counters ? hipFree(counters) : hipSuccess;
+  if (e1 != hipSuccess || e2 != hipSuccess)
+    return ellm::set_error(ELLM_ERR_HIP, "hipFree: %s", hipGetErrorString(e1 != hipSuccess ? e1 : e2));
+  return ELLM_OK;
+}
+}  // namespace
 
 extern "C" {
 
@@ -59,13 +96,21 @@ int ellm_matmul3_create(const ellm_matmul3_desc* d, ellm_matmul3** out_handle) {
   ellm_matmul3* h = new (std::nothrow) ellm_matmul3;
   if (!h) return ellm::set_error(ELLM_ERR_HIP, "out of host memory");
   h->d = *d;
+  const int rc = alloc_small_workspace((uint32_t)(d->attention_head_num + 2 * d->kv_head_num),
+                                       (uint32_t)d->hidden_size, &h->ws, &h->counters);
+  if (rc != ELLM_OK) {
+    delete h;
+    return rc;
+  }
   *out_handle = h;
   return ELLM_OK;
 }
 
 int ellm_matmul3_destroy(ellm_matmul3* h) {
+  if (!h) return ELLM_OK;
+  const int rc = free_small_workspace(h->ws, h->counters);
   delete h;
-  return ELLM_OK;
+  return rc;
 }
 
 static int matmul3_launch(ellm_matmul3* h, size_t position_index, size_t position_interval,
@@ -110,6 +155,8 @@ static int matmul3_launch(ellm_matmul3* h, size_t position_index, size_t positio
   a.finalize0 = 1;
   a.eps = d.eps;
   a.dtype = d.dtype;
+  a.ws = h->ws;
+  a.counters = h->counters;
   const hipError_t e = ellm::launch_project(a, (hipStream_t)stream);
   if (e != hipSuccess) return ellm::set_error(ELLM_ERR_HIP, "projection launch: %s", hipGetErrorString(e));
   return ELLM_OK;
@@ -149,13 +196,20 @@ int ellm_matmul_add_create(const ellm_matmul_add_desc* d, ellm_matmul_add** out_
   ellm_matmul_add* h = new (std::nothrow) ellm_matmul_add;
   if (!h) return ellm::set_error(ELLM_ERR_HIP, "out of host memory");
   h->d = *d;
+  const int rc = alloc_small_workspace((uint32_t)(d->n / 128), (uint32_t)d->k, &h->ws, &h->counters);
+  if (rc != ELLM_OK) {
+    delete h;
+    return rc;
+  }
   *out_handle = h;
   return ELLM_OK;
 }
 
 int ellm_matmul_add_destroy(ellm_matmul_add* h) {
+  if (!h) return ELLM_OK;
+  const int rc = free_small_workspace(h->ws, h->counters);
   delete h;
-  return ELLM_OK;
+  return rc;
 }
 
 int ellm_matmul_add_run(ellm_matmul_add* h, size_t position_index, size_t position_interval,
@@ -182,6 +236,8 @@ int ellm_matmul_add_run(ellm_matmul_add* h, size_t position_index, size_t positi
   a.heads_kv = 0;
   a.finalize0 = 0;
   a.dtype = d.dtype;
+  a.ws = h->ws;
+  a.counters = h->counters;
   const hipError_t e = ellm::launch_project(a, (hipStream_t)stream);
   if (e != hipSuccess) return ellm::set_error(ELLM_ERR_HIP, "projection launch: %s", hipGetErrorString(e));
   return ELLM_OK;

@@ -1,0 +1,60 @@
+// Shared by the two projection kernels (tile kernel for many rows, streaming kernel
+// for a few rows): kernel arguments and small helpers.
+#pragma once
+
+#include <type_traits>
+
+#include "common.hpp"
+#include "kernels.hpp"
+
+namespace ellm {
+namespace proj {
+
+constexpr int kBufFlags = 0x00020000;  // raw buffer of 32-bit data, no swizzle
+
+struct ProjectKernelArgs {
+  const uint16_t* x;         // [rows][K]
+  const uint16_t* w[3];      // column segments 0 (query / plain), 1 (key), 2 (value): [heads * 128][K]
+  uint16_t* out0;            // segment 0 destination, row-major [rows][ld0]
+  const uint16_t* residual;  // added to segment 0 (same layout), may be null
+  uint16_t* k_out;
+  uint16_t* v_out;
+  const uint16_t* rope;
+  const uint32_t* positions;
+  size_t kv_stride_seq, kv_stride_head, kv_stride_pos;  // elements
+  uint32_t ld0;
+  uint32_t rope_pos_stride, rope_head_stride;           // elements
+  uint32_t K, rows, batch_pitch, batch;
+  uint32_t heads0, heads_kv;
+  uint32_t tiles_m, tiles_n;
+  uint32_t position_index, max_start;
+  uint32_t finalize0;        // segment 0 rows are normalised and rotated
+  float eps;
+};
+
+template <int N, typename F>
+__device__ __forceinline__ void static_for(F&& f) {
+  if constexpr (N > 0) {
+    static_for<N - 1>(f);
+    f(std::integral_constant<int, N - 1>{});
+  }
+}
+
+__device__ __forceinline__ uint64_t uniform64(const void* p) {
+  const uint32_t lo = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(uint64_t)p);
+  const uint32_t hi = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)((uint64_t)p >> 32));
+  return ((uint64_t)hi << 32) | (uint64_t)lo;
+}
+
+constexpr int kModeQkv = 0;  // heads normalised + rotated (or passed through), K/V to token coordinates
+constexpr int kModeAdd = 1;  // plain product plus a residual of the output's layout
+
+// Streaming kernel for a few rows (project_small.hip).
+constexpr uint32_t kSmallRowsMax = 64;
+size_t small_workspace_floats(uint32_t heads, uint32_t K);
+hipError_t launch_project_small(const ProjectKernelArgs& p, float* ws, uint32_t* counters, int dtype,
+                                bool add, hipStream_t stream);
+
+
+}  // namespace proj
+}  // namespace ellm

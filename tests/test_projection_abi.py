@@ -1,5 +1,6 @@
-"""Argument checking of the projection entry points (no GPU needed: nothing is launched,
-the pointers are never dereferenced)."""
+"""Argument checking of the projection entry points: descriptions are rejected before
+anything touches a device; the range checks of run need a handle (and so a device) but
+launch nothing and never dereference the pointers."""
 import ctypes
 
 import pytest
@@ -7,7 +8,7 @@ import pytest
 import ellm_amd
 from ellm_amd import _lib
 
-OK, INVALID, UNSUPPORTED, OUT_OF_RANGE = 0, 1, 2, 3
+OK, INVALID, UNSUPPORTED, OUT_OF_RANGE, NO_DEVICE = 0, 1, 2, 3, 5
 
 
 def _m3(**over):
@@ -29,7 +30,6 @@ def _m3(**over):
 
 
 @pytest.mark.parametrize("over,status", [
-    (dict(), OK),
     (dict(hidden=None), INVALID),
     (dict(rope=0x1004), INVALID),
     (dict(dtype=3), INVALID),
@@ -45,11 +45,19 @@ def test_matmul3_create(over, status):
     lib = ellm_amd.load_library()
     h = ctypes.c_void_p()
     assert lib.ellm_matmul3_create(ctypes.byref(_m3(**over)), ctypes.byref(h)) == status
-    assert bool(h.value) == (status == OK)
-    if h.value:
-        assert lib.ellm_matmul3_destroy(h) == OK
+    assert not h.value
 
 
+def test_create_without_a_device_says_so():
+    lib = ellm_amd.load_library()
+    if lib.ellm_device_count() > 0:
+        pytest.skip("a device is present")
+    h = ctypes.c_void_p()
+    assert lib.ellm_matmul3_create(ctypes.byref(_m3()), ctypes.byref(h)) == NO_DEVICE and not h.value
+    assert lib.ellm_matmul_add_create(ctypes.byref(_ma()), ctypes.byref(h)) == NO_DEVICE and not h.value
+
+
+@pytest.mark.gpu
 def test_matmul3_run_range_checks():
     lib = ellm_amd.load_library()
     h = ctypes.c_void_p()
@@ -79,7 +87,6 @@ def _ma(**over):
 
 
 @pytest.mark.parametrize("over,status", [
-    (dict(), OK),
     (dict(output=None), INVALID),
     (dict(a=0x1008), INVALID),
     (dict(n=200), UNSUPPORTED),
@@ -87,12 +94,19 @@ def _ma(**over):
     (dict(batch_size=0), INVALID),
     (dict(dtype=-1), INVALID),
 ])
-def test_matmul_add_create_and_run_checks(over, status):
+def test_matmul_add_create(over, status):
     lib = ellm_amd.load_library()
     h = ctypes.c_void_p()
     assert lib.ellm_matmul_add_create(ctypes.byref(_ma(**over)), ctypes.byref(h)) == status
-    if status == OK:
-        assert lib.ellm_matmul_add_run(h, 0, 9, 4, None) == OUT_OF_RANGE
-        assert lib.ellm_matmul_add_run(h, 0, 1, 5, None) == OUT_OF_RANGE
-        assert lib.ellm_matmul_add_run(h, 0, 0, 4, None) == OK
-        assert lib.ellm_matmul_add_destroy(h) == OK
+    assert not h.value
+
+
+@pytest.mark.gpu
+def test_matmul_add_run_range_checks():
+    lib = ellm_amd.load_library()
+    h = ctypes.c_void_p()
+    assert lib.ellm_matmul_add_create(ctypes.byref(_ma()), ctypes.byref(h)) == OK
+    assert lib.ellm_matmul_add_run(h, 0, 9, 4, None) == OUT_OF_RANGE
+    assert lib.ellm_matmul_add_run(h, 0, 1, 5, None) == OUT_OF_RANGE
+    assert lib.ellm_matmul_add_run(h, 0, 0, 4, None) == OK
+    assert lib.ellm_matmul_add_destroy(h) == OK
