@@ -355,6 +355,49 @@ def bench_output_projection(tokens, steps, warmup, hidden=2048, hq=32, dtype_nam
             "tflops": flops / (step_ms * 1e-3) / 1e12, "kernel_tflops": flops / (kern_ms * 1e-3) / 1e12}
 
 
+def bench_step_projections(batch, steps, warmup, hidden=2048, hq=32, hkv=4, copies=8):
+    """The two projections of a single-token step (one token row per sequence): fused Q/K/V
+    and output + residual.  The weights rotate over `copies` sets (8 x 21 MB and 8 x 17 MB)
+    so that a step streams them from HBM, as a model with many layers does."""
+    import torch
+
+    import ellm_amd
+
+    dt = torch.float16
+    cap = 1024
+    x = _dev_normal((1, batch, hidden), dt, 91)
+    j = torch.arange(D // 2, device="cuda", dtype=torch.float64)
+    ang = torch.arange(cap, device="cuda", dtype=torch.float64)[:, None] * (1.0e6 ** (-2.0 * j / D))[None, :]
+    rope = torch.stack((torch.cos(ang), torch.sin(ang)), dim=-1).reshape(cap, D).to(dt)
+    q = torch.zeros((1, batch, hq, D), dtype=dt, device="cuda")
+    cache = ellm_amd.KVCache(1, batch, hkv, cap, ellm_amd.DTYPE_F16)
+    kt, vt = cache.layer_tensors(0, dt)
+    _, _, strides = cache.layer(0)
+    qkv, keep = [], []
+    for c in range(copies):
+        w = [_dev_normal((h * D, hidden), dt, 100 + 3 * c + i, scale=hidden ** -0.5) for i, h in enumerate((hq, hkv, hkv))]
+        keep.append(w)
+        qkv.append(ellm_amd.MatMul3(x, w[0], q, w[1], kt, w[2], vt, rope, D, batch, hq, hkv, strides, cap))
+    per, qkv_ms = _time_steps(lambda i: qkv[i % copies].run(7, 1, batch), steps, warmup)
+    qkv_kernel_ms = per[0]
+    a = _dev_normal((1, batch, hq * D), dt, 92)
+    r = _dev_normal((1, batch, hidden), dt, 93)
+    out = torch.zeros_like(r)
+    oproj = []
+    for c in range(copies):
+        w = _dev_normal((hidden, hq * D), dt, 200 + c, scale=(hq * D) ** -0.5)
+        keep.append(w)
+        oproj.append(ellm_amd.MatMulAdd(a, w, r, out))
+    per, o_ms = _time_steps(lambda i: oproj[i % copies].run(7, 1, batch), steps, warmup)
+    for op in qkv + oproj:
+        op.close()
+    cache.close()
+    qkv_bytes = (hq + 2 * hkv) * D * hidden * 2 + batch * hidden * 2 + batch * (hq + 2 * hkv) * D * 2
+    o_bytes = hidden * hq * D * 2 + batch * hq * D * 2 + 2 * batch * hidden * 2
+    return {"qkv_ms": qkv_ms, "qkv_kernel_ms": qkv_kernel_ms, "qkv_bytes": qkv_bytes,
+            "o_ms": o_ms, "o_kernel_ms": per[0], "o_bytes": o_bytes}
+
+
 def cpu_baseline_decode(batch, length, hq=32, hkv=4, budget_s=20.0):
     """The CPU oracle on the full single-token workload (all host cores)."""
     import numpy as np
@@ -388,7 +431,7 @@ def main():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--skip-cpu", action="store_true")
-    ap.add_argument("--only", default="", help="decode | prefill | decode128k | chunk | mixed | mixed48 | kvwrite | tokenstep | qkv | oproj")
+    ap.add_argument("--only", default="", help="decode | prefill | decode128k | chunk | mixed | mixed48 | kvwrite | tokenstep | qkv | oproj | stepproj")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="first run one plain 256 MiB device copy (a known-traffic dispatch "
                          "for scaling rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE readings)")
@@ -534,6 +577,23 @@ def main():
             "roofline": {"bound": "mfma", "achieved": round(po["kernel_tflops"], 2),
                          "peak": MFMA_F16_PEAK_TFLOPS, "unit": "TFLOP/s",
                          "frac": round(po["kernel_tflops"] / MFMA_F16_PEAK_TFLOPS, 4), "traffic": None},
+        })
+
+    if args.only in ("", "stepproj"):
+        sp = bench_step_projections(16, args.steps, args.warmup)
+        also.append({
+            "workload": "projections of a single-token step, 16 sequences: fused Q/K/V (2048 -> 5120, norm + "
+                        "rotation, K/V to the cache) and output + residual (4096 -> 2048), fp16, weights "
+                        "streamed from HBM (8 rotating sets)",
+            "metric": "weight stream GB/s (Q/K/V projection)", "unit": "GB/s",
+            "value": round(sp["qkv_bytes"] / (sp["qkv_ms"] * 1e-3) / 1e9, 1),
+            "ms_per_step": round(sp["qkv_ms"], 5), "steps": args.steps,
+            "output_projection_ms": round(sp["o_ms"], 5),
+            "output_projection_gbs": round(sp["o_bytes"] / (sp["o_ms"] * 1e-3) / 1e9, 1),
+            "roofline": {"bound": "hbm", "achieved": round(sp["qkv_bytes"] / (sp["qkv_kernel_ms"] * 1e-3) / 1e9, 1),
+                         "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                         "frac": round(sp["qkv_bytes"] / (sp["qkv_kernel_ms"] * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
+                         "traffic": None},
         })
 
     cpu = None

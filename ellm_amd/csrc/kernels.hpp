@@ -110,7 +110,6 @@ struct ProjectArgs {
 };
 hipError_t launch_project(const ProjectArgs& a, hipStream_t stream);
 // Few-rows kernel: rows it handles at most, floats of partial sums and counters it needs.
-constexpr uint32_t kProjectSmallRows = 64;
 size_t project_workspace_floats(uint32_t heads, uint32_t K);
 
 // Records the message ellm_last_error_string() returns on this thread; returns status.

@@ -17,10 +17,11 @@
 //
 // A workgroup of 4 waves (one per SIMD, 512 registers each) owns a tile of 256 tokens x
 // 256 output columns (two heads); wave (wn, wm) owns head wn and tokens 128 wm..+127 as
-// 4 x 4 accumulator blocks (256 accumulator registers).  K runs in chunks of 32
-// through a three-stage LDS ring: chunk c is read while chunk c+2 is written, chunk
-// c+1 is already complete, so the first operands of the next chunk are requested
-// before the barrier that ends the current one and the MFMA stream never drains.
+// 4 x 4 accumulator blocks (256 accumulator registers).  K runs in chunks of 64 (one
+// 128-byte cache line per operand row and chunk: a fetch of half a line costs the vector
+// cache the same miss entry as a whole one) through two LDS stages: chunk c is read while
+// chunk c + 1, fetched into registers an iteration earlier, is written to the other stage.
+// Calls with at most 32 rows go to the streaming kernel of project_small.hip instead.
 #include "project_common.hpp"
 
 namespace ellm {
@@ -28,10 +29,14 @@ using namespace proj;
 namespace {
 
 constexpr int kTile = 256;                          // tokens, and output columns, per workgroup
-constexpr int kKc = 32;                             // K elements per chunk
-constexpr int kRowPitch = (kKc + 8) * 2;            // 80 B: 16 consecutive rows' 16-byte pieces tile all 64 banks
+constexpr int kKc = 64;                             // K elements per chunk: one 128-byte line per row
+// A row of a stage is the chunk's 128 bytes, unpadded; its eight 16-byte pieces are stored
+// permuted, piece p of row r at p ^ ((r >> 1) & 7): the 16 lanes of a staging store (two
+// whole rows) and the 16 lanes of an operand read (one piece of 16 consecutive rows) then
+// both touch every LDS bank once.
+constexpr int kRowPitch = kKc * 2;
 constexpr int kStageBytes = 2 * kTile * kRowPitch;  // X rows then W rows
-constexpr int kStages = 3;
+constexpr int kStages = 2;
 constexpr int kEpPitch = kHeadDim * 2 + 16;         // output row in LDS
 constexpr int kEpWaveBytes = 32 * kEpPitch + 32 * 8;  // 32 rows and their destinations, per wave
 constexpr int kProjThreads = 256;
@@ -94,31 +99,31 @@ __global__ __launch_bounds__(kProjThreads) void project_kernel(ProjectKernelArgs
   };
   const __amdgpu_buffer_rsrc_t w_rsrc0 = head_rsrc(2 * tn), w_rsrc1 = head_rsrc(2 * tn + 1);
 
-  // staging: thread -> row tid / 4 (+ 64 i), 16-byte piece tid % 4 of the chunk's 64 B
-  const uint32_t st_row = tid >> 2, st_piece = tid & 3;
-  uint32_t src_off[4];  // rows st_row + 64 i of a 256-row (X) or, i & 1, 128-row (W head) source
+  // staging: thread -> row tid / 8 (+ 32 i), 16-byte piece tid % 8 of the chunk's 128 B:
+  // eight lanes fetch one whole cache line
+  const uint32_t st_row = tid >> 3, st_piece = tid & 7;
+  uint32_t src_off[8];  // rows st_row + 32 i of a 256-row (X) or, i & 3, 128-row (W head) source
 #pragma unroll
-  for (int i = 0; i < 4; ++i) src_off[i] = (st_row + 64 * i) * K * 2 + st_piece * 16;
+  for (int i = 0; i < 8; ++i) src_off[i] = (st_row + 32 * i) * K * 2 + st_piece * 16;
   const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t*)proj_smem;
   auto pin = [](uint32_t addr) {
     asm volatile("" : "+v"(addr));
     return addr;
   };
-  const uint32_t st_store = lds0 + st_row * kRowPitch + st_piece * 16;
-  // Two sets of staging registers: a chunk is requested two iterations (about 1.2 us)
-  // before it is stored to LDS, which is what a fetch from HBM can take under load.
-  u32x4 stg[2][8];
+  const uint32_t st_store = lds0 + st_row * kRowPitch + ((st_piece ^ ((st_row >> 1) & 7)) * 16);
+  // A chunk is requested one iteration (64 MFMAs, about 1.2 us) before it is stored to LDS.
+  u32x4 stg[16];
   // (a chunk past the last one fetches bytes of the next row, or zeros past the end of
   // the buffer, into a stage nobody reads)
-  auto load_piece = [&](auto set, uint32_t chunk, int i) {
+  auto load_piece = [&](uint32_t chunk, int i) {
     const uint32_t soff = chunk * (kKc * 2);
-    if (i < 4)
-      stg[set][i] = __builtin_amdgcn_raw_buffer_load_b128(x_rsrc, src_off[i], soff, 0);
+    if (i < 8)
+      stg[i] = __builtin_amdgcn_raw_buffer_load_b128(x_rsrc, src_off[i], soff, 0);
     else
-      stg[set][i] = __builtin_amdgcn_raw_buffer_load_b128((i < 6) ? w_rsrc0 : w_rsrc1, src_off[i & 1], soff, 0);
+      stg[i] = __builtin_amdgcn_raw_buffer_load_b128((i < 12) ? w_rsrc0 : w_rsrc1, src_off[i & 3], soff, 0);
   };
-  auto store_piece = [&](auto set, uint32_t base, int i) {
-    *(LdsVec4*)(base + 64 * i * kRowPitch) = stg[set][i];
+  auto store_piece = [&](uint32_t base, int i) {
+    *(LdsVec4*)(base + 32 * i * kRowPitch) = stg[i];
   };
 
   f32x16 acc[4][4];  // [column block nb][token block mb]
@@ -129,81 +134,77 @@ __global__ __launch_bounds__(kProjThreads) void project_kernel(ProjectKernelArgs
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[nb][mb][r] = 0.0f;
 
-  // operand reads: lane (j, g) takes row j of a 32-row block, K piece g of the 16-wide step
-  const uint32_t x_read = lds0 + (wm * 128 + j) * kRowPitch + g * 16;
-  const uint32_t w_read = lds0 + (kTile + wn * 128 + j) * kRowPitch + g * 16;
-  // operand o of a step: 0..3 = W blocks, 4..7 = X blocks
-  auto read_operand = [&](uint32_t xb, uint32_t wb, int step, int o) {
-    const uint32_t at = (o < 4 ? wb + 32 * o * kRowPitch : xb + 32 * (o - 4) * kRowPitch) + 32 * step;
+  // operand reads: lane (j, g) takes row j of a 32-row block, piece 2 step + g of the row,
+  // permuted with the row's key; the four steps of a chunk have their own lane addresses
+  const uint32_t swz = (j >> 1) & 7;
+  uint32_t x_read[4], w_read[4];
+#pragma unroll
+  for (int st = 0; st < 4; ++st) {
+    x_read[st] = lds0 + (wm * 128 + j) * kRowPitch + (((2 * st + g) ^ swz) * 16);
+    w_read[st] = lds0 + (kTile + wn * 128 + j) * kRowPitch + (((2 * st + g) ^ swz) * 16);
+  }
+  // operand o of a step: 0 = W block 0, 1..4 = X blocks, 5..7 = W blocks 1..3 (the order
+  // in which the step's MFMAs first need them)
+  auto read_operand = [&](uint32_t xb, uint32_t wb, int o) {
+    const uint32_t at = (o == 0) ? wb : (o < 5 ? xb + 32 * (o - 1) * kRowPitch : wb + 32 * (o - 4) * kRowPitch);
     return (u32x4) * (const LdsVec4*)at;
   };
+  // MFMA n of a step: W block n / 4 times X block n % 4
+  auto w_of = [](int n) { return (n >> 2) == 0 ? 0 : 4 + (n >> 2); };
+  auto x_of = [](int n) { return 1 + (n & 3); };
 
-  // prologue: chunks 0 and 1 into stages 0 and 1, chunks 2 and 3 into the staging registers
-  constexpr std::integral_constant<int, 0> kSet0{};
-  constexpr std::integral_constant<int, 1> kSet1{};
+  // prologue: chunk 0 into stage 0, chunk 1 into the staging registers
 #pragma unroll
-  for (int i = 0; i < 8; ++i) load_piece(kSet0, 0, i);
-#pragma unroll
-  for (int i = 0; i < 8; ++i) load_piece(kSet1, 1, i);
+  for (int i = 0; i < 16; ++i) load_piece(0, i);
   {
     const uint32_t base = pin(st_store);
 #pragma unroll
-    for (int i = 0; i < 8; ++i) store_piece(kSet0, base, i);
-#pragma unroll
-    for (int i = 0; i < 8; ++i) load_piece(kSet0, 2, i);
-    const uint32_t base1 = pin(st_store + kStageBytes);
-#pragma unroll
-    for (int i = 0; i < 8; ++i) store_piece(kSet1, base1, i);
-#pragma unroll
-    for (int i = 0; i < 8; ++i) load_piece(kSet1, 3, i);
+    for (int i = 0; i < 16; ++i) {
+      store_piece(base, i);
+      load_piece(1, i);
+    }
   }
   __syncthreads();
 
+  // One iteration = one chunk: four 16-wide steps, 64 MFMAs.  Chunk c sits in stage c % 2;
+  // during it the staging registers (chunk c + 1) are stored to the other stage and
+  // refilled with chunk c + 2.  The operands of a step are read during the step before
+  // it, except those of a chunk's first step: the stage is complete only at the barrier.
+  // LDS traffic is spread evenly (a read every second MFMA, a store every fourth): the four
+  // waves together keep the LDS pipe busy most of the time, and a burst of stores
+  // would still be draining when the barrier is reached.
   u32x4 opa[8], opb[8];
-  {
-    const uint32_t xb = pin(x_read), wb = pin(w_read);
+  for (uint32_t c = 0; c < n_chunks; ++c) {
+    const uint32_t cur = (c & 1) * kStageBytes, nxt = kStageBytes - cur;
+    uint32_t xb[4], wb[4];
 #pragma unroll
-    for (int o = 0; o < 8; ++o) opa[o] = read_operand(xb, wb, 0, o);
-  }
-
-  // One iteration = one chunk (two 16-wide steps, 32 MFMAs).  Chunk c sits in stage
-  // c % 3; during it the staging set c % 2 (chunk c + 2) is stored to stage (c + 2) % 3
-  // and refilled with chunk c + 4.
-  uint32_t stage = 0;
-  auto iteration = [&](auto set, uint32_t c) __attribute__((always_inline)) {
-    const uint32_t stage1 = (stage == 2) ? 0 : stage + 1;   // chunk c + 1
-    const uint32_t stage2 = (stage1 == 2) ? 0 : stage1 + 1;  // chunk c + 2 goes here
-    const uint32_t xb = pin(x_read + stage * kStageBytes), wb = pin(w_read + stage * kStageBytes);
-    const uint32_t xb1 = pin(x_read + stage1 * kStageBytes), wb1 = pin(w_read + stage1 * kStageBytes);
-    const uint32_t store_at = pin(st_store + stage2 * kStageBytes);
+    for (int st = 0; st < 4; ++st) {
+      xb[st] = pin(x_read[st] + cur);
+      wb[st] = pin(w_read[st] + cur);
+    }
+    const uint32_t store_at = pin(st_store + nxt);
+#pragma unroll
+    for (int o = 0; o < 8; ++o) opa[o] = read_operand(xb[0], wb[0], o);
     __builtin_amdgcn_sched_barrier(0);
-    // step 0: operands opa, fetch step 1 into opb
-    static_for<16>([&](auto n_) {
+    static_for<64>([&](auto n_) {
       constexpr int n = decltype(n_)::value;
-      acc[n >> 2][n & 3] = M::m32x32x16(opa[n >> 2], opa[4 + (n & 3)], acc[n >> 2][n & 3]);
-      if constexpr (n < 8) opb[n] = read_operand(xb, wb, 1, n);
-      __builtin_amdgcn_sched_barrier(0);
-    });
-    // step 1: operands opb, fetch step 0 of chunk c + 1 into opa; staging
-    static_for<16>([&](auto n_) {
-      constexpr int n = decltype(n_)::value;
-      acc[n >> 2][n & 3] = M::m32x32x16(opb[n >> 2], opb[4 + (n & 3)], acc[n >> 2][n & 3]);
-      if constexpr (n < 8) opa[n] = read_operand(xb1, wb1, 0, n);
-      if constexpr (n >= 8) {
-        store_piece(set, store_at, n - 8);
-        load_piece(set, c + 4, n - 8);
+      constexpr int st = n >> 4, m = n & 15;
+      if constexpr ((st & 1) == 0) {
+        acc[m >> 2][m & 3] = M::m32x32x16(opa[w_of(m)], opa[x_of(m)], acc[m >> 2][m & 3]);
+        if constexpr ((n & 1) == 0) opb[m >> 1] = read_operand(xb[st + 1], wb[st + 1], m >> 1);
+      } else {
+        acc[m >> 2][m & 3] = M::m32x32x16(opb[w_of(m)], opb[x_of(m)], acc[m >> 2][m & 3]);
+        if constexpr ((n & 1) == 0 && st < 3) opa[m >> 1] = read_operand(xb[st + 1], wb[st + 1], m >> 1);
+      }
+      if constexpr ((n & 3) == 3) {
+        store_piece(store_at, n >> 2);
+        load_piece(c + 2, n >> 2);
       }
       __builtin_amdgcn_sched_barrier(0);
     });
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
     __builtin_amdgcn_s_barrier();
-    stage = stage1;
-  };
-  for (uint32_t c = 0; c < n_chunks; c += 2) {  // K is a multiple of 64: chunks come in pairs
-    iteration(kSet0, c);
-    iteration(kSet1, c + 1);
   }
-  // (the reads into opa after the last chunk fetched a stage nobody wrote: discarded)
 
   // ---- epilogue: per wave one head x 128 tokens ------------------------------------
   const uint32_t hh = 2 * tn + wn;
@@ -255,7 +256,7 @@ __global__ __launch_bounds__(kProjThreads) void project_kernel(ProjectKernelArgs
       for (int i = 0; i < 16; ++i) ext[set][i] = u32x2{one_zero, one_zero};
     }
   };
-  fetch_ext(kSet0, 0);
+  fetch_ext(std::integral_constant<int, 0>{}, 0);
   static_for<4>([&](auto mb_) {
     constexpr int mb = decltype(mb_)::value;
     constexpr int set = mb & 1;
@@ -343,7 +344,7 @@ hipError_t launch_project(const ProjectArgs& a, hipStream_t stream) {
   p.max_start = a.max_start;
   p.finalize0 = a.finalize0;
   p.eps = a.eps;
-  if (a.ws && a.counters && a.rows <= kSmallRowsMax)
+  if (a.ws && a.counters && small_kernel_takes(a.rows, a.K))
     return launch_project_small(p, a.ws, a.counters, a.dtype, a.residual != nullptr, stream);
   const uint32_t blocks = p.tiles_m * p.tiles_n;
   auto go = [&](auto kernel) {
