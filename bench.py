@@ -398,6 +398,67 @@ def bench_step_projections(batch, steps, warmup, hidden=2048, hq=32, hkv=4, copi
             "o_ms": o_ms, "o_kernel_ms": per[0], "o_bytes": o_bytes}
 
 
+def bench_layer_step(layers, batch, length, steps, warmup, hidden=2048, hq=32, hkv=4):
+    """The attention block of every layer for one new token per sequence: fused Q/K/V projection
+    (norm + rotation, K/V written into the cache), attention over the cache, output projection +
+    residual; every layer has its own weights and cache; positions advance on the device.
+    Issued launch by launch and replayed from a graph recorded once through the library."""
+    import torch
+
+    import ellm_amd
+
+    dt = torch.float16
+    cap = length + 2 * (steps + warmup) + 8
+    scale = 1.0 / D ** 0.5
+    stream = torch.cuda.Stream()
+    cache = ellm_amd.KVCache(layers, batch, hkv, cap, ellm_amd.DTYPE_F16)
+    j = torch.arange(D // 2, device="cuda", dtype=torch.float64)
+    ang = torch.arange(cap, device="cuda", dtype=torch.float64)[:, None] * (1.0e6 ** (-2.0 * j / D))[None, :]
+    rope = torch.stack((torch.cos(ang), torch.sin(ang)), dim=-1).reshape(cap, D).to(dt)
+    x = [_dev_normal((1, batch, hidden), dt, 501), torch.zeros((1, batch, hidden), dtype=dt, device="cuda")]
+    q = torch.zeros((1, batch, hq, D), dtype=dt, device="cuda")
+    att = torch.zeros_like(q)
+    ops, keep = [], []
+    for layer in range(layers):
+        kt, vt = cache.layer_tensors(layer, dt)
+        kt.normal_()
+        vt.normal_()
+        _, _, strides = cache.layer(layer)
+        w = [_dev_normal((h * D, hidden), dt, 600 + 4 * layer + i, scale=hidden ** -0.5) for i, h in enumerate((hq, hkv, hkv))]
+        wo = _dev_normal((hidden, hq * D), dt, 603 + 4 * layer, scale=(hq * D) ** -0.5)
+        keep.append((w, wo))
+        src, dst = x[layer & 1], x[1 - (layer & 1)]
+        ops.append((ellm_amd.MatMul3(src, w[0], q, w[1], kt, w[2], vt, rope, D, batch, hq, hkv, strides, cap),
+                    ellm_amd.Attention(q, kt, vt, att, batch, hq, hkv, D, strides, scale,
+                                       sequence_capacity=cap, max_position_interval=1),
+                    ellm_amd.MatMulAdd(att.view(1, batch, hq * D), wo, src, dst)))
+    pos = torch.full((batch,), length - 1, dtype=torch.int32, device="cuda")
+    torch.cuda.synchronize()
+
+    def step(_=None):
+        for qkv, attn, oproj in ops:
+            qkv.run_ragged(pos, cap - 1, batch)
+            attn.run_ragged(pos, cap - 1, batch)
+            oproj.run(0, 1, batch)
+        ellm_amd.positions_advance(pos, 1)
+
+    with torch.cuda.stream(stream):
+        _, eager_ms = _time_steps(step, steps, warmup)
+        pos.fill_(length - 1)
+        stream.synchronize()
+        with ellm_amd.StepGraph(stream) as graph:
+            step()
+        _, graph_ms = _time_steps(lambda _i: graph.launch(), steps, warmup)
+    graph.close()
+    for group in ops:
+        for op in group:
+            op.close()
+    cache.close()
+    kv_bytes = layers * (2 * batch * hkv * length * D * 2)
+    w_bytes = layers * ((hq + 2 * hkv) * D * hidden * 2 + hidden * hq * D * 2)
+    return {"eager_ms": eager_ms, "graph_ms": graph_ms, "kv_bytes": kv_bytes, "w_bytes": w_bytes}
+
+
 def cpu_baseline_decode(batch, length, hq=32, hkv=4, budget_s=20.0):
     """The CPU oracle on the full single-token workload (all host cores)."""
     import numpy as np
@@ -431,7 +492,7 @@ def main():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--skip-cpu", action="store_true")
-    ap.add_argument("--only", default="", help="decode | prefill | decode128k | chunk | mixed | mixed48 | kvwrite | tokenstep | qkv | oproj | stepproj")
+    ap.add_argument("--only", default="", help="decode | prefill | decode128k | chunk | mixed | mixed48 | kvwrite | tokenstep | layerstep | qkv | oproj | stepproj")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="first run one plain 256 MiB device copy (a known-traffic dispatch "
                          "for scaling rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE readings)")
@@ -594,6 +655,20 @@ def main():
                          "peak": HBM_PEAK_GBS, "unit": "GB/s",
                          "frac": round(sp["qkv_bytes"] / (sp["qkv_kernel_ms"] * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
                          "traffic": None},
+        })
+
+    if args.only in ("", "layerstep"):
+        ls_steps = min(args.steps, 20)
+        ls = bench_layer_step(48, 16, 8192, ls_steps, min(args.warmup, 3))
+        also.append({
+            "workload": "attention blocks of a 48-layer single-token step, 16 seq x 8192 cached tokens: per layer "
+                        "fused Q/K/V projection (K/V written into the cache) + attention + output projection "
+                        "with residual, own weights and cache per layer, positions on the device; 145 launches "
+                        "issued one by one vs one recorded graph",
+            "metric": "attention-block ms per token step", "value": round(ls["graph_ms"], 4), "unit": "ms",
+            "eager_ms": round(ls["eager_ms"], 4), "graph_ms": round(ls["graph_ms"], 4), "steps": ls_steps,
+            "cache_gb_per_step": round(ls["kv_bytes"] / 1e9, 2), "weight_gb_per_step": round(ls["w_bytes"] / 1e9, 2),
+            "gbs": round((ls["kv_bytes"] + ls["w_bytes"]) / (ls["graph_ms"] * 1e-3) / 1e9, 1),
         })
 
     cpu = None

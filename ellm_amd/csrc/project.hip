@@ -348,8 +348,10 @@ hipError_t launch_project(const ProjectArgs& a, hipStream_t stream) {
     return launch_project_small(p, a.ws, a.counters, a.dtype, a.residual != nullptr, stream);
   const uint32_t blocks = p.tiles_m * p.tiles_n;
   auto go = [&](auto kernel) {
-    hipError_t e = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                       kProjLdsBytes);
+    // (once per kernel and process, not per launch: a launch may be recorded into a graph)
+    static const hipError_t attr = hipFuncSetAttribute(
+        (const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, kProjLdsBytes);
+    const hipError_t e = attr;
     if (e != hipSuccess) return e;
     hipLaunchKernelGGL(kernel, dim3(blocks), dim3(kProjThreads), kProjLdsBytes, stream, p);
     return hipGetLastError();

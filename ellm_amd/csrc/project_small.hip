@@ -2,9 +2,9 @@
 // weights are read exactly once and the kernel is bound by that stream (HBM), not by
 // MFMA.  Same arithmetic and epilogue as the tile kernel of project.hip.
 //
-// A workgroup owns 16 output columns (one 16x16x32 MFMA block row) and all of K: 16
-// whole weight rows, contiguous in memory, so the stream of a workgroup stays inside a
-// few DRAM pages.  Its waves split K, 256 elements a wave and round; a lane fetches its
+// A workgroup owns 16 or 32 output columns (one or two 16x16x32 MFMA block rows, which
+// share the token operand) and all of K: whole weight rows, contiguous in memory, so the
+// stream of a workgroup stays inside a few DRAM pages.  Its waves split K, 256 elements a wave and round; a lane fetches its
 // MFMA operands straight from memory in operand layout (row = lane % 16, eight
 // consecutive K elements at 8 * (lane / 16)), every weight byte is fetched by exactly one
 // lane, all fetches of a round are issued before the first is used, nothing of the
@@ -13,8 +13,8 @@
 // token.  The waves' sums meet in LDS.
 // Columns that are not normalised (value heads, the output projection) are finished by
 // their own workgroup.  A normalised head needs the sum of squares over its 128 columns,
-// i.e. over eight workgroups: each leaves its 16 columns in a workspace (device-coherent
-// stores) and counts itself in; the last of the eight to arrive reads the head back,
+// i.e. over four or eight workgroups: each leaves its columns in a workspace (device-coherent
+// stores) and counts itself in; the last of them to arrive reads the head back,
 // normalises, rotates and stores it.  The counters reset themselves.
 #include "project_common.hpp"
 
@@ -24,8 +24,6 @@ namespace {
 
 constexpr int kStepsPerRound = 8;            // 32-element K steps a wave has in flight: 256 elements
 constexpr int kRoundK = 32 * kStepsPerRound;
-constexpr int kGroupCols = 16;               // output columns per workgroup
-constexpr int kGroupsPerHead = kHeadDim / kGroupCols;
 
 __device__ __forceinline__ void store_coherent(float* p, float v) {
   __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -39,12 +37,14 @@ __device__ __forceinline__ f32x4 load_coherent128_nowait(const float* p) {
 }
 __device__ __forceinline__ void wait_vm_done() { __builtin_amdgcn_s_waitcnt(0x0F70); }
 
-// NTB: 16-token blocks (1 or 2).  blockDim.x = 64 * waves, waves = min(16, K / 256).
-template <typename S, int MODE, int NTB>
+// NTB: 16-token blocks (1 or 2); NB: 16-column MFMA blocks per workgroup (1 or 2).
+// blockDim.x = 64 * waves, waves = min(16, K / 256).
+template <typename S, int MODE, int NTB, int NB>
 __global__ __launch_bounds__(1024) void project_small_kernel(ProjectKernelArgs p, float* ws,
                                                              uint32_t* counters) {
   using M = Mfma<S>;
-  extern __shared__ __attribute__((aligned(16))) float sums[];  // [wave][NTB][16 tokens][16 columns]
+  constexpr int kColBlocks = NB, kGroupCols = 16 * NB, kGroupsPerHead = kHeadDim / kGroupCols;
+  extern __shared__ __attribute__((aligned(16))) float sums[];  // [wave][NTB][16 tokens][kGroupCols]
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, n_waves = blockDim.x >> 6;
   const int i16 = lane & 15, q4 = lane >> 4;
   const uint32_t K = p.K;
@@ -54,16 +54,21 @@ __global__ __launch_bounds__(1024) void project_small_kernel(ProjectKernelArgs p
   constexpr int kRowsCap = 16 * NTB;
 
   const uint16_t* wrow = p.w[seg] + ((size_t)hs * kHeadDim + kGroupCols * cg + i16) * K + 8 * q4;
+  const size_t wblock = (size_t)16 * K;  // elements between the rows of consecutive column blocks
   const __amdgpu_buffer_rsrc_t x_rsrc =
       __builtin_amdgcn_make_buffer_rsrc((void*)uniform64(p.x), 0, p.rows * K * 2, kBufFlags);
-  f32x4 acc[NTB];
+  f32x4 acc[kColBlocks][NTB];
 #pragma unroll
-  for (int tb = 0; tb < NTB; ++tb) acc[tb] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+  for (int nb = 0; nb < kColBlocks; ++nb)
+#pragma unroll
+    for (int tb = 0; tb < NTB; ++tb) acc[nb][tb] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
   for (uint32_t k0 = wave * kRoundK; k0 < K; k0 += n_waves * kRoundK) {
-    u32x4 wreg[kStepsPerRound], xreg[NTB][kStepsPerRound];  // token rows past the last read as zero
+    u32x4 wreg[kColBlocks][kStepsPerRound], xreg[NTB][kStepsPerRound];  // token rows past the last read as zero
 #pragma unroll
-    for (int s = 0; s < kStepsPerRound; ++s)
-      wreg[s] = __builtin_nontemporal_load((const u32x4*)(wrow + k0 + 32 * s));
+    for (int nb = 0; nb < kColBlocks; ++nb)
+#pragma unroll
+      for (int s = 0; s < kStepsPerRound; ++s)
+        wreg[nb][s] = __builtin_nontemporal_load((const u32x4*)(wrow + nb * wblock + k0 + 32 * s));
 #pragma unroll
     for (int tb = 0; tb < NTB; ++tb)
 #pragma unroll
@@ -74,19 +79,24 @@ __global__ __launch_bounds__(1024) void project_small_kernel(ProjectKernelArgs p
 #pragma unroll
     for (int s = 0; s < kStepsPerRound; ++s)
 #pragma unroll
-      for (int tb = 0; tb < NTB; ++tb) acc[tb] = M::m16x16x32(wreg[s], xreg[tb][s], acc[tb]);
-  }
-  // lane (token i16, columns 4 q4 .. 4 q4 + 3)
+      for (int nb = 0; nb < kColBlocks; ++nb)
 #pragma unroll
-  for (int tb = 0; tb < NTB; ++tb)
-    *(f32x4*)(sums + ((wave * NTB + tb) * 16 + i16) * kGroupCols + 4 * q4) = acc[tb];
+        for (int tb = 0; tb < NTB; ++tb) acc[nb][tb] = M::m16x16x32(wreg[nb][s], xreg[tb][s], acc[nb][tb]);
+  }
+  // lane (token i16, columns 16 nb + 4 q4 .. + 3)
+#pragma unroll
+  for (int nb = 0; nb < kColBlocks; ++nb)
+#pragma unroll
+    for (int tb = 0; tb < NTB; ++tb)
+      *(f32x4*)(sums + ((wave * NTB + tb) * 16 + i16) * kGroupCols + 16 * nb + 4 * q4) = acc[nb][tb];
   __syncthreads();
 
-  // threads 0 .. 64 NTB - 1: token tid / 4, columns 4 (tid % 4) .. + 3 of the group
+  // threads 0 .. 4 kGroupCols NTB - 1: token tid / (kGroupCols / 4), four columns of the group
   const bool finalize = MODE == kModeQkv && ((seg == 1) || (seg == 0 && p.finalize0));
   uint16_t* const dst = (seg == 0) ? p.out0 : (seg == 1 ? p.k_out : p.v_out);
-  if (tid < 64 * NTB) {
-    const uint32_t R = tid >> 2, c4 = tid & 3;
+  constexpr int kQuads = kGroupCols / 4;
+  if (tid < 16 * kQuads * NTB) {
+    const uint32_t R = tid / kQuads, c4 = tid % kQuads;
     f32x4 v = {0.0f, 0.0f, 0.0f, 0.0f};
     for (int w = 0; w < n_waves; ++w)
       v += *(const f32x4*)(sums + (w * kRowsCap + R) * kGroupCols + 4 * c4);
@@ -137,7 +147,9 @@ __global__ __launch_bounds__(1024) void project_small_kernel(ProjectKernelArgs p
   if (tid >= 256 * NTB) return;
   const uint32_t R = tid >> 4;
   const int c8 = tid & 15;
-  const float* src = ws + (((size_t)hh * kGroupsPerHead + (c8 >> 1)) * kRowsCap + R) * kGroupCols + 8 * (c8 & 1);
+  constexpr int kOctets = kGroupCols / 8;
+  const float* src =
+      ws + (((size_t)hh * kGroupsPerHead + c8 / kOctets) * kRowsCap + R) * kGroupCols + 8 * (c8 % kOctets);
   const f32x4 lo = load_coherent128_nowait(src), hi = load_coherent128_nowait(src + 4);
   const uint32_t t = R / p.batch_pitch, b = R % p.batch_pitch;
   const bool live = R < p.rows && b < p.batch;
@@ -172,20 +184,32 @@ __global__ __launch_bounds__(1024) void project_small_kernel(ProjectKernelArgs p
   }
 }
 
+// Two column blocks a workgroup halve the re-reads of the token rows (every workgroup
+// reads all of them) but also the number of workgroups; one compute unit streams at most
+// ~55 GB/s, so narrow outputs keep one block to have enough of them.
+template <typename S, int MODE, int NTB, int NB>
+hipError_t launch_one(const ProjectKernelArgs& p, float* ws, uint32_t* counters, uint32_t heads, uint32_t waves,
+                      hipStream_t stream) {
+  const dim3 grid(heads * (kHeadDim / (16 * NB))), block(64 * waves);
+  hipLaunchKernelGGL((project_small_kernel<S, MODE, NTB, NB>), grid, block, waves * NTB * 64 * 16 * NB, stream, p,
+                     ws, counters);
+  return hipGetLastError();
+}
+
 template <typename S, int MODE>
 hipError_t launch_blocks(const ProjectKernelArgs& p, float* ws, uint32_t* counters, uint32_t heads,
                          hipStream_t stream) {
   uint32_t waves = p.K / kRoundK;
   if (waves > 16) waves = 16;
-  const dim3 grid(heads * kGroupsPerHead), block(64 * waves);
+  const bool wide = heads * kHeadDim >= 4096;
   if (p.rows <= 16) {
     if (waves < 4) return hipErrorInvalidValue;  // the finishing step wants 256 threads
-    hipLaunchKernelGGL((project_small_kernel<S, MODE, 1>), grid, block, waves * 1 * 1024, stream, p, ws, counters);
-  } else {
-    if (waves < 8) return hipErrorInvalidValue;  // ... 512 threads
-    hipLaunchKernelGGL((project_small_kernel<S, MODE, 2>), grid, block, waves * 2 * 1024, stream, p, ws, counters);
+    return wide ? launch_one<S, MODE, 1, 2>(p, ws, counters, heads, waves, stream)
+                : launch_one<S, MODE, 1, 1>(p, ws, counters, heads, waves, stream);
   }
-  return hipGetLastError();
+  if (waves < 8) return hipErrorInvalidValue;  // ... 512 threads
+  return wide ? launch_one<S, MODE, 2, 2>(p, ws, counters, heads, waves, stream)
+              : launch_one<S, MODE, 2, 1>(p, ws, counters, heads, waves, stream);
 }
 
 }  // namespace

@@ -1,0 +1,117 @@
+"""One attention layer of a single-token step, end to end through the C ABI: fused Q/K/V
+projection (writes the cache in place) -> attention over the cache -> output projection +
+residual -> positions advanced on the device; launched eagerly and replayed from a graph
+recorded through the library.  Every stage is checked against the oracle run on that
+stage's own inputs as the GPU produced them, with the stage's tolerance."""
+import numpy as np
+import pytest
+
+import oracle_lib as orc
+from gpu_util import D, compare, compare_ulps, rand_storage, to_dev, to_host, torch_dtype
+
+pytestmark = pytest.mark.gpu
+
+
+def _rope_table(positions, dtype, theta=1.0e6):
+    jj = np.arange(D // 2, dtype=np.float64)
+    ang = np.arange(positions, dtype=np.float64)[:, None] * theta ** (-2.0 * jj / D)[None, :]
+    t = np.empty((positions, D), dtype=np.float32)
+    t[:, 0::2], t[:, 1::2] = np.cos(ang), np.sin(ang)
+    return orc.to_storage(t, dtype)
+
+
+def test_layer_step_eager_graph_and_oracle():
+    import torch
+
+    import ellm_amd
+
+    dtype = orc.F16
+    b, hq, hkv, cap, hidden = 5, 8, 2, 256, 512
+    steps = 3
+    start = np.array([17, 0, 200, 64, 99], dtype=np.int32)
+    scale = 1.0 / np.sqrt(D)
+    rope = _rope_table(cap, dtype)
+    wq = rand_storage((hq * D, hidden), 1, dtype, scale=hidden ** -0.5)
+    wk = rand_storage((hkv * D, hidden), 2, dtype, scale=hidden ** -0.5)
+    wv = rand_storage((hkv * D, hidden), 3, dtype, scale=hidden ** -0.5)
+    wo = rand_storage((hidden, hq * D), 4, dtype, scale=(hq * D) ** -0.5)
+    k0 = rand_storage((b, hkv, cap, D), 5, dtype)
+    v0 = rand_storage((b, hkv, cap, D), 6, dtype)
+    xs = rand_storage((steps, 1, b, hidden), 7, dtype)
+
+    def run(use_graph):
+        stream = torch.cuda.Stream()
+        cache = ellm_amd.KVCache(1, b, hkv, cap, ellm_amd.DTYPE_F16)
+        kt, vt = cache.layer_tensors(0, torch_dtype(dtype))
+        kt.copy_(to_dev(k0, dtype))
+        vt.copy_(to_dev(v0, dtype))
+        _, _, strides = cache.layer(0)
+        x = torch.zeros((1, b, hidden), dtype=torch.float16, device="cuda")
+        q = torch.zeros((1, b, hq, D), dtype=torch.float16, device="cuda")
+        att = torch.zeros_like(q)
+        out = torch.zeros_like(x)
+        dev = [to_dev(a, dtype) for a in (wq, wk, wv, wo, rope)]
+        qkv = ellm_amd.MatMul3(x, dev[0], q, dev[1], kt, dev[2], vt, dev[4], D, b, hq, hkv, strides, cap)
+        attn = ellm_amd.Attention(q, kt, vt, att, b, hq, hkv, D, strides, scale, sequence_capacity=cap,
+                                  max_position_interval=1)
+        oproj = ellm_amd.MatMulAdd(att.view(1, b, hq * D), dev[3], x, out)   # residual = the layer input
+        pos = torch.from_numpy(start.copy()).cuda()
+        max_pos = int(start.max()) + steps
+        results, graph = [], None
+        with torch.cuda.stream(stream):
+            def step():
+                qkv.run_ragged(pos, max_pos, b)
+                attn.run_ragged(pos, max_pos, b)
+                oproj.run(0, 1, b)
+                ellm_amd.positions_advance(pos, 1)
+
+            for s in range(steps):
+                x.copy_(to_dev(xs[s], dtype))
+                stream.synchronize()
+                if not use_graph:
+                    step()
+                else:
+                    if graph is None:
+                        with ellm_amd.StepGraph(stream) as graph:
+                            step()
+                    graph.launch()
+                stream.synchronize()
+                results.append(tuple(to_host(t, dtype).copy() for t in (q, att, out)) + (to_host(kt, dtype).copy(),
+                                                                                         to_host(vt, dtype).copy()))
+                _ = float(out.float().sum())      # eager work between replays
+        final_pos = pos.cpu().numpy()
+        if graph is not None:
+            graph.close()
+        for op in (qkv, attn, oproj):
+            op.close()
+        cache.close()
+        return results, final_pos
+
+    eager, pos_e = run(False)
+    replay, pos_g = run(True)
+    assert np.array_equal(pos_e, start + steps) and np.array_equal(pos_g, start + steps)
+    for s in range(steps):
+        for a, c in zip(eager[s], replay[s]):
+            assert np.array_equal(a, c), s                     # same kernels, same bits
+
+    # oracle, stage by stage, on the inputs the GPU stages saw
+    kc, vc = k0.copy(), v0.copy()
+    for s in range(steps):
+        gq, gatt, gout, gk, gv = replay[s]
+        positions = (start + s).astype(np.uint32)
+        oq = np.zeros((1, b, hq, D), dtype=np.uint16)
+        assert orc.matmul3(xs[s], wq, wk, wv, oq, kc, vc, rope, (hkv * cap * D, cap * D, D, 1), cap, 0, 1, dtype,
+                           positions=positions) == 0
+        assert compare_ulps(gq, orc.from_storage(oq, dtype), dtype)["ok"]
+        assert compare_ulps(gk, orc.from_storage(kc, dtype), dtype)["ok"]
+        assert compare_ulps(gv, orc.from_storage(vc, dtype), dtype)["ok"]
+        # attention on the GPU's own q and cache (stage tolerance, not accumulated)
+        sq, sk, sv = (orc.to_storage(a, dtype) for a in (gq, gk, gv))
+        want_att, _ = orc.attention(sq, sk, sv, scale, dtype, positions=positions)
+        assert compare(gatt, orc.from_storage(want_att, dtype), dtype)["ok"]
+        # output projection on the GPU's attention rows
+        satt = orc.to_storage(gatt.reshape(1, b, hq * D), dtype)
+        want_out = orc.matmul_add(satt, wo, xs[s], dtype)
+        assert compare_ulps(gout, orc.from_storage(want_out, dtype), dtype)["ok"]
+        # carry the GPU's cache forward so that later steps stay stage-local
+        kc, vc = sk.copy(), sv.copy()
