@@ -37,9 +37,15 @@ __device__ __forceinline__ f32x4 load_coherent128_nowait(const float* p) {
 }
 __device__ __forceinline__ void wait_vm_done() { __builtin_amdgcn_s_waitcnt(0x0F70); }
 
+typedef __attribute__((address_space(3))) u32x4 LdsVec4;
+
 // NTB: 16-token blocks (1 or 2); NB: 16-column MFMA blocks per workgroup (1 or 2).
 // blockDim.x = 64 * waves, waves = min(16, K / 256).
-template <typename S, int MODE, int NTB, int NB>
+// VIA_LDS (waves == K / 256 and the rows fit): the workgroup's weight rows, one contiguous
+// region of memory, are fetched in 1 KB pieces (a wave instruction = 1 KB of one row) and
+// handed to the MFMA operand layout through LDS; fetching them in operand layout directly
+// (16 rows x 64 B an instruction) makes the same stream a third slower.
+template <typename S, int MODE, int NTB, int NB, bool VIA_LDS>
 __global__ __launch_bounds__(1024) void project_small_kernel(ProjectKernelArgs p, float* ws,
                                                              uint32_t* counters) {
   using M = Mfma<S>;
@@ -62,27 +68,66 @@ __global__ __launch_bounds__(1024) void project_small_kernel(ProjectKernelArgs p
   for (int nb = 0; nb < kColBlocks; ++nb)
 #pragma unroll
     for (int tb = 0; tb < NTB; ++tb) acc[nb][tb] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
-  for (uint32_t k0 = wave * kRoundK; k0 < K; k0 += n_waves * kRoundK) {
-    u32x4 wreg[kColBlocks][kStepsPerRound], xreg[NTB][kStepsPerRound];  // token rows past the last read as zero
+  if constexpr (VIA_LDS) {
+    const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) float*)sums;
+    const uint8_t* wg_rows = (const uint8_t*)(p.w[seg] + ((size_t)hs * kHeadDim + kGroupCols * cg) * K);
+    const uint32_t row_bytes = 2 * K, pitch = row_bytes + 16;  // + 16: the 16 rows of an operand read tile the banks
+    constexpr int kPieces = 8 * NB;                            // 1 KB pieces per wave
+    const uint32_t k0 = wave * kRoundK;
+    u32x4 stg[kPieces], xreg[NTB][kStepsPerRound];
 #pragma unroll
-    for (int nb = 0; nb < kColBlocks; ++nb)
-#pragma unroll
-      for (int s = 0; s < kStepsPerRound; ++s)
-        wreg[nb][s] = __builtin_nontemporal_load((const u32x4*)(wrow + nb * wblock + k0 + 32 * s));
+    for (int u = 0; u < kPieces; ++u)
+      stg[u] = __builtin_nontemporal_load((const u32x4*)(wg_rows + (size_t)(wave * kPieces + u) * 1024 + lane * 16));
 #pragma unroll
     for (int tb = 0; tb < NTB; ++tb)
 #pragma unroll
       for (int s = 0; s < kStepsPerRound; ++s)
         xreg[tb][s] = __builtin_amdgcn_raw_buffer_load_b128(
             x_rsrc, ((16 * tb + i16) * K + k0 + 8 * q4 + 32 * s) * 2, 0, 0);
-    __builtin_amdgcn_sched_barrier(0);  // every fetch of the round is on its way before the first use
+    __builtin_amdgcn_sched_barrier(0);  // every fetch is on its way before the first use
+#pragma unroll
+    for (int u = 0; u < kPieces; ++u) {
+      const uint32_t off = (wave * kPieces + u) * 1024 + lane * 16;
+      const uint32_t row = off / row_bytes;
+      *(LdsVec4*)(lds0 + row * pitch + (off - row * row_bytes)) = stg[u];
+    }
+    __syncthreads();
+    u32x4 wreg[kColBlocks][kStepsPerRound];
+#pragma unroll
+    for (int nb = 0; nb < kColBlocks; ++nb)
+#pragma unroll
+      for (int s = 0; s < kStepsPerRound; ++s)
+        wreg[nb][s] = *(const LdsVec4*)(lds0 + (16 * nb + i16) * pitch + (k0 + 32 * s + 8 * q4) * 2);
 #pragma unroll
     for (int s = 0; s < kStepsPerRound; ++s)
 #pragma unroll
       for (int nb = 0; nb < kColBlocks; ++nb)
 #pragma unroll
         for (int tb = 0; tb < NTB; ++tb) acc[nb][tb] = M::m16x16x32(wreg[nb][s], xreg[tb][s], acc[nb][tb]);
-  }
+    __syncthreads();  // the sums below reuse the rows' LDS
+  } else {
+  for (uint32_t k0 = wave * kRoundK; k0 < K; k0 += n_waves * kRoundK) {
+      u32x4 wreg[kColBlocks][kStepsPerRound], xreg[NTB][kStepsPerRound];  // token rows past the last read as zero
+  #pragma unroll
+      for (int nb = 0; nb < kColBlocks; ++nb)
+  #pragma unroll
+        for (int s = 0; s < kStepsPerRound; ++s)
+          wreg[nb][s] = __builtin_nontemporal_load((const u32x4*)(wrow + nb * wblock + k0 + 32 * s));
+  #pragma unroll
+      for (int tb = 0; tb < NTB; ++tb)
+  #pragma unroll
+        for (int s = 0; s < kStepsPerRound; ++s)
+          xreg[tb][s] = __builtin_amdgcn_raw_buffer_load_b128(
+              x_rsrc, ((16 * tb + i16) * K + k0 + 8 * q4 + 32 * s) * 2, 0, 0);
+      __builtin_amdgcn_sched_barrier(0);  // every fetch of the round is on its way before the first use
+  #pragma unroll
+      for (int s = 0; s < kStepsPerRound; ++s)
+  #pragma unroll
+        for (int nb = 0; nb < kColBlocks; ++nb)
+  #pragma unroll
+          for (int tb = 0; tb < NTB; ++tb) acc[nb][tb] = M::m16x16x32(wreg[nb][s], xreg[tb][s], acc[nb][tb]);
+    }
+}
   // lane (token i16, columns 16 nb + 4 q4 .. + 3)
 #pragma unroll
   for (int nb = 0; nb < kColBlocks; ++nb)
@@ -187,12 +232,26 @@ __global__ __launch_bounds__(1024) void project_small_kernel(ProjectKernelArgs p
 // Two column blocks a workgroup halve the re-reads of the token rows (every workgroup
 // reads all of them) but also the number of workgroups; one compute unit streams at most
 // ~55 GB/s, so narrow outputs keep one block to have enough of them.
+constexpr uint32_t kLdsBudget = 150 * 1024;
+
 template <typename S, int MODE, int NTB, int NB>
 hipError_t launch_one(const ProjectKernelArgs& p, float* ws, uint32_t* counters, uint32_t heads, uint32_t waves,
                       hipStream_t stream) {
   const dim3 grid(heads * (kHeadDim / (16 * NB))), block(64 * waves);
-  hipLaunchKernelGGL((project_small_kernel<S, MODE, NTB, NB>), grid, block, waves * NTB * 64 * 16 * NB, stream, p,
-                     ws, counters);
+  const uint32_t sums_bytes = waves * NTB * 64 * 16 * NB;
+  const uint32_t rows_bytes = 16 * NB * (2 * p.K + 16);
+  if (waves * kRoundK == p.K && rows_bytes <= kLdsBudget) {
+    auto kernel = project_small_kernel<S, MODE, NTB, NB, true>;
+    const uint32_t lds = rows_bytes > sums_bytes ? rows_bytes : sums_bytes;
+    // (once per kernel and process, not per launch: a launch may be recorded into a graph)
+    static const hipError_t attr = hipFuncSetAttribute(
+        (const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBudget);
+    if (attr != hipSuccess) return attr;
+    hipLaunchKernelGGL(kernel, grid, block, lds, stream, p, ws, counters);
+  } else {
+    hipLaunchKernelGGL((project_small_kernel<S, MODE, NTB, NB, false>), grid, block, sums_bytes, stream, p, ws,
+                       counters);
+  }
   return hipGetLastError();
 }
 
@@ -201,7 +260,8 @@ hipError_t launch_blocks(const ProjectKernelArgs& p, float* ws, uint32_t* counte
                          hipStream_t stream) {
   uint32_t waves = p.K / kRoundK;
   if (waves > 16) waves = 16;
-  const bool wide = heads * kHeadDim >= 4096;
+  // two column blocks: enough columns for >= 128 workgroups, and (where the rows go through LDS) room for 32 rows
+  const bool wide = heads * kHeadDim >= 4096 && (waves * kRoundK != p.K || 32 * (2 * p.K + 16) <= kLdsBudget);
   if (p.rows <= 16) {
     if (waves < 4) return hipErrorInvalidValue;  // the finishing step wants 256 threads
     return wide ? launch_one<S, MODE, 1, 2>(p, ws, counters, heads, waves, stream)

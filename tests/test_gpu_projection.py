@@ -81,6 +81,11 @@ CASES = [
     (1, 16, 16, 2048, 32, 4, 256, 100, orc.F16),   # the single-token step of the benchmark model
     (513, 1, 1, 192, 2, 2, 1024, 3, orc.BF16),     # three token tiles, bfloat16
     (40, 3, 2, 128, 4, 4, 64, 0, orc.BF16),
+    # few rows (the weight-streaming kernel): two token blocks x two column blocks, rows through LDS
+    (2, 16, 12, 2048, 32, 4, 64, 5, orc.F16),
+    (1, 16, 16, 1024, 4, 2, 64, 9, orc.BF16),      # four waves, one column block
+    (1, 8, 8, 8192, 2, 1, 32, 3, orc.F16),         # two rounds of K per wave, operands fetched directly
+    (2, 12, 12, 4096, 34, 2, 32, 1, orc.F16),      # wide output but rows too long for two column blocks in LDS
 ]
 
 
@@ -132,6 +137,8 @@ def test_matmul3_in_the_reference_state_layout_and_table_indexing():
     (3, 5, 4, 64, 384, orc.BF16),
     (1, 16, 16, 4096, 2048, orc.F16),              # the output projection of the benchmark model, one token
     (257, 2, 2, 128, 128, orc.F16),
+    (1, 8, 8, 2048, 256, orc.BF16),                # few rows, bfloat16
+    (2, 16, 10, 2048, 4096, orc.F16),              # few rows, two token blocks, wide output
 ])
 def test_matmul_add_against_the_oracle(interval, pitch, batch, k, n, dtype):
     import torch
