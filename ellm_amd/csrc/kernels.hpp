@@ -111,6 +111,8 @@ struct ProjectArgs {
 hipError_t launch_project(const ProjectArgs& a, hipStream_t stream);
 // Few-rows kernel: rows it handles at most, floats of partial sums and counters it needs.
 size_t project_workspace_floats(uint32_t heads, uint32_t K);
+// Per-device set-up of the projection kernels (LDS limits); call with the device current.
+hipError_t project_prepare();
 
 // Records the message ellm_last_error_string() returns on this thread; returns status.
 int set_error(int status, const char* fmt, ...) __attribute__((format(printf, 2, 3)));

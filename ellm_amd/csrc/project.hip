@@ -348,17 +348,24 @@ hipError_t launch_project(const ProjectArgs& a, hipStream_t stream) {
     return launch_project_small(p, a.ws, a.counters, a.dtype, a.residual != nullptr, stream);
   const uint32_t blocks = p.tiles_m * p.tiles_n;
   auto go = [&](auto kernel) {
-    // (once per kernel and process, not per launch: a launch may be recorded into a graph)
-    static const hipError_t attr = hipFuncSetAttribute(
-        (const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, kProjLdsBytes);
-    const hipError_t e = attr;
-    if (e != hipSuccess) return e;
     hipLaunchKernelGGL(kernel, dim3(blocks), dim3(kProjThreads), kProjLdsBytes, stream, p);
     return hipGetLastError();
   };
   if (a.residual)
     return a.dtype == 0 ? go(project_kernel<F16, kModeAdd>) : go(project_kernel<BF16, kModeAdd>);
   return a.dtype == 0 ? go(project_kernel<F16, kModeQkv>) : go(project_kernel<BF16, kModeQkv>);
+}
+
+// The kernels' LDS needs exceed the default limit; raised here, on the current device, when
+// a handle is created, not at launch (a launch may be recorded into a graph).
+hipError_t project_prepare() {
+  const void* kernels[] = {(const void*)project_kernel<F16, kModeQkv>, (const void*)project_kernel<BF16, kModeQkv>,
+                           (const void*)project_kernel<F16, kModeAdd>, (const void*)project_kernel<BF16, kModeAdd>};
+  for (const void* k : kernels) {
+    const hipError_t e = hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, kProjLdsBytes);
+    if (e != hipSuccess) return e;
+  }
+  return small_prepare();
 }
 
 size_t project_workspace_floats(uint32_t heads, uint32_t K) {

@@ -36,6 +36,8 @@ int alloc_small_workspace(uint32_t heads, uint32_t K, float** ws, uint32_t** cou
     (void)hipGetLastError();
     return ellm::set_error(ELLM_ERR_NO_DEVICE, "no HIP device visible");
   }
+  const hipError_t prep = ellm::project_prepare();
+  if (prep != hipSuccess) return ellm::set_error(ELLM_ERR_HIP, "projection kernels: %s", hipGetErrorString(prep));
   const size_t floats = ellm::project_workspace_floats(heads, K);
   if (floats * sizeof(float) > (size_t)64 << 20) return ELLM_OK;
   hipError_t e = hipMalloc((void**)ws, floats * sizeof(float));

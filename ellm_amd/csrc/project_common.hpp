@@ -51,6 +51,7 @@ constexpr int kModeAdd = 1;  // plain product plus a residual of the output's la
 
 // Streaming kernel for a few rows (project_small.hip).
 constexpr uint32_t kSmallRowsMax = 32;
+hipError_t small_prepare();
 bool small_kernel_takes(uint32_t rows, uint32_t K);
 size_t small_workspace_floats(uint32_t heads, uint32_t K);
 hipError_t launch_project_small(const ProjectKernelArgs& p, float* ws, uint32_t* counters, int dtype,

@@ -243,10 +243,6 @@ hipError_t launch_one(const ProjectKernelArgs& p, float* ws, uint32_t* counters,
   if (waves * kRoundK == p.K && rows_bytes <= kLdsBudget) {
     auto kernel = project_small_kernel<S, MODE, NTB, NB, true>;
     const uint32_t lds = rows_bytes > sums_bytes ? rows_bytes : sums_bytes;
-    // (once per kernel and process, not per launch: a launch may be recorded into a graph)
-    static const hipError_t attr = hipFuncSetAttribute(
-        (const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBudget);
-    if (attr != hipSuccess) return attr;
     hipLaunchKernelGGL(kernel, grid, block, lds, stream, p, ws, counters);
   } else {
     hipLaunchKernelGGL((project_small_kernel<S, MODE, NTB, NB, false>), grid, block, sums_bytes, stream, p, ws,
@@ -275,6 +271,27 @@ hipError_t launch_blocks(const ProjectKernelArgs& p, float* ws, uint32_t* counte
 }  // namespace
 
 namespace proj {
+
+template <typename S, int MODE>
+static hipError_t prepare_mode() {
+  const void* kernels[] = {(const void*)project_small_kernel<S, MODE, 1, 1, true>,
+                           (const void*)project_small_kernel<S, MODE, 1, 2, true>,
+                           (const void*)project_small_kernel<S, MODE, 2, 1, true>,
+                           (const void*)project_small_kernel<S, MODE, 2, 2, true>};
+  for (const void* k : kernels) {
+    const hipError_t e = hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBudget);
+    if (e != hipSuccess) return e;
+  }
+  return hipSuccess;
+}
+
+hipError_t small_prepare() {
+  hipError_t e = prepare_mode<F16, kModeQkv>();
+  if (e == hipSuccess) e = prepare_mode<BF16, kModeQkv>();
+  if (e == hipSuccess) e = prepare_mode<F16, kModeAdd>();
+  if (e == hipSuccess) e = prepare_mode<BF16, kModeAdd>();
+  return e;
+}
 
 bool small_kernel_takes(uint32_t rows, uint32_t K) {
   if (K % kRoundK != 0) return false;
