@@ -207,48 +207,74 @@ def bench_kv_write(n_tokens, steps, warmup, hkv=4, seqs=1):
             "kernel_gbs": alg_bytes / (kern_ms * 1e-3) / 1e9}
 
 
-def bench_mixed_step(layers, prefill_tokens, batch, lo, hi, steps, warmup, hq=32, hkv=4, seed=7):
-    """One step of the mixed configuration end to end: for each layer a prefill of
-    `prefill_tokens` tokens of one sequence and a single-token step over `batch` other
-    sequences with cache lengths U{lo..hi}, all launches on one stream.  The layers use the
-    same device buffers (a full set of 48 caches at this capacity does not fit; the work per
-    layer is the same and nothing stays in a cache between layers: one layer's K/V is 8.6 GB)."""
+def bench_mixed_step(layers, prefill_tokens, batch, lo, hi, steps, warmup, hidden=2048, hq=32, hkv=4, seed=7):
+    """One step of the mixed configuration end to end: for each layer the fused Q/K/V projection
+    (random-init weights of the layer, norm + rotation, K/V written into the caches) and the
+    attention of a `prefill_tokens`-token prefill of one sequence, and the same two for one new
+    token of `batch` other sequences with cache lengths U{lo..hi}; all launches on one stream.
+    Every layer has its own weights; the layers share the activations and the caches (a full
+    set of 48 caches at this capacity does not fit: one layer's K/V is 8.6 GB; the work per layer
+    is the same and nothing stays in a cache between layers)."""
     import numpy as np
     import torch
 
     import ellm_amd
 
+    dt = torch.float16
     rng = np.random.default_rng(seed)
     lengths = rng.integers(lo, hi + 1, size=batch)
     cap = int(hi)
     scale = 1.0 / D ** 0.5
-    k = torch.empty((batch, hkv, cap, D), dtype=torch.float16, device="cuda").normal_()
-    v = torch.empty((batch, hkv, cap, D), dtype=torch.float16, device="cuda").normal_()
-    q = _dev_normal((1, batch, hq, D), torch.float16, 301)
+    j = torch.arange(D // 2, device="cuda", dtype=torch.float64)
+    ang = torch.arange(cap, device="cuda", dtype=torch.float64)[:, None] * (1.0e6 ** (-2.0 * j / D))[None, :]
+    rope = torch.stack((torch.cos(ang), torch.sin(ang)), dim=-1).reshape(cap, D).to(dt)
+    del ang
+    # single-token side: `batch` sequences, caches at capacity `hi`
+    k = torch.empty((batch, hkv, cap, D), dtype=dt, device="cuda").normal_()
+    v = torch.empty((batch, hkv, cap, D), dtype=dt, device="cuda").normal_()
+    kv_strides = [hkv * cap * D, cap * D, D, 1]
+    x_dec = _dev_normal((1, batch, hidden), dt, 300)
+    q = torch.zeros((1, batch, hq, D), dtype=dt, device="cuda")
     out = torch.zeros_like(q)
     pos = torch.tensor((lengths - 1).astype(np.int32), dtype=torch.int32, device="cuda")
-    dec = ellm_amd.Attention(q, k, v, out, batch, hq, hkv, D, [hkv * cap * D, cap * D, D, 1], scale,
-                             sequence_capacity=cap, max_position_interval=1)
     max_pos = int(lengths.max() - 1)
-    pq = _dev_normal((prefill_tokens, 1, hq, D), torch.float16, 311)
-    pk = _dev_normal((1, hkv, prefill_tokens, D), torch.float16, 312)
-    pv = _dev_normal((1, hkv, prefill_tokens, D), torch.float16, 313)
+    dec = ellm_amd.Attention(q, k, v, out, batch, hq, hkv, D, kv_strides, scale,
+                             sequence_capacity=cap, max_position_interval=1)
+    # prefill side: one sequence
+    x_pre = _dev_normal((prefill_tokens, 1, hidden), dt, 310)
+    pq = torch.zeros((prefill_tokens, 1, hq, D), dtype=dt, device="cuda")
+    pk = torch.zeros((1, hkv, prefill_tokens, D), dtype=dt, device="cuda")
+    pv = torch.zeros_like(pk)
     pout = torch.zeros_like(pq)
-    pre = ellm_amd.Attention(pq, pk, pv, pout, 1, hq, hkv, D,
-                             [hkv * prefill_tokens * D, prefill_tokens * D, D, 1], scale,
+    p_strides = [hkv * prefill_tokens * D, prefill_tokens * D, D, 1]
+    pre = ellm_amd.Attention(pq, pk, pv, pout, 1, hq, hkv, D, p_strides, scale,
                              sequence_capacity=prefill_tokens, max_position_interval=prefill_tokens)
+    proj, keep = [], []
+    for layer in range(layers):
+        w = [_dev_normal((h * D, hidden), dt, 700 + 3 * layer + i, scale=hidden ** -0.5) for i, h in enumerate((hq, hkv, hkv))]
+        keep.append(w)
+        proj.append((ellm_amd.MatMul3(x_pre, w[0], pq, w[1], pk, w[2], pv, rope, D, 1, hq, hkv, p_strides,
+                                      prefill_tokens),
+                     ellm_amd.MatMul3(x_dec, w[0], q, w[1], k, w[2], v, rope, D, batch, hq, hkv, kv_strides, cap)))
 
     def step(_):
-        for _layer in range(layers):
+        for qkv_pre, qkv_dec in proj:
+            qkv_pre.run(0, prefill_tokens, 1)
             pre.run(0, prefill_tokens, 1)
+            qkv_dec.run_ragged(pos, max_pos, batch)
             dec.run_ragged(pos, max_pos, batch)
 
     _, step_ms = _time_steps(step, steps, warmup)
     flops = layers * 4 * D * hq * (prefill_tokens * (prefill_tokens + 1) // 2)
+    proj_flops = layers * 2 * (prefill_tokens + batch) * hidden * (hq + 2 * hkv) * D
     nbytes = layers * int(2 * hkv * D * 2 * lengths.sum() + 2 * batch * hq * D * 2)
+    for pair in proj:
+        for op in pair:
+            op.close()
     pre.close()
     dec.close()
-    return {"ms_per_step": step_ms, "flops": flops, "bytes": nbytes, "tokens": int(lengths.sum())}
+    return {"ms_per_step": step_ms, "flops": flops, "proj_flops": proj_flops, "bytes": nbytes,
+            "tokens": int(lengths.sum())}
 
 
 def bench_token_step(layers, batch, length, steps, warmup, hq=32, hkv=4):
@@ -583,11 +609,13 @@ def main():
     if args.only in ("", "mixed48"):
         ms = bench_mixed_step(48, 16384, 32, 1024, 131072, 3, 1)
         also.append({
-            "workload": "mixed step end to end (BASELINE configs[4]): 48 layers x (prefill 16384 tokens + "
-                        "single-token step over 32 sequences, cache lengths U{1024..131072}, seed 7), "
-                        "Q/K/V drawn directly (no projections), one stream",
+            "workload": "mixed step end to end (BASELINE configs[4]): 48 layers x (Q/K/V projection + attention "
+                        "of a 16384-token prefill, Q/K/V projection + attention of one new token of 32 "
+                        "sequences with cache lengths U{1024..131072}, seed 7), random-init fp16 projection "
+                        "weights per layer, K/V written into the caches by the projections, one stream",
             "metric": "attention ms per step", "value": round(ms["ms_per_step"], 3), "unit": "ms",
             "steps": 3, "prefill_tflop_per_step": round(ms["flops"] / 1e12, 2),
+            "projection_tflop_per_step": round(ms["proj_flops"] / 1e12, 2),
             "decode_gb_per_step": round(ms["bytes"] / 1e9, 1),
         })
     if args.only in ("", "kvwrite"):

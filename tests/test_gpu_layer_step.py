@@ -115,3 +115,57 @@ def test_layer_step_eager_graph_and_oracle():
         assert compare_ulps(gout, orc.from_storage(want_out, dtype), dtype)["ok"]
         # carry the GPU's cache forward so that later steps stay stage-local
         kc, vc = sk.copy(), sv.copy()
+
+
+def test_chunked_prefill_projection_feeds_attention():
+    """Two chunks of a prompt: the fused projection writes each chunk's K/V into the cache at
+    its positions and the chunk's queries to the scratch, attention then reads the cache
+    up to each query's position; stagewise against the oracle."""
+    import torch
+
+    import ellm_amd
+
+    dtype = orc.BF16
+    b, hq, hkv, cap, hidden = 2, 4, 2, 512, 256
+    chunks = [(0, 300), (300, 77)]
+    scale = 1.0 / np.sqrt(D)
+    rope = _rope_table(cap, dtype)
+    wq = rand_storage((hq * D, hidden), 11, dtype, scale=hidden ** -0.5)
+    wk = rand_storage((hkv * D, hidden), 12, dtype, scale=hidden ** -0.5)
+    wv = rand_storage((hkv * D, hidden), 13, dtype, scale=hidden ** -0.5)
+    xs = rand_storage((377, b, hidden), 14, dtype)
+
+    cache = ellm_amd.KVCache(1, b, hkv, cap, ellm_amd.DTYPE_BF16)
+    kt, vt = cache.layer_tensors(0, torch_dtype(dtype))
+    kt.zero_()
+    vt.zero_()
+    _, _, strides = cache.layer(0)
+    x = torch.zeros((300, b, hidden), dtype=torch.bfloat16, device="cuda")
+    q = torch.zeros((300, b, hq, D), dtype=torch.bfloat16, device="cuda")
+    att = torch.zeros_like(q)
+    dev = [to_dev(a, dtype) for a in (wq, wk, wv, rope)]
+    qkv = ellm_amd.MatMul3(x, dev[0], q, dev[1], kt, dev[2], vt, dev[3], D, b, hq, hkv, strides, cap)
+    attn = ellm_amd.Attention(q, kt, vt, att, b, hq, hkv, D, strides, scale, sequence_capacity=cap,
+                              max_position_interval=300)
+    kc = np.zeros((b, hkv, cap, D), dtype=np.uint16)
+    vc = np.zeros_like(kc)
+    for p0, n in chunks:
+        x[:n].copy_(to_dev(xs[p0:p0 + n], dtype))
+        qkv.run(p0, n, b)
+        attn.run(p0, n, b)
+        torch.cuda.synchronize()
+        gq, gatt = to_host(q, dtype)[:n], to_host(att, dtype)[:n]
+        gk, gv = to_host(kt, dtype), to_host(vt, dtype)
+        oq = np.zeros((n, b, hq, D), dtype=np.uint16)
+        assert orc.matmul3(np.ascontiguousarray(xs[p0:p0 + n]), wq, wk, wv, oq, kc, vc, rope,
+                           (hkv * cap * D, cap * D, D, 1), cap, p0, n, dtype) == 0
+        assert compare_ulps(gq, orc.from_storage(oq, dtype), dtype)["ok"]
+        assert compare_ulps(gk, orc.from_storage(kc, dtype), dtype)["ok"]
+        assert compare_ulps(gv, orc.from_storage(vc, dtype), dtype)["ok"]
+        sq, sk, sv = (orc.to_storage(a, dtype) for a in (gq, gk, gv))
+        want, _ = orc.attention(sq, sk, sv, scale, dtype, position_index=p0)
+        assert compare(gatt, orc.from_storage(want, dtype), dtype)["ok"]
+        kc, vc = sk.copy(), sv.copy()
+    qkv.close()
+    attn.close()
+    cache.close()
