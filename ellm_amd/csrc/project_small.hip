@@ -195,16 +195,17 @@ __global__ __launch_bounds__(1024) void project_small_kernel(ProjectKernelArgs p
   constexpr int kOctets = kGroupCols / 8;
   const float* src =
       ws + (((size_t)hh * kGroupsPerHead + c8 / kOctets) * kRowsCap + R) * kGroupCols + 8 * (c8 % kOctets);
-  const f32x4 lo = load_coherent128_nowait(src), hi = load_coherent128_nowait(src + 4);
+  // (the two results are not to be copied or read before the wait below: the compiler takes the
+  // asm statements for ordinary instructions whose results exist at once)
+  f32x4 lo = load_coherent128_nowait(src), hi = load_coherent128_nowait(src + 4);
   const uint32_t t = R / p.batch_pitch, b = R % p.batch_pitch;
   const bool live = R < p.rows && b < p.batch;
   const uint32_t pos = t + (p.positions ? (live ? min(p.positions[b], p.max_start) : 0u) : p.position_index);
   const uint32_t one_zero = M::pack2(1.0f, 0.0f);
   u32x4 rr = {one_zero, one_zero, one_zero, one_zero};
   if (live) rr = load16(p.rope + (size_t)pos * p.rope_pos_stride + (size_t)hs * p.rope_head_stride + 8 * c8);
-  f32x4 lo2 = lo, hi2 = hi;
-  asm volatile("s_waitcnt vmcnt(0)" : "+v"(lo2), "+v"(hi2), "+v"(rr));
-  float o[8] = {lo2[0], lo2[1], lo2[2], lo2[3], hi2[0], hi2[1], hi2[2], hi2[3]};
+  asm volatile("s_waitcnt vmcnt(0)" : "+v"(lo), "+v"(hi), "+v"(rr));
+  float o[8] = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
   float ss = 0.0f;
 #pragma unroll
   for (int e = 0; e < 8; ++e) ss = fmaf(o[e], o[e], ss);
