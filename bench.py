@@ -593,14 +593,23 @@ def main():
         mx_steps = max(3, min(args.steps, 10))
         mp = bench_prefill(16384, mx_steps, min(args.warmup, 2))
         md = bench_ragged_decode(32, 1024, 131072, mx_steps, min(args.warmup, 2))
+        mq = bench_qkv_projection(16384, mx_steps, min(args.warmup, 2))
+        msp = bench_step_projections(32, mx_steps, min(args.warmup, 2))
         also.append({
-            "workload": "mixed step, one of 48 layers (BASELINE configs[4]): prefill 16384 tokens + "
-                        "single-token step over 32 sequences, cache lengths U{1024..131072} (seed 7)",
+            "workload": "mixed step, one of 48 layers (BASELINE configs[4]), kernel by kernel: Q/K/V projection + "
+                        "attention of a 16384-token prefill, Q/K/V projection + attention of one new token of 32 "
+                        "sequences, cache lengths U{1024..131072} (seed 7)",
             "metric": "attention ms per layer",
             "value": round(mp["ms_per_step"] + md["ms_per_step"], 4), "unit": "ms",
             "prefill_ms": round(mp["ms_per_step"], 4), "prefill_tflops": round(mp["tflops"], 1),
+            "prefill_frac_of_mfma_peak": round(mp["kernel_tflops"] / MFMA_F16_PEAK_TFLOPS, 4),
             "decode_ms": round(md["ms_per_step"], 4), "decode_gbs": round(md["gbs"], 1),
             "decode_cached_tokens": md["tokens"], "steps": mx_steps,
+            "prefill_projection_ms": round(mq["ms_per_step"], 4),
+            "prefill_projection_frac_of_mfma_peak": round(mq["kernel_tflops"] / MFMA_F16_PEAK_TFLOPS, 4),
+            "decode_projection_ms": round(msp["qkv_ms"], 5),
+            "decode_projection_frac_of_hbm_peak": round(
+                msp["qkv_bytes"] / (msp["qkv_kernel_ms"] * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
             "roofline": {"bound": "hbm", "achieved": round(md["kernel_gbs"], 1),
                          "peak": HBM_PEAK_GBS, "unit": "GB/s",
                          "frac": round(md["kernel_gbs"] / HBM_PEAK_GBS, 4), "traffic": None},
