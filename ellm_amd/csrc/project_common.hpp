@@ -50,7 +50,7 @@ constexpr int kModeQkv = 0;  // heads normalised + rotated (or passed through), 
 constexpr int kModeAdd = 1;  // plain product plus a residual of the output's layout
 
 // Streaming kernel for a few rows (project_small.hip).
-constexpr uint32_t kSmallRowsMax = 32;
+constexpr uint32_t kSmallRowsMax = 128;
 hipError_t small_prepare();
 bool small_kernel_takes(uint32_t rows, uint32_t K);
 size_t small_workspace_floats(uint32_t heads, uint32_t K);

@@ -1,6 +1,6 @@
-// Projections for a few token rows (a single-token step over up to 32 sequences): the
-// weights are read exactly once and the kernel is bound by that stream (HBM), not by
-// MFMA.  Same arithmetic and epilogue as the tile kernel of project.hip.
+// Projections for up to 128 token rows (a single-token step over that many sequences, a
+// short chunk): the weights are read exactly once and the kernel is bound by that stream
+// (HBM), not by MFMA.  Same arithmetic and epilogue as the tile kernel of project.hip.
 //
 // A workgroup owns 16 or 32 output columns (one or two 16x16x32 MFMA block rows, which
 // share the token operand) and all of K: whole weight rows, contiguous in memory, so the
@@ -39,17 +39,20 @@ __device__ __forceinline__ void wait_vm_done() { __builtin_amdgcn_s_waitcnt(0x0F
 
 typedef __attribute__((address_space(3))) u32x4 LdsVec4;
 
-// NTB: 16-token blocks (1 or 2); NB: 16-column MFMA blocks per workgroup (1 or 2).
-// blockDim.x = 64 * waves, waves = min(16, K / 256).
+// NTB: 16-token blocks per pass (1 or 2); NB: 16-column MFMA blocks per workgroup (1 or 2).
+// blockDim.x = 64 * waves, waves = min(16, K / 256).  `passes` passes of 16 NTB token rows
+// each reuse the weight operands, which stay in registers; more than one pass needs
+// waves == K / 256 (one round of K per wave).
 // VIA_LDS (waves == K / 256 and the rows fit): the workgroup's weight rows, one contiguous
 // region of memory, are fetched in 1 KB pieces (a wave instruction = 1 KB of one row) and
 // handed to the MFMA operand layout through LDS; fetching them in operand layout directly
 // (16 rows x 64 B an instruction) makes the same stream a third slower.
 template <typename S, int MODE, int NTB, int NB, bool VIA_LDS>
-__global__ __launch_bounds__(1024) void project_small_kernel(ProjectKernelArgs p, float* ws,
-                                                             uint32_t* counters) {
+__global__ __launch_bounds__((NTB == 2 || NB == 2) ? 512 : 1024) void project_small_kernel(ProjectKernelArgs p, float* ws,
+                                                             uint32_t* counters, uint32_t passes) {
   using M = Mfma<S>;
   constexpr int kColBlocks = NB, kGroupCols = 16 * NB, kGroupsPerHead = kHeadDim / kGroupCols;
+  constexpr int kPassRows = 16 * NTB;
   extern __shared__ __attribute__((aligned(16))) float sums[];  // [wave][NTB][16 tokens][kGroupCols]
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, n_waves = blockDim.x >> 6;
   const int i16 = lane & 15, q4 = lane >> 4;
@@ -57,120 +60,151 @@ __global__ __launch_bounds__(1024) void project_small_kernel(ProjectKernelArgs p
   const uint32_t hh = blockIdx.x / kGroupsPerHead, cg = blockIdx.x % kGroupsPerHead;
   const uint32_t seg = (hh < p.heads0) ? 0u : (hh < p.heads0 + p.heads_kv ? 1u : 2u);
   const uint32_t hs = hh - (seg == 0 ? 0u : (seg == 1 ? p.heads0 : p.heads0 + p.heads_kv));
-  constexpr int kRowsCap = 16 * NTB;
+  const uint32_t rows_cap = passes * kPassRows;
+  const bool finalize = MODE == kModeQkv && ((seg == 1) || (seg == 0 && p.finalize0));
+  uint16_t* const dst = (seg == 0) ? p.out0 : (seg == 1 ? p.k_out : p.v_out);
 
   const uint16_t* wrow = p.w[seg] + ((size_t)hs * kHeadDim + kGroupCols * cg + i16) * K + 8 * q4;
   const size_t wblock = (size_t)16 * K;  // elements between the rows of consecutive column blocks
   const __amdgpu_buffer_rsrc_t x_rsrc =
       __builtin_amdgcn_make_buffer_rsrc((void*)uniform64(p.x), 0, p.rows * K * 2, kBufFlags);
-  f32x4 acc[kColBlocks][NTB];
-#pragma unroll
-  for (int nb = 0; nb < kColBlocks; ++nb)
-#pragma unroll
-    for (int tb = 0; tb < NTB; ++tb) acc[nb][tb] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
-  if constexpr (VIA_LDS) {
-    const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) float*)sums;
-    const uint8_t* wg_rows = (const uint8_t*)(p.w[seg] + ((size_t)hs * kHeadDim + kGroupCols * cg) * K);
-    const uint32_t row_bytes = 2 * K, pitch = row_bytes + 16;  // + 16: the 16 rows of an operand read tile the banks
-    constexpr int kPieces = 8 * NB;                            // 1 KB pieces per wave
-    const uint32_t k0 = wave * kRoundK;
-    u32x4 stg[kPieces], xreg[NTB][kStepsPerRound];
-#pragma unroll
-    for (int u = 0; u < kPieces; ++u)
-      stg[u] = __builtin_nontemporal_load((const u32x4*)(wg_rows + (size_t)(wave * kPieces + u) * 1024 + lane * 16));
+  const uint32_t k_first = wave * kRoundK;
+  // token rows of pass `pass`, K slice at k0 (rows past the last read as zero)
+  auto fetch_x = [&](u32x4 (&x)[NTB][kStepsPerRound], uint32_t pass, uint32_t k0) {
 #pragma unroll
     for (int tb = 0; tb < NTB; ++tb)
 #pragma unroll
       for (int s = 0; s < kStepsPerRound; ++s)
-        xreg[tb][s] = __builtin_amdgcn_raw_buffer_load_b128(
-            x_rsrc, ((16 * tb + i16) * K + k0 + 8 * q4 + 32 * s) * 2, 0, 0);
-    __builtin_amdgcn_sched_barrier(0);  // every fetch is on its way before the first use
-#pragma unroll
-    for (int u = 0; u < kPieces; ++u) {
-      const uint32_t off = (wave * kPieces + u) * 1024 + lane * 16;
-      const uint32_t row = off / row_bytes;
-      *(LdsVec4*)(lds0 + row * pitch + (off - row * row_bytes)) = stg[u];
-    }
-    __syncthreads();
-    u32x4 wreg[kColBlocks][kStepsPerRound];
+        x[tb][s] = __builtin_amdgcn_raw_buffer_load_b128(
+            x_rsrc, ((pass * kPassRows + 16 * tb + i16) * K + k0 + 8 * q4 + 32 * s) * 2, 0, 0);
+  };
+  auto fetch_w = [&](u32x4 (&w)[kColBlocks][kStepsPerRound], uint32_t k0) {
 #pragma unroll
     for (int nb = 0; nb < kColBlocks; ++nb)
 #pragma unroll
       for (int s = 0; s < kStepsPerRound; ++s)
-        wreg[nb][s] = *(const LdsVec4*)(lds0 + (16 * nb + i16) * pitch + (k0 + 32 * s + 8 * q4) * 2);
-#pragma unroll
-    for (int s = 0; s < kStepsPerRound; ++s)
-#pragma unroll
-      for (int nb = 0; nb < kColBlocks; ++nb)
-#pragma unroll
-        for (int tb = 0; tb < NTB; ++tb) acc[nb][tb] = M::m16x16x32(wreg[nb][s], xreg[tb][s], acc[nb][tb]);
-    __syncthreads();  // the sums below reuse the rows' LDS
-  } else {
-  for (uint32_t k0 = wave * kRoundK; k0 < K; k0 += n_waves * kRoundK) {
-      u32x4 wreg[kColBlocks][kStepsPerRound], xreg[NTB][kStepsPerRound];  // token rows past the last read as zero
-  #pragma unroll
-      for (int nb = 0; nb < kColBlocks; ++nb)
-  #pragma unroll
-        for (int s = 0; s < kStepsPerRound; ++s)
-          wreg[nb][s] = __builtin_nontemporal_load((const u32x4*)(wrow + nb * wblock + k0 + 32 * s));
-  #pragma unroll
-      for (int tb = 0; tb < NTB; ++tb)
-  #pragma unroll
-        for (int s = 0; s < kStepsPerRound; ++s)
-          xreg[tb][s] = __builtin_amdgcn_raw_buffer_load_b128(
-              x_rsrc, ((16 * tb + i16) * K + k0 + 8 * q4 + 32 * s) * 2, 0, 0);
-      __builtin_amdgcn_sched_barrier(0);  // every fetch of the round is on its way before the first use
-  #pragma unroll
-      for (int s = 0; s < kStepsPerRound; ++s)
-  #pragma unroll
-        for (int nb = 0; nb < kColBlocks; ++nb)
-  #pragma unroll
-          for (int tb = 0; tb < NTB; ++tb) acc[nb][tb] = M::m16x16x32(wreg[nb][s], xreg[tb][s], acc[nb][tb]);
-    }
-}
-  // lane (token i16, columns 16 nb + 4 q4 .. + 3)
-#pragma unroll
-  for (int nb = 0; nb < kColBlocks; ++nb)
-#pragma unroll
-    for (int tb = 0; tb < NTB; ++tb)
-      *(f32x4*)(sums + ((wave * NTB + tb) * 16 + i16) * kGroupCols + 16 * nb + 4 * q4) = acc[nb][tb];
-  __syncthreads();
+        w[nb][s] = __builtin_nontemporal_load((const u32x4*)(wrow + nb * wblock + k0 + 32 * s));
+  };
 
-  // threads 0 .. 4 kGroupCols NTB - 1: token tid / (kGroupCols / 4), four columns of the group
-  const bool finalize = MODE == kModeQkv && ((seg == 1) || (seg == 0 && p.finalize0));
-  uint16_t* const dst = (seg == 0) ? p.out0 : (seg == 1 ? p.k_out : p.v_out);
   constexpr int kQuads = kGroupCols / 4;
-  if (tid < 16 * kQuads * NTB) {
-    const uint32_t R = tid / kQuads, c4 = tid % kQuads;
-    f32x4 v = {0.0f, 0.0f, 0.0f, 0.0f};
-    for (int w = 0; w < n_waves; ++w)
-      v += *(const f32x4*)(sums + (w * kRowsCap + R) * kGroupCols + 4 * c4);
-    if (finalize) {
-      float* to = ws + (((size_t)hh * kGroupsPerHead + cg) * kRowsCap + R) * kGroupCols + 4 * c4;
+  // The waves' sums of one pass meet in LDS; threads 0 .. 4 kGroupCols NTB - 1 (token tid / kQuads
+  // of the pass, four columns of the group) add them up and either finish the row or leave it
+  // for the head's last workgroup.
+  auto finish_pass = [&](uint32_t pass, f32x4 (&acc)[kColBlocks][NTB]) {
+    // lane (token i16, columns 16 nb + 4 q4 .. + 3)
 #pragma unroll
-      for (int e = 0; e < 4; ++e) store_coherent(to + e, v[e]);
-    } else {
-      const uint32_t t = R / p.batch_pitch, b = R % p.batch_pitch;
-      if (R < p.rows && b < p.batch) {
-        size_t off;
-        if (seg == 0) {
-          off = (size_t)R * p.ld0 + hs * kHeadDim + kGroupCols * cg + 4 * c4;
-        } else {
-          const uint32_t pos = t + (p.positions ? min(p.positions[b], p.max_start) : p.position_index);
-          off = (size_t)b * p.kv_stride_seq + (size_t)hs * p.kv_stride_head +
-                (size_t)pos * p.kv_stride_pos + kGroupCols * cg + 4 * c4;
+    for (int nb = 0; nb < kColBlocks; ++nb)
+#pragma unroll
+      for (int tb = 0; tb < NTB; ++tb)
+        *(f32x4*)(sums + ((wave * NTB + tb) * 16 + i16) * kGroupCols + 16 * nb + 4 * q4) = acc[nb][tb];
+    __syncthreads();
+    if (tid < 16 * kQuads * NTB) {
+      const uint32_t R = pass * kPassRows + tid / kQuads, c4 = tid % kQuads;
+      f32x4 v = {0.0f, 0.0f, 0.0f, 0.0f};
+      for (int w = 0; w < n_waves; ++w)
+        v += *(const f32x4*)(sums + (w * kPassRows + tid / kQuads) * kGroupCols + 4 * c4);
+      if (finalize) {
+        float* to = ws + (((size_t)hh * kGroupsPerHead + cg) * rows_cap + R) * kGroupCols + 4 * c4;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) store_coherent(to + e, v[e]);
+      } else {
+        const uint32_t t = R / p.batch_pitch, b = R % p.batch_pitch;
+        if (R < p.rows && b < p.batch) {
+          size_t off;
+          if (seg == 0) {
+            off = (size_t)R * p.ld0 + hs * kHeadDim + kGroupCols * cg + 4 * c4;
+          } else {
+            const uint32_t pos = t + (p.positions ? min(p.positions[b], p.max_start) : p.position_index);
+            off = (size_t)b * p.kv_stride_seq + (size_t)hs * p.kv_stride_head +
+                  (size_t)pos * p.kv_stride_pos + kGroupCols * cg + 4 * c4;
+          }
+          if (MODE == kModeAdd) {
+            const u32x2 rs = *(const u32x2*)(p.residual + off);
+            v[0] += M::to_float((uint16_t)(rs[0] & 0xffffu));
+            v[1] += M::to_float((uint16_t)(rs[0] >> 16));
+            v[2] += M::to_float((uint16_t)(rs[1] & 0xffffu));
+            v[3] += M::to_float((uint16_t)(rs[1] >> 16));
+          }
+          const u32x2 packed = {M::pack2(v[0], v[1]), M::pack2(v[2], v[3])};
+          *(u32x2*)(dst + off) = packed;
         }
-        if (MODE == kModeAdd) {
-          const u32x2 rs = *(const u32x2*)(p.residual + off);
-          v[0] += M::to_float((uint16_t)(rs[0] & 0xffffu));
-          v[1] += M::to_float((uint16_t)(rs[0] >> 16));
-          v[2] += M::to_float((uint16_t)(rs[1] & 0xffffu));
-          v[3] += M::to_float((uint16_t)(rs[1] >> 16));
-        }
-        const u32x2 packed = {M::pack2(v[0], v[1]), M::pack2(v[2], v[3])};
-        *(u32x2*)(dst + off) = packed;
       }
     }
+  };
+
+  if constexpr (VIA_LDS) {
+    u32x4 wreg[kColBlocks][kStepsPerRound], xcur[NTB][kStepsPerRound];
+    {
+      const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) float*)sums;
+      const uint8_t* wg_rows = (const uint8_t*)(p.w[seg] + ((size_t)hs * kHeadDim + kGroupCols * cg) * K);
+      const uint32_t row_bytes = 2 * K, pitch = row_bytes + 16;  // + 16: the 16 rows of an operand read tile the banks
+      constexpr int kPieces = 8 * NB;                            // 1 KB pieces per wave
+      u32x4 stg[kPieces];
+#pragma unroll
+      for (int u = 0; u < kPieces; ++u)
+        stg[u] = __builtin_nontemporal_load((const u32x4*)(wg_rows + (size_t)(wave * kPieces + u) * 1024 + lane * 16));
+      fetch_x(xcur, 0, k_first);
+      __builtin_amdgcn_sched_barrier(0);  // every fetch is on its way before the first use
+#pragma unroll
+      for (int u = 0; u < kPieces; ++u) {
+        const uint32_t off = (wave * kPieces + u) * 1024 + lane * 16;
+        const uint32_t row = off / row_bytes;
+        *(LdsVec4*)(lds0 + row * pitch + (off - row * row_bytes)) = stg[u];
+      }
+      __syncthreads();
+#pragma unroll
+      for (int nb = 0; nb < kColBlocks; ++nb)
+#pragma unroll
+        for (int s = 0; s < kStepsPerRound; ++s)
+          wreg[nb][s] = *(const LdsVec4*)(lds0 + (16 * nb + i16) * pitch + (k_first + 32 * s + 8 * q4) * 2);
+      __syncthreads();  // the sums reuse the rows' LDS
+    }
+    // the weight operands stay in registers; the token rows of the next pass are requested
+    // before those of this one are used
+    for (uint32_t pass = 0; pass < passes; ++pass) {
+      u32x4 xnext[NTB][kStepsPerRound];
+      const bool more = pass + 1 < passes;  // (uniform)
+      if (more) fetch_x(xnext, pass + 1, k_first);
+      f32x4 acc[kColBlocks][NTB];
+#pragma unroll
+      for (int nb = 0; nb < kColBlocks; ++nb)
+#pragma unroll
+        for (int tb = 0; tb < NTB; ++tb) acc[nb][tb] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+      for (int s = 0; s < kStepsPerRound; ++s)
+#pragma unroll
+        for (int nb = 0; nb < kColBlocks; ++nb)
+#pragma unroll
+          for (int tb = 0; tb < NTB; ++tb) acc[nb][tb] = M::m16x16x32(wreg[nb][s], xcur[tb][s], acc[nb][tb]);
+      finish_pass(pass, acc);
+      if (more) {
+        __syncthreads();  // the sums are rewritten by the next pass
+#pragma unroll
+        for (int tb = 0; tb < NTB; ++tb)
+#pragma unroll
+          for (int s = 0; s < kStepsPerRound; ++s) xcur[tb][s] = xnext[tb][s];
+      }
+    }
+  } else {
+    // one pass; a wave walks its rounds of K, operands fetched in MFMA layout
+    f32x4 acc[kColBlocks][NTB];
+#pragma unroll
+    for (int nb = 0; nb < kColBlocks; ++nb)
+#pragma unroll
+      for (int tb = 0; tb < NTB; ++tb) acc[nb][tb] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+    for (uint32_t k0 = k_first; k0 < K; k0 += n_waves * kRoundK) {
+      u32x4 wreg[kColBlocks][kStepsPerRound], xreg[NTB][kStepsPerRound];
+      fetch_w(wreg, k0);
+      fetch_x(xreg, 0, k0);
+      __builtin_amdgcn_sched_barrier(0);  // every fetch of the round is on its way before the first use
+#pragma unroll
+      for (int s = 0; s < kStepsPerRound; ++s)
+#pragma unroll
+        for (int nb = 0; nb < kColBlocks; ++nb)
+#pragma unroll
+          for (int tb = 0; tb < NTB; ++tb) acc[nb][tb] = M::m16x16x32(wreg[nb][s], xreg[tb][s], acc[nb][tb]);
+    }
+    finish_pass(0, acc);
   }
   if (!finalize) return;  // (uniform over the workgroup)
 
@@ -188,45 +222,45 @@ __global__ __launch_bounds__(1024) void project_small_kernel(ProjectKernelArgs p
   __syncthreads();
   if (s_last == 0) return;
 
-  // ---- the head's last workgroup: thread -> token tid / 16, columns 8 c .. 8 c + 7 ------
-  if (tid >= 256 * NTB) return;
-  const uint32_t R = tid >> 4;
+  // ---- the head's last workgroup: thread -> token tid / 16 (+ blockDim / 16 a turn), columns 8 c .. 8 c + 7
   const int c8 = tid & 15;
   constexpr int kOctets = kGroupCols / 8;
-  const float* src =
-      ws + (((size_t)hh * kGroupsPerHead + c8 / kOctets) * kRowsCap + R) * kGroupCols + 8 * (c8 % kOctets);
-  // (the two results are not to be copied or read before the wait below: the compiler takes the
-  // asm statements for ordinary instructions whose results exist at once)
-  f32x4 lo = load_coherent128_nowait(src), hi = load_coherent128_nowait(src + 4);
-  const uint32_t t = R / p.batch_pitch, b = R % p.batch_pitch;
-  const bool live = R < p.rows && b < p.batch;
-  const uint32_t pos = t + (p.positions ? (live ? min(p.positions[b], p.max_start) : 0u) : p.position_index);
   const uint32_t one_zero = M::pack2(1.0f, 0.0f);
-  u32x4 rr = {one_zero, one_zero, one_zero, one_zero};
-  if (live) rr = load16(p.rope + (size_t)pos * p.rope_pos_stride + (size_t)hs * p.rope_head_stride + 8 * c8);
-  asm volatile("s_waitcnt vmcnt(0)" : "+v"(lo), "+v"(hi), "+v"(rr));
-  float o[8] = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-  float ss = 0.0f;
+  for (uint32_t R = tid >> 4; R < rows_cap; R += blockDim.x >> 4) {
+    const float* src =
+        ws + (((size_t)hh * kGroupsPerHead + c8 / kOctets) * rows_cap + R) * kGroupCols + 8 * (c8 % kOctets);
+    // (the two results are not to be copied or read before the wait below: the compiler takes the
+    // asm statements for ordinary instructions whose results exist at once)
+    f32x4 lo = load_coherent128_nowait(src), hi = load_coherent128_nowait(src + 4);
+    const uint32_t t = R / p.batch_pitch, b = R % p.batch_pitch;
+    const bool live = R < p.rows && b < p.batch;
+    const uint32_t pos = t + (p.positions ? (live ? min(p.positions[b], p.max_start) : 0u) : p.position_index);
+    u32x4 rr = {one_zero, one_zero, one_zero, one_zero};
+    if (live) rr = load16(p.rope + (size_t)pos * p.rope_pos_stride + (size_t)hs * p.rope_head_stride + 8 * c8);
+    asm volatile("s_waitcnt vmcnt(0)" : "+v"(lo), "+v"(hi), "+v"(rr));
+    float o[8] = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+    float ss = 0.0f;
 #pragma unroll
-  for (int e = 0; e < 8; ++e) ss = fmaf(o[e], o[e], ss);
+    for (int e = 0; e < 8; ++e) ss = fmaf(o[e], o[e], ss);
 #pragma unroll
-  for (int m = 1; m < 16; m <<= 1) ss += __shfl_xor(ss, m, 16);
-  const float inv = 1.0f / (sqrtf(ss / (float)kHeadDim) + p.eps);
+    for (int m = 1; m < 16; m <<= 1) ss += __shfl_xor(ss, m, 16);
+    const float inv = 1.0f / (sqrtf(ss / (float)kHeadDim) + p.eps);
 #pragma unroll
-  for (int e = 0; e < 4; ++e) {
-    const float cs = M::to_float((uint16_t)(rr[e] & 0xffffu)), sn = M::to_float((uint16_t)(rr[e] >> 16));
-    const float y0 = o[2 * e] * inv, y1 = o[2 * e + 1] * inv;
-    o[2 * e] = y0 * cs - y1 * sn;
-    o[2 * e + 1] = y0 * sn + y1 * cs;
-  }
-  if (live) {
-    size_t off;
-    if (seg == 0)
-      off = (size_t)R * p.ld0 + hs * kHeadDim + 8 * c8;
-    else
-      off = (size_t)b * p.kv_stride_seq + (size_t)hs * p.kv_stride_head + (size_t)pos * p.kv_stride_pos + 8 * c8;
-    const u32x4 packed = {M::pack2(o[0], o[1]), M::pack2(o[2], o[3]), M::pack2(o[4], o[5]), M::pack2(o[6], o[7])};
-    store16(dst + off, packed);
+    for (int e = 0; e < 4; ++e) {
+      const float cs = M::to_float((uint16_t)(rr[e] & 0xffffu)), sn = M::to_float((uint16_t)(rr[e] >> 16));
+      const float y0 = o[2 * e] * inv, y1 = o[2 * e + 1] * inv;
+      o[2 * e] = y0 * cs - y1 * sn;
+      o[2 * e + 1] = y0 * sn + y1 * cs;
+    }
+    if (live) {
+      size_t off;
+      if (seg == 0)
+        off = (size_t)R * p.ld0 + hs * kHeadDim + 8 * c8;
+      else
+        off = (size_t)b * p.kv_stride_seq + (size_t)hs * p.kv_stride_head + (size_t)pos * p.kv_stride_pos + 8 * c8;
+      const u32x4 packed = {M::pack2(o[0], o[1]), M::pack2(o[2], o[3]), M::pack2(o[4], o[5]), M::pack2(o[6], o[7])};
+      store16(dst + off, packed);
+    }
   }
 }
 
@@ -239,15 +273,17 @@ template <typename S, int MODE, int NTB, int NB>
 hipError_t launch_one(const ProjectKernelArgs& p, float* ws, uint32_t* counters, uint32_t heads, uint32_t waves,
                       hipStream_t stream) {
   const dim3 grid(heads * (kHeadDim / (16 * NB))), block(64 * waves);
+  const uint32_t passes = (p.rows + 16 * NTB - 1) / (16 * NTB);
   const uint32_t sums_bytes = waves * NTB * 64 * 16 * NB;
   const uint32_t rows_bytes = 16 * NB * (2 * p.K + 16);
   if (waves * kRoundK == p.K && rows_bytes <= kLdsBudget) {
-    auto kernel = project_small_kernel<S, MODE, NTB, NB, true>;
     const uint32_t lds = rows_bytes > sums_bytes ? rows_bytes : sums_bytes;
-    hipLaunchKernelGGL(kernel, grid, block, lds, stream, p, ws, counters);
+    hipLaunchKernelGGL((project_small_kernel<S, MODE, NTB, NB, true>), grid, block, lds, stream, p, ws, counters,
+                       passes);
   } else {
+    if (passes > 1) return hipErrorInvalidValue;  // (small_kernel_takes keeps such calls away)
     hipLaunchKernelGGL((project_small_kernel<S, MODE, NTB, NB, false>), grid, block, sums_bytes, stream, p, ws,
-                       counters);
+                       counters, passes);
   }
   return hipGetLastError();
 }
@@ -258,13 +294,13 @@ hipError_t launch_blocks(const ProjectKernelArgs& p, float* ws, uint32_t* counte
   uint32_t waves = p.K / kRoundK;
   if (waves > 16) waves = 16;
   // two column blocks: enough columns for >= 128 workgroups, and (where the rows go through LDS) room for 32 rows
-  const bool wide = heads * kHeadDim >= 4096 && (waves * kRoundK != p.K || 32 * (2 * p.K + 16) <= kLdsBudget);
-  if (p.rows <= 16) {
-    if (waves < 4) return hipErrorInvalidValue;  // the finishing step wants 256 threads
+  const bool wide = heads * kHeadDim >= 4096 && waves <= 8 &&
+                    (waves * kRoundK != p.K || 32 * (2 * p.K + 16) <= kLdsBudget);
+  // two token blocks a pass want 512 threads for the finishing step and 256 registers a lane
+  const bool two_blocks = p.rows > 16 && waves == 8;
+  if (!two_blocks)
     return wide ? launch_one<S, MODE, 1, 2>(p, ws, counters, heads, waves, stream)
                 : launch_one<S, MODE, 1, 1>(p, ws, counters, heads, waves, stream);
-  }
-  if (waves < 8) return hipErrorInvalidValue;  // ... 512 threads
   return wide ? launch_one<S, MODE, 2, 2>(p, ws, counters, heads, waves, stream)
               : launch_one<S, MODE, 2, 1>(p, ws, counters, heads, waves, stream);
 }
@@ -295,16 +331,19 @@ hipError_t small_prepare() {
 }
 
 bool small_kernel_takes(uint32_t rows, uint32_t K) {
-  if (K % kRoundK != 0) return false;
+  if (K % kRoundK != 0 || rows > kSmallRowsMax) return false;
   const uint32_t waves = K / kRoundK;
-  return rows <= 16 ? waves >= 4 : (rows <= kSmallRowsMax && waves >= 8);
+  if (waves < 4) return false;  // the finishing steps want 256 threads
+  if (rows <= 16) return true;
+  // several passes (or two token blocks): one round of K per wave, rows through LDS
+  return waves <= 16 && 16 * (2 * K + 16) <= kLdsBudget;
 }
 
-// Workspace of the streaming kernel: the normalised heads' sums, [head][32][128] floats;
-// one counter per head.
+// Workspace of the streaming kernel: the normalised heads' sums, [head][rows][128] floats
+// (rows rounded up to a pass); one counter per head.
 size_t small_workspace_floats(uint32_t heads, uint32_t K) {
   (void)K;
-  return (size_t)heads * kSmallRowsMax * kHeadDim;
+  return (size_t)heads * (kSmallRowsMax + 32) * kHeadDim;
 }
 
 hipError_t launch_project_small(const ProjectKernelArgs& p, float* ws, uint32_t* counters, int dtype,
