@@ -227,3 +227,51 @@ def test_matmul3_full_size_properties():
     assert compare_ulps(gv, wv_rows, dtype)["ok"]
     op.close()
     cache.close()
+
+
+def test_matmul3_and_matmul_add_random_shapes():
+    """A seeded sweep over shapes that cross every dispatch boundary (few rows / passes / tile
+    kernel, K a multiple of 64 or of 256, one or two column blocks, odd head counts, partial
+    batches, ragged positions)."""
+    import torch
+
+    import ellm_amd
+
+    rng = np.random.default_rng(2024)
+    for case in range(24):
+        dtype = orc.F16 if case % 3 else orc.BF16
+        k = int(rng.choice([64, 192, 256, 512, 1024, 1280, 2048]))
+        hq = int(rng.integers(1, 7))
+        hkv = int(rng.integers(1, 4))
+        if case % 6 == 0:
+            hq, hkv = 30, 2                      # wide output: two column blocks in the few-rows kernel
+        pitch = int(rng.integers(1, 20))
+        batch = int(rng.integers(1, pitch + 1))
+        interval = int(rng.choice([1, 1, 2, 7, 40])) if k <= 1024 else int(rng.choice([1, 1, 3]))
+        cap = 64
+        p0 = int(rng.integers(0, cap - interval + 1))
+        ragged = interval == 1 and case % 2 == 0
+        hidden = rand_storage((interval, pitch, k), 1000 + case, dtype)
+        wq, wk, wv = _weights(k, hq, hkv, dtype, 2000 + 3 * case)
+        rope = _rope_table(cap, dtype)
+        positions = rng.integers(0, cap, size=pitch).astype(np.uint32) if ragged else None
+        got, want = _run_matmul3(hidden, wq, wk, wv, rope, dtype, pitch, hq, hkv, cap, 0 if ragged else p0,
+                                 interval, batch, positions=positions)
+        for name, g, w in zip("qkv", got, want):
+            r = compare_ulps(g, w, dtype)
+            assert r["ok"], (case, name, dict(k=k, hq=hq, hkv=hkv, pitch=pitch, batch=batch, interval=interval), r)
+        # output projection on the same activations: k -> n
+        n = 128 * int(rng.integers(1, 5))
+        w = rand_storage((n, k), 3000 + case, dtype, scale=k ** -0.5)
+        res = rand_storage((interval, pitch, n), 4000 + case, dtype)
+        da, dw, dr = to_dev(hidden, dtype), to_dev(w, dtype), to_dev(res, dtype)
+        out = torch.zeros_like(dr)
+        op = ellm_amd.MatMulAdd(da, dw, dr, out)
+        op.run(0, interval, batch)
+        torch.cuda.synchronize()
+        g = to_host(out, dtype)
+        wnt = orc.from_storage(orc.matmul_add(hidden, w, res, dtype, batch_size=batch), dtype)
+        r = compare_ulps(g, wnt, dtype)
+        assert r["ok"], (case, "add", dict(k=k, n=n, pitch=pitch, batch=batch, interval=interval), r)
+        assert not g[:, batch:].any()
+        op.close()
