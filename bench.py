@@ -114,7 +114,7 @@ def bench_decode(batch, length, steps, warmup, hq=32, hkv=4, copies=4):
     }
 
 
-def bench_prefill(seq, steps, warmup, hq=32, hkv=4, dtype_name="f16", p0=0):
+def bench_prefill(seq, steps, warmup, hq=32, hkv=4, dtype_name="f16", p0=0, zero_kv=False):
     import torch
 
     import ellm_amd
@@ -129,6 +129,9 @@ def bench_prefill(seq, steps, warmup, hq=32, hkv=4, dtype_name="f16", p0=0):
     q = (_dev_normal((seq, 1, hq, D), torch.float32, 11) * qs).to(dt)
     k = (_dev_normal((1, hkv, cap, D), torch.float32, 12) * ks).to(dt)
     v = (_dev_normal((1, hkv, cap, D), torch.float32, 13) * ks).to(dt)
+    if zero_kv:  # diagnostic: same instruction stream, operands that toggle nothing
+        k.zero_()
+        v.zero_()
     out = torch.zeros_like(q)
     lse = torch.zeros((seq, 1, hq), dtype=torch.float32, device="cuda")
     op = ellm_amd.Attention(q, k, v, out, 1, hq, hkv, D, [hkv * cap * D, cap * D, D, 1], scale,
@@ -519,6 +522,10 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--skip-cpu", action="store_true")
     ap.add_argument("--only", default="", help="decode | prefill | decode128k | chunk | mixed | mixed48 | kvwrite | tokenstep | layerstep | qkv | oproj | stepproj")
+    ap.add_argument("--prefill-zero-kv", action="store_true",
+                    help="diagnostic for --only prefill: K and V all zero (the kernel issues the same "
+                         "instructions; separates its cycle count from the clock the part sustains "
+                         "under dense random operands); the line it prints is not a benchmark result")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="first run one plain 256 MiB device copy (a known-traffic dispatch "
                          "for scaling rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE readings)")
@@ -551,9 +558,10 @@ def main():
         dec = bench_decode(16, 8192, args.steps, args.warmup)
     if args.only in ("", "prefill"):
         pf_steps = max(3, min(args.steps, 10))
-        pf = bench_prefill(32768, pf_steps, min(args.warmup, 2))
+        pf = bench_prefill(32768, pf_steps, min(args.warmup, 2), zero_kv=args.prefill_zero_kv)
         also.append({
-            "workload": "prefill: 1 seq x 32768 tokens, 32q/4kv heads, fp16, causal",
+            "workload": "prefill: 1 seq x 32768 tokens, 32q/4kv heads, fp16, causal"
+                        + (" [DIAGNOSTIC: K = V = 0]" if args.prefill_zero_kv else ""),
             "metric": "prefill attn TFLOP/s", "value": round(pf["tflops"], 2), "unit": "TFLOP/s",
             "ms_per_step": round(pf["ms_per_step"], 4), "steps": pf_steps,
             "roofline": {"bound": "mfma", "achieved": round(pf["kernel_tflops"], 2),
