@@ -138,6 +138,15 @@ def load_library():
     path = lib_path()
     if not os.path.exists(path):
         raise LibraryMissing(f"{path} not found; build it with __graft_entry__.build()")
+    # PyTorch carries a HIP runtime of its own under the same soname.  A process that
+    # loaded the system's runtime first and PyTorch's second holds two runtimes, and the
+    # one that reaches the device second finds none ("no ROCm-capable device is
+    # detected").  Importing torch first makes the library bind to the runtime torch
+    # uses, so the tensors whose addresses it is given and its own calls share one.
+    try:
+        import torch  # noqa: F401
+    except ImportError:
+        pass  # a host without PyTorch uses the system's runtime alone
     lib = ctypes.CDLL(path)
     for name, (res, args) in ABI_SYMBOLS.items():
         fn = getattr(lib, name)

@@ -33,6 +33,25 @@ def test_missing_library_fails_loudly(monkeypatch, tmp_path):
         _lib.load_library()
 
 
+def test_loading_before_torch_leaves_one_hip_runtime_in_the_process():
+    """A process that loads the library before it imports torch must not end up with the
+    system's HIP runtime beside PyTorch's own copy: the second of two runtimes to reach
+    the device finds none."""
+    import subprocess
+    import sys
+    code = (
+        "import ellm_amd\n"
+        "ellm_amd.load_library()\n"
+        "import torch\n"
+        "paths = {l.split()[-1] for l in open('/proc/self/maps') if 'libamdhip64' in l}\n"
+        "print(len(paths), sorted(paths))\n"
+    )
+    r = subprocess.run([sys.executable, "-c", code], cwd=ROOT, capture_output=True, text=True,
+                       timeout=300)
+    assert r.returncode == 0, r.stderr[-2000:]
+    assert r.stdout.split()[0] == "1", r.stdout
+
+
 def test_version_and_device_count():
     lib = ellm_amd.load_library()
     assert lib.ellm_attn_version() >= 100
