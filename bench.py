@@ -581,6 +581,20 @@ def main():
                          "traffic": TRAFFIC_BYTES["decode128k"]},
         })
 
+        # the batch of configs[1] at the full cache length: 4.3 GB of K/V a step, far beyond
+        # every cache, so one set of buffers is enough
+        b128_steps = max(3, min(args.steps, 20))
+        b128 = bench_decode(16, 131072, b128_steps, min(args.warmup, 3), copies=1)
+        also.append({
+            "workload": "decode: 16 seq x 131072 cached tokens, 32q/4kv heads, fp16",
+            "metric": "decode attn HBM GB/s", "value": round(b128["gbs"], 1), "unit": "GB/s",
+            "ms_per_step": round(b128["ms_per_step"], 5), "steps": b128_steps,
+            "roofline": {"bound": "hbm", "achieved": round(b128["kernel_gbs"], 1),
+                         "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                         "frac": round(b128["kernel_gbs"] / HBM_PEAK_GBS, 4),
+                         "traffic": None},
+        })
+
     if args.only in ("", "chunk"):
         ck_steps = max(3, min(args.steps, 5))
         ck = bench_prefill(8192, ck_steps, min(args.warmup, 1), hq=64, hkv=8, dtype_name="bf16",
