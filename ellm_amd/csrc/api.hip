@@ -26,24 +26,38 @@ int fail_hip(hipError_t e, const char* what) {
   return fail(ELLM_ERR_HIP, "%s: %s", what, hipGetErrorString(e));
 }
 
-// Compute units of the current device, or 0 when it is not a gfx950 part.
-int device_cu_count(int* out_cu) {
+bool aligned16(const void* p) { return ((uintptr_t)p & 15u) == 0; }
+
+}  // namespace
+
+int ellm::current_gfx950_device(int* device, int* n_cu) {
   int dev = 0;
   hipError_t e = hipGetDevice(&dev);
-  if (e != hipSuccess) return fail(ELLM_ERR_NO_DEVICE, "hipGetDevice: %s", hipGetErrorString(e));
+  if (e != hipSuccess) {
+    (void)hipGetLastError();
+    return fail(ELLM_ERR_NO_DEVICE, "hipGetDevice: %s", hipGetErrorString(e));
+  }
   hipDeviceProp_t prop;
   e = hipGetDeviceProperties(&prop, dev);
   if (e != hipSuccess) return fail_hip(e, "hipGetDeviceProperties");
   if (strncmp(prop.gcnArchName, "gfx950", 6) != 0)
     return fail(ELLM_ERR_NO_DEVICE, "device %d is %s; this library carries gfx950 code only", dev,
                 prop.gcnArchName);
-  *out_cu = prop.multiProcessorCount;
+  *device = dev;
+  *n_cu = prop.multiProcessorCount;
   return ELLM_OK;
 }
 
-bool aligned16(const void* p) { return ((uintptr_t)p & 15u) == 0; }
-
-}  // namespace
+int ellm::check_current_device(int device) {
+  int now = -1;
+  const hipError_t e = hipGetDevice(&now);
+  if (e != hipSuccess) return fail_hip(e, "hipGetDevice");
+  if (now != device)
+    return fail(ELLM_ERR_INVALID_ARGUMENT,
+                "the handle was created on device %d; the calling thread's current device is %d",
+                device, now);
+  return ELLM_OK;
+}
 
 int ellm::set_error(int status, const char* fmt, ...) {
   va_list ap;
@@ -55,6 +69,7 @@ int ellm::set_error(int status, const char* fmt, ...) {
 
 struct ellm_attn {
   ellm_attn_desc desc;
+  int device;
   int n_cu;
   float* ws_acc;
   float* ws_ml;
@@ -66,6 +81,7 @@ struct ellm_attn {
 
 struct ellm_kv_cache {
   ellm_kv_desc desc;
+  int device;
   void* k;
   void* v;
   size_t layer_elems;  // elements per layer
@@ -147,13 +163,14 @@ int ellm_attn_create(const ellm_attn_desc* d, ellm_attn** out_handle) {
   if (!(d->inverse_sqrt_head == d->inverse_sqrt_head))
     return fail(ELLM_ERR_INVALID_ARGUMENT, "inverse_sqrt_head is NaN");
 
-  int n_cu = 0;
-  int st = device_cu_count(&n_cu);
+  int device = 0, n_cu = 0;
+  int st = ellm::current_gfx950_device(&device, &n_cu);
   if (st != ELLM_OK) return st;
 
   ellm_attn* h = new (std::nothrow) ellm_attn;
-  if (!h) return fail(ELLM_ERR_INVALID_ARGUMENT, "out of host memory");
+  if (!h) return fail(ELLM_ERR_HIP, "out of host memory");
   h->desc = *d;
+  h->device = device;
   h->n_cu = n_cu;
   h->ws = ellm::decode_workspace((uint32_t)d->batch_size, (uint32_t)d->attention_head_num,
                                  (uint32_t)d->kv_head_num, (uint32_t)n_cu);
@@ -224,6 +241,7 @@ int ellm_attn_run(ellm_attn* h, size_t position_index, size_t position_interval,
                   void* stream) {
   if (!h) return fail(ELLM_ERR_INVALID_ARGUMENT, "null handle");
   if (batch_size == 0 || position_interval == 0) return ELLM_OK;
+  if (int st = ellm::check_current_device(h->device)) return st;
   const ellm_attn_desc& d = h->desc;
   if (batch_size > d.batch_size)
     return fail(ELLM_ERR_OUT_OF_RANGE, "batch_size %zu exceeds the capacity %zu", batch_size,
@@ -252,6 +270,7 @@ int ellm_attn_run_ragged(ellm_attn* h, const uint32_t* positions, size_t max_pos
   if (!h) return fail(ELLM_ERR_INVALID_ARGUMENT, "null handle");
   if (batch_size == 0) return ELLM_OK;
   if (!positions) return fail(ELLM_ERR_INVALID_ARGUMENT, "null positions");
+  if (int st = ellm::check_current_device(h->device)) return st;
   const ellm_attn_desc& d = h->desc;
   if (batch_size > d.batch_size)
     return fail(ELLM_ERR_OUT_OF_RANGE, "batch_size %zu exceeds the capacity %zu", batch_size,
@@ -282,15 +301,22 @@ int ellm_kv_create(const ellm_kv_desc* d, ellm_kv_cache** out_cache) {
     return fail(ELLM_ERR_INVALID_ARGUMENT, "layers, sequences, kv_head_num and capacity must be > 0");
   if (d->capacity > 0x7fffffffu || d->sequences > 65535 || d->kv_head_num > 65535)
     return fail(ELLM_ERR_UNSUPPORTED, "capacity / sequences / kv_head_num too large");
-  int n_cu = 0;
-  int st = device_cu_count(&n_cu);
+  // capacity, sequences and kv_head_num are bounded above; layers is not
+  size_t layer_elems = d->sequences * d->kv_head_num;
+  size_t bytes = 0;
+  if (__builtin_mul_overflow(layer_elems, d->capacity * d->head_size, &layer_elems) ||
+      __builtin_mul_overflow(layer_elems, d->layers, &bytes) ||
+      __builtin_mul_overflow(bytes, (size_t)2, &bytes))
+    return fail(ELLM_ERR_UNSUPPORTED, "the cache's size in bytes does not fit 64 bits");
+  int device = 0, n_cu = 0;
+  int st = ellm::current_gfx950_device(&device, &n_cu);
   if (st != ELLM_OK) return st;
 
   ellm_kv_cache* c = new (std::nothrow) ellm_kv_cache;
-  if (!c) return fail(ELLM_ERR_INVALID_ARGUMENT, "out of host memory");
+  if (!c) return fail(ELLM_ERR_HIP, "out of host memory");
   c->desc = *d;
-  c->layer_elems = d->sequences * d->kv_head_num * d->capacity * d->head_size;
-  const size_t bytes = c->layer_elems * d->layers * 2;
+  c->device = device;
+  c->layer_elems = layer_elems;
   c->k = c->v = nullptr;
   hipError_t e = hipMalloc(&c->k, bytes);
   if (e == hipSuccess) e = hipMalloc(&c->v, bytes);
@@ -335,6 +361,7 @@ int ellm_kv_append(ellm_kv_cache* c, size_t layer, size_t position_index, size_t
   if (!c) return fail(ELLM_ERR_INVALID_ARGUMENT, "null cache");
   if (n_tokens == 0 || batch_size == 0) return ELLM_OK;
   if (!k_src || !v_src) return fail(ELLM_ERR_INVALID_ARGUMENT, "null source");
+  if (int st = ellm::check_current_device(c->device)) return st;
   if (!aligned16(k_src) || !aligned16(v_src))
     return fail(ELLM_ERR_INVALID_ARGUMENT, "sources must be 16-byte aligned");
   if (layer >= c->desc.layers)
@@ -365,6 +392,7 @@ int ellm_kv_append_norm_rope(ellm_kv_cache* c, size_t layer, size_t position_ind
   if (!c) return fail(ELLM_ERR_INVALID_ARGUMENT, "null cache");
   if (n_tokens == 0 || batch_size == 0) return ELLM_OK;
   if (!k_src || !v_src || !rope) return fail(ELLM_ERR_INVALID_ARGUMENT, "null source or rotary table");
+  if (int st = ellm::check_current_device(c->device)) return st;
   if (!aligned16(k_src) || !aligned16(v_src) || !aligned16(rope))
     return fail(ELLM_ERR_INVALID_ARGUMENT, "sources and rotary table must be 16-byte aligned");
   if (!(eps >= 0.0f)) return fail(ELLM_ERR_INVALID_ARGUMENT, "eps must be >= 0");

@@ -114,6 +114,13 @@ size_t project_workspace_floats(uint32_t heads, uint32_t K);
 // Per-device set-up of the projection kernels (LDS limits); call with the device current.
 hipError_t project_prepare();
 
+// The current device and its compute-unit count.  ELLM_ERR_NO_DEVICE (message recorded) when
+// there is none or it is not a gfx950 part.
+int current_gfx950_device(int* device, int* n_cu);
+// ELLM_OK when `device` (the one a handle was created on) is the calling thread's current
+// device; a handle's workspace and the caller's buffers live on that device only.
+int check_current_device(int device);
+
 // Records the message ellm_last_error_string() returns on this thread; returns status.
 int set_error(int status, const char* fmt, ...) __attribute__((format(printf, 2, 3)));
 

@@ -1,6 +1,6 @@
 // C ABI of the projections either side of attention (declared in
 // include/ellm_attn.h): validation and handles for ellm_matmul3_* and
-// ellm_matmul_add_*.  No device memory is owned here.
+// ellm_matmul_add_*.  A handle owns the workspace of the few-rows kernel only.
 #include <hip/hip_runtime.h>
 
 #include <cmath>
@@ -16,11 +16,13 @@ constexpr size_t kMaxK = 1u << 16;
 
 struct ellm_matmul3 {
   ellm_matmul3_desc d;
+  int device;
   float* ws;
   uint32_t* counters;
 };
 struct ellm_matmul_add {
   ellm_matmul_add_desc d;
+  int device;
   float* ws;
   uint32_t* counters;
 };
@@ -28,14 +30,11 @@ struct ellm_matmul_add {
 namespace {
 // Partial sums and arrival counters of the few-rows kernel; left null (the tile kernel then
 // runs every call) when they would take more than 64 MiB.
-int alloc_small_workspace(uint32_t heads, uint32_t K, float** ws, uint32_t** counters) {
+int alloc_small_workspace(uint32_t heads, uint32_t K, int* device, float** ws, uint32_t** counters) {
   *ws = nullptr;
   *counters = nullptr;
-  int n_dev = 0;
-  if (hipGetDeviceCount(&n_dev) != hipSuccess || n_dev == 0) {
-    (void)hipGetLastError();
-    return ellm::set_error(ELLM_ERR_NO_DEVICE, "no HIP device visible");
-  }
+  int n_cu = 0;
+  if (int st = ellm::current_gfx950_device(device, &n_cu)) return st;
   const hipError_t prep = ellm::project_prepare();
   if (prep != hipSuccess) return ellm::set_error(ELLM_ERR_HIP, "projection kernels: %s", hipGetErrorString(prep));
   const size_t floats = ellm::project_workspace_floats(heads, K);
@@ -99,7 +98,7 @@ int ellm_matmul3_create(const ellm_matmul3_desc* d, ellm_matmul3** out_handle) {
   if (!h) return ellm::set_error(ELLM_ERR_HIP, "out of host memory");
   h->d = *d;
   const int rc = alloc_small_workspace((uint32_t)(d->attention_head_num + 2 * d->kv_head_num),
-                                       (uint32_t)d->hidden_size, &h->ws, &h->counters);
+                                       (uint32_t)d->hidden_size, &h->device, &h->ws, &h->counters);
   if (rc != ELLM_OK) {
     delete h;
     return rc;
@@ -120,6 +119,7 @@ static int matmul3_launch(ellm_matmul3* h, size_t position_index, size_t positio
                           void* stream) {
   const ellm_matmul3_desc& d = h->d;
   if (position_interval == 0 || batch_size == 0) return ELLM_OK;
+  if (int st = ellm::check_current_device(h->device)) return st;
   if (position_interval > d.max_position_interval)
     return ellm::set_error(ELLM_ERR_OUT_OF_RANGE, "position_interval %zu exceeds max_position_interval %zu", position_interval, d.max_position_interval);
   if (batch_size > d.batch_size)
@@ -198,7 +198,7 @@ int ellm_matmul_add_create(const ellm_matmul_add_desc* d, ellm_matmul_add** out_
   ellm_matmul_add* h = new (std::nothrow) ellm_matmul_add;
   if (!h) return ellm::set_error(ELLM_ERR_HIP, "out of host memory");
   h->d = *d;
-  const int rc = alloc_small_workspace((uint32_t)(d->n / 128), (uint32_t)d->k, &h->ws, &h->counters);
+  const int rc = alloc_small_workspace((uint32_t)(d->n / 128), (uint32_t)d->k, &h->device, &h->ws, &h->counters);
   if (rc != ELLM_OK) {
     delete h;
     return rc;
@@ -220,6 +220,7 @@ int ellm_matmul_add_run(ellm_matmul_add* h, size_t position_index, size_t positi
   if (!h) return ellm::set_error(ELLM_ERR_INVALID_ARGUMENT, "null handle");
   const ellm_matmul_add_desc& d = h->d;
   if (position_interval == 0 || batch_size == 0) return ELLM_OK;
+  if (int st = ellm::check_current_device(h->device)) return st;
   if (position_interval > d.max_position_interval)
     return ellm::set_error(ELLM_ERR_OUT_OF_RANGE, "position_interval %zu exceeds max_position_interval %zu", position_interval, d.max_position_interval);
   if (batch_size > d.batch_size)

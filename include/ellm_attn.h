@@ -10,7 +10,10 @@
  * All pointers named "device" are HIP device pointers.  Every function returns
  * ELLM_OK (0) or an ellm_status; nothing aborts the process.  Functions taking a
  * stream enqueue work on it and return without waiting (stream = NULL is the
- * HIP null stream).  A handle may be used from one host thread at a time.
+ * HIP null stream).  A handle may be used from one host thread at a time.  A
+ * handle (operator, cache, projection) belongs to the device that was current
+ * when it was created: its workspace lives there, and a run or append called
+ * while another device is current returns ELLM_ERR_INVALID_ARGUMENT.
  *
  * Only head_size == 128 and 16-bit storage (binary16 / bfloat16) are supported,
  * like the reference's AVX-512 kernel (head_size hard-wired to 128 there,
@@ -32,7 +35,7 @@ typedef enum ellm_status {
   ELLM_ERR_INVALID_ARGUMENT = 1, /* null pointer, zero size, bad dtype, strides, ... */
   ELLM_ERR_UNSUPPORTED = 2,      /* head_size != 128, group size not supported, ...   */
   ELLM_ERR_OUT_OF_RANGE = 3,     /* position / batch / slot beyond the stated capacity */
-  ELLM_ERR_HIP = 4,              /* a HIP runtime call failed; see ellm_last_error_string */
+  ELLM_ERR_HIP = 4,              /* a HIP runtime call (or a host allocation) failed      */
   ELLM_ERR_NO_DEVICE = 5         /* no gfx950 device visible                           */
 } ellm_status;
 

@@ -114,6 +114,10 @@ def test_null_arguments():
     assert lib.ellm_kv_create(ctypes.byref(kd), ctypes.byref(c)) == UNSUPPORTED
     kd = _lib.KvDesc(0, 1, 1, 128, 16, 0)
     assert lib.ellm_kv_create(ctypes.byref(kd), ctypes.byref(c)) == INVALID
+    # a size that does not fit 64 bits is refused before anything is allocated
+    kd = _lib.KvDesc(1 << 40, 65535, 65535, 128, (1 << 31) - 1, 0)
+    assert lib.ellm_kv_create(ctypes.byref(kd), ctypes.byref(c)) == UNSUPPORTED
+    assert b"64 bits" in lib.ellm_last_error_string()
 
 
 def test_valid_description_without_a_device_reports_no_device():
