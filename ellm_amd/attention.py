@@ -34,6 +34,30 @@ def _stream_ptr(stream):
     return ctypes.c_void_p(stream.cuda_stream)
 
 
+def _device_buffer(name, t, need_elems=None, dtype=None):
+    """The library is handed raw addresses: make sure `t` is device memory of the stated
+    type that holds, from its first element on, the `need_elems` elements the operator
+    addresses.  A host address or a short buffer would be a device memory fault."""
+    if not getattr(t, "is_cuda", False):
+        raise TypeError(f"{name} must be a device (CUDA/HIP) tensor, got {getattr(t, 'device', type(t))}")
+    if dtype is not None and t.dtype != dtype:
+        raise TypeError(f"{name} is {t.dtype}, expected {dtype}")
+    if need_elems is not None:
+        have = t.untyped_storage().nbytes() // t.element_size() - t.storage_offset()
+        if have < need_elems:
+            raise ValueError(f"{name} holds {have} elements from its first one; "
+                             f"the operator addresses {need_elems}")
+    return t.data_ptr()
+
+
+def _positions_ptr(positions, batch_size):
+    import torch
+
+    if positions.dtype not in (torch.int32, torch.uint32):
+        raise TypeError(f"positions must be 32-bit integers, got {positions.dtype}")
+    return ctypes.c_void_p(_device_buffer("positions", positions, batch_size))
+
+
 class Attention:
     """Attention::new / run over device buffers.
 
@@ -44,11 +68,21 @@ class Attention:
     def __init__(self, q, k, v, out, batch_size, attention_head_num, kv_head_num, head_size,
                  kv_strides, inverse_sqrt_head, lse=None, sequence_capacity=None,
                  max_position_interval=None):
+        import torch
+
         self._lib = load_library()
         self._keep = (q, k, v, out, lse)
+        cap = int(sequence_capacity if sequence_capacity is not None else k.shape[2])
+        interval = int(max_position_interval if max_position_interval is not None else q.shape[0])
+        rows = interval * batch_size * attention_head_num
+        kv_span = ((batch_size - 1) * int(kv_strides[0]) + (kv_head_num - 1) * int(kv_strides[1])
+                   + (cap - 1) * int(kv_strides[2]) + head_size)
         d = AttnDesc()
-        d.q, d.k, d.v, d.out = q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr()
-        d.lse = lse.data_ptr() if lse is not None else None
+        d.q = _device_buffer("q", q, rows * head_size)
+        d.out = _device_buffer("out", out, rows * head_size, q.dtype)
+        d.k = _device_buffer("k", k, kv_span, q.dtype)
+        d.v = _device_buffer("v", v, kv_span, q.dtype)
+        d.lse = _device_buffer("lse", lse, rows, torch.float32) if lse is not None else None
         d.batch_size = batch_size
         d.attention_head_num = attention_head_num
         d.kv_head_num = kv_head_num
@@ -57,9 +91,8 @@ class Attention:
             d.kv_strides[i] = int(kv_strides[i])
         d.inverse_sqrt_head = float(inverse_sqrt_head)
         d.dtype = _dtype_code(q)
-        d.sequence_capacity = int(sequence_capacity if sequence_capacity is not None else k.shape[2])
-        d.max_position_interval = int(
-            max_position_interval if max_position_interval is not None else q.shape[0])
+        d.sequence_capacity = cap
+        d.max_position_interval = interval
         self.desc = d
         self._handle = ctypes.c_void_p()
         check(self._lib.ellm_attn_create(ctypes.byref(d), ctypes.byref(self._handle)))
@@ -77,7 +110,7 @@ class Attention:
 
     def run_ragged(self, positions, max_position, batch_size, stream=None):
         """Single-token step; positions: uint32/int32 device tensor, one entry per sequence."""
-        check(self._lib.ellm_attn_run_ragged(self._handle, ctypes.c_void_p(positions.data_ptr()),
+        check(self._lib.ellm_attn_run_ragged(self._handle, _positions_ptr(positions, batch_size),
                                              int(max_position), batch_size, _stream_ptr(stream)))
 
     def close(self):
@@ -130,10 +163,11 @@ class KVCache:
         n_tokens, pitch = k_src.shape[0], k_src.shape[1]
         if batch_size is None:
             batch_size = pitch
+        need = n_tokens * pitch * self.desc.kv_head_num * self.desc.head_size
         check(self._lib.ellm_kv_append(self._handle, layer, position_index, n_tokens, batch_size,
-                                       ctypes.c_void_p(k_src.data_ptr()),
-                                       ctypes.c_void_p(v_src.data_ptr()), pitch,
-                                       _stream_ptr(stream)))
+                                       ctypes.c_void_p(_device_buffer("k_src", k_src, need)),
+                                       ctypes.c_void_p(_device_buffer("v_src", v_src, need, k_src.dtype)),
+                                       pitch, _stream_ptr(stream)))
 
     def append_norm_rope(self, layer, position_index, k_src, v_src, rope, eps=1e-6, batch_size=None,
                          positions=None, max_position=0, stream=None):
@@ -144,12 +178,14 @@ class KVCache:
         n_tokens, pitch = k_src.shape[0], k_src.shape[1]
         if batch_size is None:
             batch_size = pitch
-        pos_ptr = ctypes.c_void_p(positions.data_ptr()) if positions is not None else None
+        pos_ptr = _positions_ptr(positions, batch_size) if positions is not None else None
+        need = n_tokens * pitch * self.desc.kv_head_num * self.desc.head_size
         check(self._lib.ellm_kv_append_norm_rope(
             self._handle, layer, position_index, n_tokens, batch_size,
-            ctypes.c_void_p(k_src.data_ptr()), ctypes.c_void_p(v_src.data_ptr()), pitch,
-            ctypes.c_void_p(rope.data_ptr()), rope.shape[0], ctypes.c_float(eps), pos_ptr,
-            int(max_position), _stream_ptr(stream)))
+            ctypes.c_void_p(_device_buffer("k_src", k_src, need)),
+            ctypes.c_void_p(_device_buffer("v_src", v_src, need, k_src.dtype)), pitch,
+            ctypes.c_void_p(_device_buffer("rope", rope, rope.shape[0] * 128, k_src.dtype)),
+            rope.shape[0], ctypes.c_float(eps), pos_ptr, int(max_position), _stream_ptr(stream)))
 
     def close(self):
         if self._handle:

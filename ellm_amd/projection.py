@@ -5,7 +5,7 @@ residual, src/compiler/mul/matmul_add.rs).  torch tensors are device buffers onl
 import ctypes
 
 from ._lib import MatMul3Desc, MatMulAddDesc, check, load_library
-from .attention import _dtype_code, _stream_ptr
+from .attention import _device_buffer, _dtype_code, _positions_ptr, _stream_ptr
 
 
 class MatMul3:
@@ -25,21 +25,30 @@ class MatMul3:
                  max_position_interval=None):
         self._lib = load_library()
         self._keep = (hidden, q_weight, q_state, k_weight, k_state, v_weight, v_state, rope)
+        dt = hidden.dtype
+        hidden_size = hidden.shape[-1]
+        interval = int(max_position_interval if max_position_interval is not None else hidden.shape[0])
+        rows = interval * batch_size
+        kv_span = ((batch_size - 1) * int(kv_strides[0]) + (kv_head_num - 1) * int(kv_strides[1])
+                   + (int(sequence_capacity) - 1) * int(kv_strides[2]) + head_dim)
         d = MatMul3Desc()
-        d.hidden, d.q_weight, d.k_weight, d.v_weight = (hidden.data_ptr(), q_weight.data_ptr(),
-                                                        k_weight.data_ptr(), v_weight.data_ptr())
-        d.q_state, d.k_state, d.v_state = q_state.data_ptr(), k_state.data_ptr(), v_state.data_ptr()
-        d.rope = rope.data_ptr()
+        d.hidden = _device_buffer("hidden", hidden, rows * hidden_size)
+        d.q_weight = _device_buffer("q_weight", q_weight, attention_head_num * head_dim * hidden_size, dt)
+        d.k_weight = _device_buffer("k_weight", k_weight, kv_head_num * head_dim * hidden_size, dt)
+        d.v_weight = _device_buffer("v_weight", v_weight, kv_head_num * head_dim * hidden_size, dt)
+        d.q_state = _device_buffer("q_state", q_state, rows * attention_head_num * head_dim, dt)
+        d.k_state = _device_buffer("k_state", k_state, kv_span, dt)
+        d.v_state = _device_buffer("v_state", v_state, kv_span, dt)
+        d.rope = _device_buffer("rope", rope, rope.numel(), dt)
         d.rope_position_stride, d.rope_head_stride = int(rope_position_stride), int(rope_head_stride)
         d.rope_elems = rope.numel()
-        d.hidden_size = hidden.shape[-1]
+        d.hidden_size = hidden_size
         d.batch_size = batch_size
         d.attention_head_num, d.kv_head_num, d.head_size = attention_head_num, kv_head_num, head_dim
         for i in range(4):
             d.kv_strides[i] = int(kv_strides[i])
         d.sequence_capacity = int(sequence_capacity)
-        d.max_position_interval = int(
-            max_position_interval if max_position_interval is not None else hidden.shape[0])
+        d.max_position_interval = interval
         d.eps = float(eps)
         d.dtype = _dtype_code(hidden)
         self.desc = d
@@ -58,7 +67,7 @@ class MatMul3:
                                          batch_size, _stream_ptr(stream)))
 
     def run_ragged(self, positions, max_position, batch_size, stream=None):
-        check(self._lib.ellm_matmul3_run_ragged(self._handle, ctypes.c_void_p(positions.data_ptr()),
+        check(self._lib.ellm_matmul3_run_ragged(self._handle, _positions_ptr(positions, batch_size),
                                                 int(max_position), batch_size, _stream_ptr(stream)))
 
     def close(self):
@@ -85,13 +94,16 @@ class MatMulAdd:
         self._lib = load_library()
         self._keep = (a, b_nt, residual, output)
         d = MatMulAddDesc()
-        d.a, d.b_nt, d.residual, d.output = (a.data_ptr(), b_nt.data_ptr(), residual.data_ptr(),
-                                             output.data_ptr())
         d.batch_size = int(m_max if m_max is not None else a.shape[1])
         d.n = int(n_max if n_max is not None else b_nt.shape[0])
         d.k = int(k_max if k_max is not None else b_nt.shape[1])
         d.max_position_interval = int(
             max_position_interval if max_position_interval is not None else a.shape[0])
+        rows = d.max_position_interval * d.batch_size
+        d.a = _device_buffer("a", a, rows * d.k)
+        d.b_nt = _device_buffer("b_nt", b_nt, d.n * d.k, a.dtype)
+        d.residual = _device_buffer("residual", residual, rows * d.n, a.dtype)
+        d.output = _device_buffer("output", output, rows * d.n, a.dtype)
         d.dtype = _dtype_code(a)
         self.desc = d
         self._handle = ctypes.c_void_p()

@@ -136,3 +136,22 @@ def test_host_mirror_only_thread_zero_launches():
     op._handle = None
     op._lib = None
     op.run(0, 1, 1, cpu_num=8, thread_id=3)   # would raise if it reached the library
+
+
+def test_host_mirrors_refuse_host_memory_and_wrong_types():
+    """The mirrors hand raw addresses to the library: a host tensor or a tensor of another
+    type must be refused on the host, before any handle exists."""
+    import torch
+
+    q = torch.zeros((1, 1, 2, 128), dtype=torch.float16)
+    kv = torch.zeros((1, 1, 16, 128), dtype=torch.float16)
+    with pytest.raises(TypeError, match="device"):
+        ellm_amd.Attention(q, kv, kv, q.clone(), 1, 2, 1, 128, [16 * 128, 16 * 128, 128, 1], 0.1)
+    x = torch.zeros((1, 1, 256), dtype=torch.float16)
+    w = torch.zeros((128, 256), dtype=torch.float16)
+    with pytest.raises(TypeError, match="device"):
+        ellm_amd.MatMulAdd(x, w, torch.zeros((1, 1, 128), dtype=torch.float16),
+                           torch.zeros((1, 1, 128), dtype=torch.float16))
+    with pytest.raises(TypeError, match="device"):
+        ellm_amd.MatMul3(x, w, q, w, kv, w, kv, torch.zeros((16, 128), dtype=torch.float16), 128, 1,
+                         1, 1, [16 * 128, 16 * 128, 128, 1], 16)

@@ -314,3 +314,31 @@ def test_host_mirror_thread_convention():
     want, _ = orc.attention(q, k, v, 0.09, dtype, position_index=63)
     assert compare(to_host(dout, dtype), orc.from_storage(want, dtype), dtype)["ok"]
     op.close()
+
+
+@pytest.mark.gpu
+def test_host_mirror_refuses_short_or_mistyped_buffers():
+    """Extents are checked against what the operator will address (the C ABI sees addresses
+    only): a cache shorter than capacity x stride, an output of another type, 64-bit positions."""
+    import torch
+
+    import ellm_amd
+
+    hq, hkv, cap = 8, 2, 64
+    q = torch.zeros((1, 2, hq, 128), dtype=torch.float16, device="cuda")
+    out = torch.zeros_like(q)
+    k = torch.zeros((2, hkv, cap, 128), dtype=torch.float16, device="cuda")
+    strides = [hkv * cap * 128, cap * 128, 128, 1]
+    with pytest.raises(ValueError, match="addresses"):
+        ellm_amd.Attention(q, k[:, :, : cap // 2].contiguous(), k, out, 2, hq, hkv, 128, strides, 0.1,
+                           sequence_capacity=cap)
+    with pytest.raises(TypeError, match="expected"):
+        ellm_amd.Attention(q, k, k, out.to(torch.bfloat16), 2, hq, hkv, 128, strides, 0.1)
+    with pytest.raises(ValueError, match="addresses"):
+        ellm_amd.Attention(q, k, k, out, 3, hq, hkv, 128, strides, 0.1)   # batch capacity 3, buffers for 2
+    op = ellm_amd.Attention(q, k, k, out, 2, hq, hkv, 128, strides, 0.1)
+    with pytest.raises(TypeError, match="32-bit"):
+        op.run_ragged(torch.zeros(2, dtype=torch.int64, device="cuda"), 3, 2)
+    with pytest.raises(ValueError, match="addresses"):
+        op.run_ragged(torch.zeros(1, dtype=torch.int32, device="cuda"), 3, 2)
+    op.close()
