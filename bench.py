@@ -521,7 +521,7 @@ def main():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--skip-cpu", action="store_true")
-    ap.add_argument("--only", default="", help="decode | prefill | decode128k | chunk | mixed | mixed48 | kvwrite | tokenstep | layerstep | qkv | oproj | stepproj")
+    ap.add_argument("--only", default="", help="decode | prefill | decode128k | chunk | mixed | mixed48 | kvwrite | tokenstep | layerstep | qkv | oproj | chunkproj | stepproj")
     ap.add_argument("--prefill-zero-kv", action="store_true",
                     help="diagnostic for --only prefill: K and V all zero (the kernel issues the same "
                          "instructions; separates its cycle count from the clock the part sustains "
@@ -697,6 +697,23 @@ def main():
             "roofline": {"bound": "mfma", "achieved": round(po["kernel_tflops"], 2),
                          "peak": MFMA_F16_PEAK_TFLOPS, "unit": "TFLOP/s",
                          "frac": round(po["kernel_tflops"] / MFMA_F16_PEAK_TFLOPS, 4), "traffic": None},
+        })
+
+    if args.only in ("", "chunkproj"):
+        # the reference's serving shape: chunks of 64 positions x 24 sequences (src/serving/start copy.rs:30)
+        cq = bench_qkv_projection(64, args.steps, min(args.warmup, 5), batch=24)
+        co = bench_output_projection(64 * 24, args.steps, min(args.warmup, 5))
+        also.append({
+            "workload": "projections of a prompt chunk of 64 positions x 24 sequences (1536 rows, the reference's "
+                        "serving shape): fused Q/K/V 2048 -> 5120 and output + residual 4096 -> 2048, fp16 "
+                        "(128-token x one-head tiles)",
+            "metric": "projection TFLOP/s (Q/K/V)", "value": round(cq["tflops"], 2), "unit": "TFLOP/s",
+            "ms_per_step": round(cq["ms_per_step"], 5), "steps": args.steps,
+            "output_projection_ms": round(co["ms_per_step"], 5),
+            "output_projection_tflops": round(co["tflops"], 2),
+            "roofline": {"bound": "mfma", "achieved": round(cq["kernel_tflops"], 2),
+                         "peak": MFMA_F16_PEAK_TFLOPS, "unit": "TFLOP/s",
+                         "frac": round(cq["kernel_tflops"] / MFMA_F16_PEAK_TFLOPS, 4), "traffic": None},
         })
 
     if args.only in ("", "stepproj"):

@@ -125,6 +125,7 @@ ABI_SYMBOLS = {
     "ellm_matmul_add_create": (ctypes.c_int, [ctypes.POINTER(MatMulAddDesc), _pvp]),
     "ellm_matmul_add_run": (ctypes.c_int, [_vp, _sz, _sz, _sz, _vp]),
     "ellm_matmul_add_destroy": (ctypes.c_int, [_vp]),
+    "ellm_projection_path": (ctypes.c_int, [_sz, _sz, _sz]),
 }
 
 _lib = None

@@ -22,7 +22,7 @@
 // cache the same miss entry as a whole one) through two LDS stages: chunk c is read while
 // chunk c + 1, fetched into registers an iteration earlier, is written to the other stage.
 // Calls with at most 128 rows go to the streaming kernel of project_small.hip instead.
-#include "project_common.hpp"
+#include "project_epilogue.hpp"
 
 namespace ellm {
 using namespace proj;
@@ -37,16 +37,11 @@ constexpr int kKc = 64;                             // K elements per chunk: one
 constexpr int kRowPitch = kKc * 2;
 constexpr int kStageBytes = 2 * kTile * kRowPitch;  // X rows then W rows
 constexpr int kStages = 2;
-constexpr int kEpPitch = kHeadDim * 2 + 16;         // output row in LDS
-constexpr int kEpWaveBytes = 32 * kEpPitch + 32 * 8;  // 32 rows and their destinations, per wave
 constexpr int kProjThreads = 256;
 constexpr int kProjLdsBytes = kStages * kStageBytes;
 static_assert(4 * kEpWaveBytes <= kProjLdsBytes, "the epilogue reuses the stages");
 constexpr int kGroupM = 4;                          // token tiles that take turns on one column tile
 
-typedef __attribute__((address_space(3))) u32x4 LdsVec4;
-typedef __attribute__((address_space(3))) u32x2 LdsVec2;
-typedef __attribute__((address_space(3))) uint64_t LdsU64;
 
 template <typename S, int MODE>
 __global__ __launch_bounds__(kProjThreads) void project_kernel(ProjectKernelArgs p) {
@@ -206,112 +201,25 @@ __global__ __launch_bounds__(kProjThreads) void project_kernel(ProjectKernelArgs
     __builtin_amdgcn_s_barrier();
   }
 
-  // ---- epilogue: per wave one head x 128 tokens ------------------------------------
-  const uint32_t hh = 2 * tn + wn;
-  if (hh >= heads_total) return;
-  const uint32_t seg = (hh < p.heads0) ? 0u : (hh < p.heads0 + p.heads_kv ? 1u : 2u);
-  const uint32_t hs = hh - (seg == 0 ? 0u : (seg == 1 ? p.heads0 : p.heads0 + p.heads_kv));
-  const bool finalize = MODE == kModeQkv && ((seg == 1) || (seg == 0 && p.finalize0));
-  uint16_t* const dst = (seg == 0) ? p.out0 : (seg == 1 ? p.k_out : p.v_out);
-  // In the accumulator layout lane (j, g) holds, for token 32 mb + j, the
-  // columns 32 nb + 8 b + 4 g + (0..3) of the head: four consecutive columns = two rotation
-  // pairs = one 8-byte piece of the rotary row, of the residual row and of the output
-  // row; lanes l and l ^ 32 together own the token's 128 columns.  The extra operand
-  // (table or residual) of token block mb + 1 is requested before block mb is worked on.
-  // One code path: a head that is not normalised and rotated runs the same arithmetic
-  // with scale 1 and the rotation (cos, sin) = (1, 0), which leaves every value as it is.
-  uint16_t* out_row[4];
-  const uint16_t* ext_row[4];
-  bool live[4];
-#pragma unroll
-  for (int mb = 0; mb < 4; ++mb) {
-    const uint32_t R = row0 + wm * 128 + 32 * mb + j;
-    const uint32_t t = R / p.batch_pitch, b = R % p.batch_pitch;
-    live[mb] = R < p.rows && b < p.batch;
-    uint32_t pos = t;
-    if (p.positions)
-      pos += live[mb] ? min(p.positions[b], p.max_start) : 0u;
-    else
-      pos += p.position_index;
-    const size_t col = hs * kHeadDim;
-    if (seg == 0)
-      out_row[mb] = dst + (size_t)R * p.ld0 + col;
-    else
-      out_row[mb] = dst + (size_t)b * p.kv_stride_seq + (size_t)hs * p.kv_stride_head +
-                    (size_t)pos * p.kv_stride_pos;
-    if (MODE == kModeQkv)
-      ext_row[mb] = p.rope + (size_t)pos * p.rope_pos_stride + (size_t)hs * p.rope_head_stride + 4 * g;
-    else
-      ext_row[mb] = p.residual + (size_t)R * p.ld0 + col + 4 * g;
-  }
-  const uint32_t ep_rows = lds0 + wave * kEpWaveBytes, ep_table = ep_rows + 32 * kEpPitch;
-  const uint32_t one_zero = M::pack2(1.0f, 0.0f);
-  u32x2 ext[2][16];
-  auto fetch_ext = [&](auto set, int mb) {
-    if ((MODE == kModeAdd || finalize) && live[mb]) {
-#pragma unroll
-      for (int i = 0; i < 16; ++i) ext[set][i] = *(const u32x2*)(ext_row[mb] + 32 * (i >> 2) + 8 * (i & 3));
-    } else {
-#pragma unroll
-      for (int i = 0; i < 16; ++i) ext[set][i] = u32x2{one_zero, one_zero};
-    }
-  };
-  fetch_ext(std::integral_constant<int, 0>{}, 0);
-  static_for<4>([&](auto mb_) {
-    constexpr int mb = decltype(mb_)::value;
-    constexpr int set = mb & 1;
-    __builtin_amdgcn_sched_barrier(0);  // one token block's accumulators at a time leave the AGPRs
-    if constexpr (mb + 1 < 4) fetch_ext(std::integral_constant<int, 1 - set>{}, mb + 1);
-    float inv = 1.0f;
-    if (MODE == kModeQkv) {
-      float ss = 0.0f;
-#pragma unroll
-      for (int nb = 0; nb < 4; ++nb)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) ss = fmaf(acc[nb][mb][r], acc[nb][mb][r], ss);
-      ss = sum_with_partner_half(ss);
-      inv = finalize ? 1.0f / (sqrtf(ss / (float)kHeadDim) + p.eps) : 1.0f;
-    }
-    u32x2 packed[16];
-#pragma unroll
-    for (int i = 0; i < 16; ++i) {
-      const int nb = i >> 2, b4 = i & 3;
-      float o0 = acc[nb][mb][4 * b4], o1 = acc[nb][mb][4 * b4 + 1];
-      float o2 = acc[nb][mb][4 * b4 + 2], o3 = acc[nb][mb][4 * b4 + 3];
-      const u32x2 rr = ext[set][i];
-      const float e0 = M::to_float((uint16_t)(rr[0] & 0xffffu)), e1 = M::to_float((uint16_t)(rr[0] >> 16));
-      const float e2 = M::to_float((uint16_t)(rr[1] & 0xffffu)), e3 = M::to_float((uint16_t)(rr[1] >> 16));
-      if (MODE == kModeQkv) {
-        const float y0 = o0 * inv, y1 = o1 * inv, y2 = o2 * inv, y3 = o3 * inv;
-        o0 = y0 * e0 - y1 * e1;
-        o1 = y0 * e1 + y1 * e0;
-        o2 = y2 * e2 - y3 * e3;
-        o3 = y2 * e3 + y3 * e2;
-      } else {
-        o0 += e0;
-        o1 += e1;
-        o2 += e2;
-        o3 += e3;
-      }
-      packed[i] = u32x2{M::pack2(o0, o1), M::pack2(o2, o3)};
-    }
-    // out through LDS so that a store instruction covers whole 256-byte rows: the lane
-    // that owns token j also leaves the row's destination (0: nothing to write)
-    if (g == 0) *(LdsU64*)(ep_table + 8 * j) = live[mb] ? (uint64_t)out_row[mb] : 0ull;
-#pragma unroll
-    for (int i = 0; i < 16; ++i)
-      *(LdsVec2*)(ep_rows + j * kEpPitch + 2 * (32 * (i >> 2) + 8 * (i & 3) + 4 * g)) = packed[i];
-#pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      const uint32_t row = 4 * i + (lane >> 4);
-      uint16_t* const to = (uint16_t*)*(const LdsU64*)(ep_table + 8 * row);
-      const u32x4 v = *(const LdsVec4*)(ep_rows + row * kEpPitch + 16 * (lane & 15));
-      if (to) store16(to + 8 * (lane & 15), v);
-    }
-  });
+  finish_head<S, MODE, 4>(p, acc, 2 * tn + wn, row0 + wm * 128, lds0 + wave * kEpWaveBytes, lane);
 }
 
 }  // namespace
+
+// Compute units of the device the kernels were prepared on (project_prepare()).
+static uint32_t g_n_cu = 256;
+
+// Which kernel a call runs: the few-rows streaming kernel when the handle has its workspace
+// and the shape fits it; else 128-token x one-head tiles when the 256 x 256 tiles would leave
+// compute units idle and the small tiles are all resident at once (two per compute unit:
+// beyond that the large tiles' lower traffic per flop wins, measured); else 256 x 256 tiles.
+int project_path(uint32_t rows, uint32_t heads, uint32_t K, bool has_workspace) {
+  if (has_workspace && small_kernel_takes(rows, K)) return kPathFewRows;
+  const uint32_t big = ((rows + kTile - 1) / kTile) * ((heads + 1) / 2);
+  const uint32_t mid = ((rows + 127) / 128) * heads;
+  if (big < g_n_cu && mid <= 2 * g_n_cu) return kPathMidTiles;
+  return kPathTiles;
+}
 
 hipError_t launch_project(const ProjectArgs& a, hipStream_t stream) {
   if (a.rows == 0) return hipSuccess;
@@ -344,8 +252,10 @@ hipError_t launch_project(const ProjectArgs& a, hipStream_t stream) {
   p.max_start = a.max_start;
   p.finalize0 = a.finalize0;
   p.eps = a.eps;
-  if (a.ws && a.counters && small_kernel_takes(a.rows, a.K))
+  const int path = project_path(a.rows, a.heads0 + 2 * a.heads_kv, a.K, a.ws && a.counters);
+  if (path == kPathFewRows)
     return launch_project_small(p, a.ws, a.counters, a.dtype, a.residual != nullptr, stream);
+  if (path == kPathMidTiles) return launch_project_mid(p, a.dtype, a.residual != nullptr, stream);
   const uint32_t blocks = p.tiles_m * p.tiles_n;
   auto go = [&](auto kernel) {
     hipLaunchKernelGGL(kernel, dim3(blocks), dim3(kProjThreads), kProjLdsBytes, stream, p);
@@ -365,6 +275,12 @@ hipError_t project_prepare() {
     const hipError_t e = hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, kProjLdsBytes);
     if (e != hipSuccess) return e;
   }
+  int dev = 0, n_cu = 0;
+  if (hipGetDevice(&dev) == hipSuccess &&
+      hipDeviceGetAttribute(&n_cu, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && n_cu > 0)
+    g_n_cu = (uint32_t)n_cu;
+  const hipError_t e = mid_prepare();
+  if (e != hipSuccess) return e;
   return small_prepare();
 }
 

@@ -177,6 +177,12 @@ int ellm_matmul3_run_ragged(ellm_matmul3* h, const uint32_t* positions, size_t m
   return matmul3_launch(h, 0, 1, batch_size, positions, max_position, stream);
 }
 
+int ellm_projection_path(size_t rows, size_t heads, size_t k) {
+  if (rows == 0 || heads == 0 || k == 0 || rows > 0xffffffffu / 2 || heads > 3 * 4096 || k > kMaxK)
+    return -1;
+  return ellm::project_path((uint32_t)rows, (uint32_t)heads, (uint32_t)k, true);
+}
+
 int ellm_matmul_add_create(const ellm_matmul_add_desc* d, ellm_matmul_add** out_handle) {
   if (!d || !out_handle) return ellm::set_error(ELLM_ERR_INVALID_ARGUMENT, "null descriptor or handle pointer");
   *out_handle = nullptr;

@@ -57,6 +57,10 @@ size_t small_workspace_floats(uint32_t heads, uint32_t K);
 hipError_t launch_project_small(const ProjectKernelArgs& p, float* ws, uint32_t* counters, int dtype,
                                 bool add, hipStream_t stream);
 
+// Tile kernel with 128-token x one-head tiles (project_mid.hip), for row counts at which
+// the 256 x 256 tiles are fewer than the compute units.
+hipError_t mid_prepare();
+hipError_t launch_project_mid(ProjectKernelArgs p, int dtype, bool add, hipStream_t stream);
 
 }  // namespace proj
 }  // namespace ellm

@@ -74,12 +74,27 @@ def _weights(k, hq, hkv, dtype, seed):
             rand_storage((hkv * D, k), seed + 2, dtype, scale=s))
 
 
+FEW_ROWS, MID_TILES, TILES = 0, 1, 2     # ellm_projection_path
+
+
+def _path(rows, heads, k):
+    import ellm_amd
+
+    return ellm_amd.load_library().ellm_projection_path(rows, heads, k)
+
+
 CASES = [
     # interval, pitch, batch, k, hq, hkv, cap, p0, dtype
-    (300, 1, 1, 256, 8, 2, 512, 17, orc.F16),      # two token tiles, the second partial; 5 column tiles
+    # 128-token x one-head tiles (more than 128 rows, too few for 256 x 256 tiles to fill the part)
+    (300, 1, 1, 256, 8, 2, 512, 17, orc.F16),      # three token tiles, the last partial
+    (513, 1, 1, 192, 2, 2, 1024, 3, orc.BF16),     # five token tiles, bfloat16
+    (9, 100, 97, 2048, 32, 4, 64, 7, orc.F16),     # 897 rows of the benchmark model, sequences beyond batch_size skipped
+    (33, 5, 4, 64, 3, 1, 64, 9, orc.BF16),         # one chunk of K, odd head count
+    # 256 x 256 tiles (many rows; K kept small so that the oracle stays quick)
+    (2081, 8, 5, 64, 3, 1, 4096, 9, orc.F16),      # 16645 rows: last token tile partial, odd head count, batch < pitch
+    (130, 128, 128, 128, 2, 2, 256, 3, orc.BF16),  # 16640 rows, bfloat16, two chunks of K
     (5, 7, 5, 64, 3, 1, 64, 9, orc.F16),           # odd head count, sequences beyond batch_size skipped
     (1, 16, 16, 2048, 32, 4, 256, 100, orc.F16),   # the single-token step of the benchmark model
-    (513, 1, 1, 192, 2, 2, 1024, 3, orc.BF16),     # three token tiles, bfloat16
     (40, 3, 2, 128, 4, 4, 64, 0, orc.BF16),
     # few rows (the weight-streaming kernel): two token blocks x two column blocks, rows through LDS
     (2, 16, 12, 2048, 32, 4, 64, 5, orc.F16),
@@ -105,6 +120,34 @@ def test_matmul3_against_the_oracle(interval, pitch, batch, k, hq, hkv, cap, p0,
     # rows of sequences beyond batch_size and positions outside the call stay untouched (zero)
     assert not got[0][:, batch:].any()
     assert not got[1][batch:].any() and not got[1][:, :, :p0].any() and not got[1][:, :, p0 + interval:].any()
+
+
+def test_cases_reach_every_projection_kernel():
+    seen = {_path((i - 1) * pitch + b, hq + 2 * hkv, k) for (i, pitch, b, k, hq, hkv, _, _, _) in CASES}
+    assert seen == {FEW_ROWS, MID_TILES, TILES}, seen
+    seen = {_path((i - 1) * pitch + b, n // D, k) for (i, pitch, b, k, n, _) in ADD_CASES}
+    assert seen == {FEW_ROWS, MID_TILES, TILES}, seen
+    # the benchmark shapes: 32768 rows on the large tiles, the reference's serving shape
+    # (64 positions x 24 sequences, src/serving/start copy.rs:30) on the small ones
+    assert _path(32768, 40, 2048) == TILES and _path(32768, 16, 4096) == TILES
+    assert _path(64 * 24, 40, 2048) == MID_TILES and _path(64 * 24, 16, 4096) == MID_TILES
+    assert _path(16, 40, 2048) == FEW_ROWS
+
+
+def test_matmul3_ragged_step_of_many_sequences():
+    """A single-token step of more sequences than the few-rows kernel takes: per-sequence
+    positions on the tile kernel."""
+    dtype = orc.F16
+    pitch, batch, k, hq, hkv, cap = 200, 150, 256, 3, 2, 96
+    assert _path(batch, hq + 2 * hkv, k) == MID_TILES
+    hidden = rand_storage((1, pitch, k), 61, dtype)
+    wq, wk, wv = _weights(k, hq, hkv, dtype, 62)
+    rope = _rope_table(cap, dtype)
+    pos = np.random.default_rng(63).integers(0, cap, size=pitch).astype(np.uint32)
+    got, want = _run_matmul3(hidden, wq, wk, wv, rope, dtype, pitch, hq, hkv, cap, 0, 1, batch, positions=pos)
+    for g, w in zip(got, want):
+        assert compare_ulps(g, w, dtype)["ok"]
+    assert not got[1][batch:].any()
 
 
 def test_matmul3_ragged_single_token_step():
@@ -136,16 +179,22 @@ def test_matmul3_in_the_reference_state_layout_and_table_indexing():
     assert got[1][2].any() and not got[1][:2].any() and not got[1][3:].any()     # only position 2 written
 
 
-@pytest.mark.parametrize("interval,pitch,batch,k,n,dtype", [
-    (300, 1, 1, 512, 256, orc.F16),
+ADD_CASES = [
+    (300, 1, 1, 512, 256, orc.F16),                # 128-token tiles
+    (257, 2, 2, 128, 128, orc.F16),
+    (65, 24, 20, 4096, 256, orc.BF16),             # 1556 rows of which 20 in 24 live, K of the benchmark model
+    (4100, 4, 3, 64, 640, orc.F16),                # 256 x 256 tiles: 16399 rows, last tile partial, odd head count
+    (2049, 8, 8, 192, 512, orc.BF16),              # 16392 rows, bfloat16, three chunks of K
     (3, 5, 4, 64, 384, orc.BF16),
     (1, 16, 16, 4096, 2048, orc.F16),              # the output projection of the benchmark model, one token
-    (257, 2, 2, 128, 128, orc.F16),
     (1, 8, 8, 2048, 256, orc.BF16),                # few rows, bfloat16
     (2, 16, 10, 2048, 4096, orc.F16),              # few rows, two token blocks, wide output
     (1, 128, 128, 2048, 256, orc.F16),             # 128 rows, four passes
     (5, 20, 13, 4096, 128, orc.BF16),              # 93 rows of which 65 live, sixteen waves
-])
+]
+
+
+@pytest.mark.parametrize("interval,pitch,batch,k,n,dtype", ADD_CASES)
 def test_matmul_add_against_the_oracle(interval, pitch, batch, k, n, dtype):
     import torch
 
@@ -230,8 +279,8 @@ def test_matmul3_full_size_properties():
 
 
 def test_matmul3_and_matmul_add_random_shapes():
-    """A seeded sweep over shapes that cross every dispatch boundary (few rows / passes / tile
-    kernel, K a multiple of 64 or of 256, one or two column blocks, odd head counts, partial
+    """A seeded sweep over shapes that cross the dispatch boundaries (few rows / passes / small
+    tiles, K a multiple of 64 or of 256, one or two column blocks, odd head counts, partial
     batches, ragged positions)."""
     import torch
 
@@ -247,8 +296,8 @@ def test_matmul3_and_matmul_add_random_shapes():
             hq, hkv = 30, 2                      # wide output: two column blocks in the few-rows kernel
         pitch = int(rng.integers(1, 20))
         batch = int(rng.integers(1, pitch + 1))
-        interval = int(rng.choice([1, 1, 2, 7, 40])) if k <= 1024 else int(rng.choice([1, 1, 3]))
-        cap = 64
+        interval = int(rng.choice([1, 1, 2, 7, 40, 150])) if k <= 1024 else int(rng.choice([1, 1, 3, 30]))
+        cap = 64 if interval <= 64 else 256
         p0 = int(rng.integers(0, cap - interval + 1))
         ragged = interval == 1 and case % 2 == 0
         hidden = rand_storage((interval, pitch, k), 1000 + case, dtype)
