@@ -3,8 +3,11 @@
 // reference's own serving shape of 64 positions x 24 sequences, src/serving/start copy.rs:30,
 // make 6 x 20 of them for the fused Q/K/V projection and 6 x 8 for the output projection).
 // Same formulation (C^T = W . X^T on v_mfma_f32_32x32x16, a lane owns a token), same LDS
-// layout and the same epilogue; the tile is 128 tokens x one head, two workgroups fit a
-// compute unit (the second one fills the gaps a short loop leaves).
+// layout and the same epilogue; the tile is 128 tokens x one head.  A tile this small moves
+// twice the LDS bytes per MFMA, and 128-bit LDS stores are slow (13 cycles an instruction
+// against 4.7 for a read): here the operand tiles go from memory straight into LDS (buffer
+// loads with the LDS bit) through four stages, and the LDS instruction pipe carries the
+// operand reads only.
 #include "project_epilogue.hpp"
 
 namespace ellm {
@@ -14,13 +17,14 @@ namespace {
 constexpr int kMidTokens = 128;                   // tokens per workgroup; output columns: one head
 constexpr int kMidKc = 64;                        // K elements per chunk: one 128-byte line per row
 constexpr int kMidRowPitch = kMidKc * 2;          // unpadded; pieces permuted as in project.hip
-constexpr int kMidStageBytes = (kMidTokens + kHeadDim) * kMidRowPitch;  // X rows then W rows
-constexpr int kMidLdsBytes = 2 * kMidStageBytes;
+constexpr int kMidStageBytes = (kMidTokens + kHeadDim) * kMidRowPitch;  // X rows then W rows: 32 KB
+constexpr int kMidStages = 4;                     // chunk c in stage c % 4, three chunks ahead in flight
+constexpr int kMidLdsBytes = kMidStages * kMidStageBytes;
 constexpr int kMidThreads = 256;
 static_assert(4 * kEpWaveBytes <= kMidLdsBytes, "the epilogue reuses the stages");
 
 template <typename S, int MODE>
-__global__ __launch_bounds__(kMidThreads, 2) void project_mid_kernel(ProjectKernelArgs p) {
+__global__ __launch_bounds__(kMidThreads) void project_mid_kernel(ProjectKernelArgs p) {
   using M = Mfma<S>;
   extern __shared__ __attribute__((aligned(16))) uint8_t mid_smem[];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -40,8 +44,11 @@ __global__ __launch_bounds__(kMidThreads, 2) void project_mid_kernel(ProjectKern
   const uint32_t n_chunks = K / kMidKc;
   const uint32_t row0 = tm * kMidTokens;
   const uint32_t rows_here = min(p.rows - row0, (uint32_t)kMidTokens);
-  const __amdgpu_buffer_rsrc_t x_rsrc = __builtin_amdgcn_make_buffer_rsrc(
-      (void*)(uniform64(p.x) + (uint64_t)row0 * K * 2), 0, rows_here * K * 2, kBufFlags);
+  // (descriptors as four plain words: base, base >> 32, bytes, flags; they go into inline asm)
+  auto make_rsrc = [](uint64_t base, uint32_t bytes) {
+    return u32x4{(uint32_t)base, (uint32_t)(base >> 32) & 0xffffu, bytes, (uint32_t)kBufFlags};
+  };
+  const u32x4 x_rsrc = make_rsrc(uniform64(p.x) + (uint64_t)row0 * K * 2, rows_here * K * 2);
   const uint16_t* wbase = p.w[0];
   uint32_t hs = tn;
   if (tn >= p.heads0 + p.heads_kv) {
@@ -51,28 +58,35 @@ __global__ __launch_bounds__(kMidThreads, 2) void project_mid_kernel(ProjectKern
     wbase = p.w[1];
     hs = tn - p.heads0;
   }
-  const __amdgpu_buffer_rsrc_t w_rsrc = __builtin_amdgcn_make_buffer_rsrc(
-      (void*)(uniform64(wbase) + (uint64_t)hs * kHeadDim * K * 2), 0, kHeadDim * K * 2, kBufFlags);
+  const u32x4 w_rsrc = make_rsrc(uniform64(wbase) + (uint64_t)hs * kHeadDim * K * 2, kHeadDim * K * 2);
 
-  // staging: thread -> row tid / 8 (+ 32 i) of the 128 X rows (i < 4) or the 128 W rows,
-  // 16-byte piece tid % 8 of the chunk's 128 bytes: eight lanes fetch one whole cache line
-  const uint32_t st_row = tid >> 3, st_piece = tid & 7;
+  // staging: lane l of a wave instruction delivers its 16 bytes to M0 + 16 l, so a wave fills
+  // 1 KB = eight whole rows of a stage per instruction; thread -> row tid / 8 (+ 32 i: the 128
+  // X rows for i < 4, then the 128 W rows), LDS piece tid % 8.  The permutation of the pieces
+  // within a row (piece p of row r sits at p ^ ((r >> 1) & 7)) is applied on the memory side:
+  // which piece of the line a lane asks for.  Eight lanes still fetch one whole 128-byte line.
+  // Rows past the end of the activations read zeros.
+  const uint32_t st_row = tid >> 3, st_piece = (tid & 7) ^ ((tid >> 4) & 7);
+  uint32_t src_off[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) src_off[i] = (st_row + 32 * i) * K * 2 + st_piece * 16;
   const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t*)mid_smem;
-  const uint32_t st_store = lds0 + st_row * kMidRowPitch + ((st_piece ^ ((st_row >> 1) & 7)) * 16);
-  u32x4 stg[8];
-  // (a chunk past the last one fetches bytes of the next row, or zeros past the end of the
-  // buffer, into a stage nobody reads)
-  auto load_chunk = [&](uint32_t chunk) {
-    const uint32_t soff = chunk * (kMidKc * 2);
-#pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      const uint32_t off = (st_row + 32 * (i & 3)) * K * 2 + st_piece * 16;
-      stg[i] = __builtin_amdgcn_raw_buffer_load_b128(i < 4 ? x_rsrc : w_rsrc, off, soff, 0);
-    }
+  const uint32_t st_wave = lds0 + (uint32_t)__builtin_amdgcn_readfirstlane(wave) * 1024;
+  // Written as asm: the compiler's own form of this load makes it wait for every outstanding
+  // one before each later LDS read (it cannot see that the two touch different stages).  M0
+  // carries the LDS address of the wave's 1 KB; one wait state between its write and the load.
+  // (M0 is a register the compiler reserves and, in this kernel, never uses itself.)
+  auto load_lds = [](const u32x4& rsrc, uint32_t voff, uint32_t soff, uint32_t lds_at) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
+                 :: "s"(lds_at), "v"(voff), "s"(rsrc), "s"(soff) : "memory");
   };
-  auto store_chunk = [&](uint32_t stage) {
-#pragma unroll
-    for (int i = 0; i < 8; ++i) *(LdsVec4*)(st_store + stage + 32 * i * kMidRowPitch) = stg[i];
+  // A chunk past the last one is requested through descriptors of size zero: no memory
+  // access, zeros into a stage nobody reads, and every iteration issues the same eight loads.
+  const u32x4 none_rsrc = make_rsrc(uniform64(p.x), 0);
+  auto load_piece = [&](uint32_t chunk, int i) {
+    const uint32_t to = st_wave + (chunk % kMidStages) * kMidStageBytes + 4096 * i;
+    const bool real = chunk < n_chunks;
+    load_lds(real ? (i < 4 ? x_rsrc : w_rsrc) : none_rsrc, src_off[i & 3], chunk * (kMidKc * 2), to);
   };
 
   f32x16 acc[4][1];  // [column block nb][token block]
@@ -85,7 +99,6 @@ __global__ __launch_bounds__(kMidThreads, 2) void project_mid_kernel(ProjectKern
   const uint32_t swz = (j >> 1) & 7;
   const uint32_t x_row = lds0 + (wave * 32 + j) * kMidRowPitch;
   const uint32_t w_row = lds0 + (kMidTokens + j) * kMidRowPitch;
-
   // operands of one 16-wide step: the X block of this wave and the head's four W blocks
   u32x4 ox[2], ow[2][4];
   auto read_operand = [&](auto set_, uint32_t stage, int st, int o) {
@@ -96,27 +109,28 @@ __global__ __launch_bounds__(kMidThreads, 2) void project_mid_kernel(ProjectKern
     else
       ow[set][o - 1] = *(const LdsVec4*)(w_row + stage + 32 * (o - 1) * kMidRowPitch + piece);
   };
-  auto load_piece = [&](uint32_t chunk, int i) {
-    const uint32_t off = (st_row + 32 * (i & 3)) * K * 2 + st_piece * 16;
-    stg[i] = __builtin_amdgcn_raw_buffer_load_b128(i < 4 ? x_rsrc : w_rsrc, off, chunk * (kMidKc * 2), 0);
-  };
 
-  load_chunk(0);
-  store_chunk(0);
-  load_chunk(1);
+  // prologue: chunks 0, 1, 2 on their way; chunk 0 has landed in every wave's rows
+#pragma unroll
+  for (int k = 0; k < kMidStages - 1; ++k)
+#pragma unroll
+    for (int i = 0; i < 8; ++i) load_piece(k, i);
+  asm volatile("s_waitcnt vmcnt(16)" ::: "memory");
   __syncthreads();
 #pragma unroll
   for (int o = 0; o < 5; ++o) read_operand(std::integral_constant<int, 0>{}, 0, 0, o);
 
   // One iteration = one chunk = four 16-wide steps of four MFMAs.  The operands of a step
-  // are read during the step before it, across chunks too; the staging registers (chunk
-  // c + 1, requested an iteration earlier) are stored during steps 0-2 and refilled with
-  // chunk c + 2 during step 3.  One barrier, after step 2.  It orders both hazards: the
-  // stage that this iteration's stores fill (chunk c - 1's) was last read for step 3 of
-  // chunk c - 1, and those reads had returned before the previous barrier; and chunk c + 1
-  // is complete before the reads of its first step, issued during step 3.
+  // are read during the step before it, across chunks too.  During steps 0-1 chunk c + 3 is
+  // requested into the stage chunk c - 1 has left; after step 2 the wave waits for its own
+  // pieces of chunk c + 1 (requested two iterations ago: all but the 16 youngest loads) and
+  // meets the others at the one barrier of the iteration.  The barrier orders both hazards:
+  // the stage being refilled was last read for step 3 of chunk c - 1, and those reads had
+  // returned before the previous barrier; and chunk c + 1 is complete before the reads of
+  // its first step, issued during step 3.
   for (uint32_t c = 0; c < n_chunks; ++c) {
-    const uint32_t cur = (c & 1) * kMidStageBytes, nxt = kMidStageBytes - cur;
+    const uint32_t cur = (c % kMidStages) * kMidStageBytes;
+    const uint32_t nxt = ((c + 1) % kMidStages) * kMidStageBytes;
     __builtin_amdgcn_sched_barrier(0);
     static_for<16>([&](auto n_) {
       constexpr int n = decltype(n_)::value;
@@ -128,20 +142,17 @@ __global__ __launch_bounds__(kMidThreads, 2) void project_mid_kernel(ProjectKern
       constexpr int next_st = (st + 1) & 3;
       read_operand(std::integral_constant<int, 1 - set>{}, from, next_st, nb == 0 ? 0 : nb + 1);
       if constexpr (nb == 0) read_operand(std::integral_constant<int, 1 - set>{}, from, next_st, 1);
-      if constexpr (st < 3) {
-        // eight staging stores over twelve MFMAs
-        if constexpr (n % 3 != 2) *(LdsVec4*)(st_store + nxt + 32 * (n - n / 3) * kMidRowPitch) = stg[n - n / 3];
-      } else {
-        load_piece(c + 2, 2 * nb);
-        load_piece(c + 2, 2 * nb + 1);
-      }
+      if constexpr (n < 8) load_piece(c + kMidStages - 1, n);
       if constexpr (n == 11) {
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+        // this wave's pieces of chunk c + 1 are in LDS, and its reads of this chunk's stage
+        // have returned
+        asm volatile("s_waitcnt vmcnt(16) lgkmcnt(0)" ::: "memory");
         __builtin_amdgcn_s_barrier();
       }
       __builtin_amdgcn_sched_barrier(0);
     });
   }
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the last (empty) requests still write LDS
   __syncthreads();
   finish_head<S, MODE, 1>(p, acc, tn, row0 + 32 * wave, lds0 + wave * kEpWaveBytes, lane);
 }
