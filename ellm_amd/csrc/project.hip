@@ -21,7 +21,8 @@
 // 128-byte cache line per operand row and chunk: a fetch of half a line costs the vector
 // cache the same miss entry as a whole one) through two LDS stages: chunk c is read while
 // chunk c + 1, fetched into registers an iteration earlier, is written to the other stage.
-// Calls with at most 128 rows go to the streaming kernel of project_small.hip instead.
+// Calls with at most 64 rows go to the streaming kernel of project_small.hip, calls that would
+// leave these tiles fewer than the compute units to the 128-token tiles of project_mid.hip.
 #include "project_epilogue.hpp"
 
 namespace ellm {

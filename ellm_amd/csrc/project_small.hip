@@ -1,4 +1,4 @@
-// Projections for up to 128 token rows (a single-token step over that many sequences, a
+// Projections for up to 64 token rows (a single-token step over that many sequences, a
 // short chunk): the weights are read exactly once and the kernel is bound by that stream
 // (HBM), not by MFMA.  Same arithmetic and epilogue as the tile kernel of project.hip.
 //

@@ -337,7 +337,7 @@ int ellm_matmul_add_destroy(ellm_matmul_add* handle);
  * Which of the three projection kernels a call with `rows` activation rows
  * ((position_interval - 1) * batch capacity + batch_size), `heads` output column groups
  * of 128 (attention_head_num + 2 * kv_head_num, or n / 128) and inner size k runs on the
- * current device: 0 = the weight-streaming kernel for at most 128 rows, 1 = 128-token x
+ * current device: 0 = the weight-streaming kernel for at most 64 rows, 1 = 128-token x
  * one-head MFMA tiles, 2 = 256 x 256 MFMA tiles; -1 for sizes no handle accepts.  No
  * counterpart in the reference (its MatMul3::run has one code path); it lets a test or a
  * harness see that its shapes reach every kernel.

@@ -101,10 +101,14 @@ CASES = [
     (1, 16, 16, 1024, 4, 2, 64, 9, orc.BF16),      # four waves, one column block
     (1, 8, 8, 8192, 2, 1, 32, 3, orc.F16),         # two rounds of K per wave, operands fetched directly
     (2, 12, 12, 4096, 34, 2, 32, 1, orc.F16),      # wide output but rows too long for two column blocks in LDS
-    # 33 .. 128 rows: several passes over weight operands kept in registers
-    (1, 100, 97, 2048, 32, 4, 64, 7, orc.F16),     # 97 rows: four passes of two token blocks, last one partial
-    (3, 40, 40, 1024, 6, 2, 64, 2, orc.BF16),      # 120 rows, four waves: eight passes of one token block
-    (2, 64, 64, 4096, 3, 1, 32, 0, orc.F16),       # 128 rows, sixteen waves
+    # 33 .. 64 rows: several passes over weight operands kept in registers
+    (1, 60, 57, 2048, 32, 4, 64, 7, orc.F16),      # 57 rows: two passes of two token blocks, last one partial
+    (3, 20, 20, 1024, 6, 2, 64, 2, orc.BF16),      # 60 rows, four waves: four passes of one token block
+    (2, 32, 32, 4096, 3, 1, 32, 0, orc.F16),       # 64 rows, sixteen waves
+    # 65 .. 128 rows: one 128-token tile per head
+    (1, 100, 97, 2048, 32, 4, 64, 7, orc.F16),
+    (3, 40, 40, 1024, 6, 2, 64, 2, orc.BF16),
+    (2, 64, 64, 4096, 3, 1, 32, 0, orc.F16),
 ]
 
 
@@ -189,8 +193,10 @@ ADD_CASES = [
     (1, 16, 16, 4096, 2048, orc.F16),              # the output projection of the benchmark model, one token
     (1, 8, 8, 2048, 256, orc.BF16),                # few rows, bfloat16
     (2, 16, 10, 2048, 4096, orc.F16),              # few rows, two token blocks, wide output
-    (1, 128, 128, 2048, 256, orc.F16),             # 128 rows, four passes
-    (5, 20, 13, 4096, 128, orc.BF16),              # 93 rows of which 65 live, sixteen waves
+    (1, 64, 64, 2048, 256, orc.F16),               # 64 rows, two passes
+    (3, 20, 13, 4096, 128, orc.BF16),              # 53 rows of which 39 live, sixteen waves
+    (1, 128, 128, 2048, 256, orc.F16),             # 128 rows: one 128-token tile per head
+    (5, 20, 13, 4096, 128, orc.BF16),              # 93 rows of which 65 live
 ]
 
 
