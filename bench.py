@@ -488,8 +488,9 @@ def bench_layer_step(layers, batch, length, steps, warmup, hidden=2048, hq=32, h
     return {"eager_ms": eager_ms, "graph_ms": graph_ms, "kv_bytes": kv_bytes, "w_bytes": w_bytes}
 
 
-def cpu_baseline_decode(batch, length, hq=32, hkv=4, budget_s=20.0):
-    """The CPU oracle on the full single-token workload (all host cores)."""
+def cpu_baseline_decode(batch, length, hq=32, hkv=4, budget_s=1.5):
+    """The CPU oracle on the full single-token workload (all host cores), repeated for about
+    `budget_s` seconds of wall time (x 16 threads: 20-odd core-seconds of CPU work)."""
     import numpy as np
     import oracle_lib as orc
 
@@ -502,7 +503,7 @@ def cpu_baseline_decode(batch, length, hq=32, hkv=4, budget_s=20.0):
     op = orc.Operator(q, k, v, out, None, batch, hq, hkv, D, [hkv * length * D, length * D, D, 1],
                       1.0 / D ** 0.5, orc.F16)
     t1 = op.run_threads(length - 1, 1, batch, cores, pin=False)
-    repeats = max(1, min(10, int(budget_s / max(t1, 1e-3)) - 1))
+    repeats = max(1, min(200, int(budget_s / max(t1, 1e-3))))
     t = op.run_threads(length - 1, 1, batch, cores, pin=False, repeats=repeats) / repeats
     alg_bytes = 2 * batch * hkv * length * D * 2 + 2 * batch * hq * D * 2
     return {
