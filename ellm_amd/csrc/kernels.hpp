@@ -112,7 +112,7 @@ hipError_t launch_project(const ProjectArgs& a, hipStream_t stream);
 // Few-rows kernel: rows it handles at most, floats of partial sums and counters it needs.
 size_t project_workspace_floats(uint32_t heads, uint32_t K);
 // The kernel a projection of this shape runs (heads = 128-wide output column groups).
-enum { kPathFewRows = 0, kPathMidTiles = 1, kPathTiles = 2 };
+enum { kPathFewRows = 0, kPathTiles128 = 1, kPathTiles256x1 = 2, kPathTiles = 3 };
 int project_path(uint32_t rows, uint32_t heads, uint32_t K, bool has_workspace);
 // Per-device set-up of the projection kernels (LDS limits); call with the device current.
 hipError_t project_prepare();

@@ -211,14 +211,15 @@ __global__ __launch_bounds__(kProjThreads) void project_kernel(ProjectKernelArgs
 static uint32_t g_n_cu = 256;
 
 // Which kernel a call runs: the few-rows streaming kernel when the handle has its workspace
-// and the shape fits it; else 128-token x one-head tiles when the 256 x 256 tiles would leave
-// compute units idle and the small tiles are all resident at once (two per compute unit:
-// beyond that the large tiles' lower traffic per flop wins, measured); else 256 x 256 tiles.
+// and the shape fits it; else the smallest tile whose workgroups all fit the part at once, one
+// per compute unit (128 tokens x one head, then 256 tokens x one head); else 256 x 256 tiles,
+// whose traffic per flop is the lowest.  Measured on 256 compute units for 2048 -> 5120: 128-token
+// tiles 20 us up to 768 rows, 256-token tiles 38-42 us up to 1536 rows (128-token tiles in two
+// rounds: 40-44 us), 256 x 256 tiles 58 us at 2048 rows (61 and 70 us for the other two).
 int project_path(uint32_t rows, uint32_t heads, uint32_t K, bool has_workspace) {
   if (has_workspace && small_kernel_takes(rows, K)) return kPathFewRows;
-  const uint32_t big = ((rows + kTile - 1) / kTile) * ((heads + 1) / 2);
-  const uint32_t mid = ((rows + 127) / 128) * heads;
-  if (big < g_n_cu && mid <= 2 * g_n_cu) return kPathMidTiles;
+  if (((rows + 127) / 128) * heads <= g_n_cu) return kPathTiles128;
+  if (((rows + 255) / 256) * heads <= g_n_cu) return kPathTiles256x1;
   return kPathTiles;
 }
 
@@ -256,7 +257,8 @@ hipError_t launch_project(const ProjectArgs& a, hipStream_t stream) {
   const int path = project_path(a.rows, a.heads0 + 2 * a.heads_kv, a.K, a.ws && a.counters);
   if (path == kPathFewRows)
     return launch_project_small(p, a.ws, a.counters, a.dtype, a.residual != nullptr, stream);
-  if (path == kPathMidTiles) return launch_project_mid(p, a.dtype, a.residual != nullptr, stream);
+  if (path == kPathTiles128 || path == kPathTiles256x1)
+    return launch_project_mid(p, path == kPathTiles128 ? 1 : 2, a.dtype, a.residual != nullptr, stream);
   const uint32_t blocks = p.tiles_m * p.tiles_n;
   auto go = [&](auto kernel) {
     hipLaunchKernelGGL(kernel, dim3(blocks), dim3(kProjThreads), kProjLdsBytes, stream, p);

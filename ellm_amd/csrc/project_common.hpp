@@ -62,7 +62,9 @@ hipError_t launch_project_small(const ProjectKernelArgs& p, float* ws, uint32_t*
 // Tile kernel with 128-token x one-head tiles (project_mid.hip), for row counts at which
 // the 256 x 256 tiles are fewer than the compute units.
 hipError_t mid_prepare();
-hipError_t launch_project_mid(ProjectKernelArgs p, int dtype, bool add, hipStream_t stream);
+// token_blocks: 1 = 128-token tiles, 2 = 256-token tiles
+hipError_t launch_project_mid(ProjectKernelArgs p, uint32_t token_blocks, int dtype, bool add,
+                              hipStream_t stream);
 
 }  // namespace proj
 }  // namespace ellm

@@ -3,10 +3,11 @@
 // reference's own serving shape of 64 positions x 24 sequences, src/serving/start copy.rs:30,
 // make 6 x 20 of them for the fused Q/K/V projection and 6 x 8 for the output projection).
 // Same formulation (C^T = W . X^T on v_mfma_f32_32x32x16, a lane owns a token), same LDS
-// layout and the same epilogue; the tile is 128 tokens x one head.  A tile this small moves
-// twice the LDS bytes per MFMA, and 128-bit LDS stores are slow (13 cycles an instruction
-// against 4.7 for a read): here the operand tiles go from memory straight into LDS (buffer
-// loads with the LDS bit) through four stages, and the LDS instruction pipe carries the
+// layout and the same epilogue; the tile is 128 or 256 tokens x one head (a wave owns one or
+// two 32-token blocks x the head's four column blocks).  Tiles this small move up to twice
+// the LDS bytes per MFMA, and 128-bit LDS stores are slow (13 cycles an instruction against
+// 4.7 for a read): here the operand tiles go from memory straight into LDS (buffer loads
+// with the LDS bit) through four (three) stages, and the LDS instruction pipe carries the
 // operand reads only.
 #include "project_epilogue.hpp"
 
@@ -14,18 +15,27 @@ namespace ellm {
 namespace proj {
 namespace {
 
-constexpr int kMidTokens = 128;                   // tokens per workgroup; output columns: one head
 constexpr int kMidKc = 64;                        // K elements per chunk: one 128-byte line per row
 constexpr int kMidRowPitch = kMidKc * 2;          // unpadded; pieces permuted as in project.hip
-constexpr int kMidStageBytes = (kMidTokens + kHeadDim) * kMidRowPitch;  // X rows then W rows: 32 KB
-constexpr int kMidStages = 4;                     // chunk c in stage c % 4, three chunks ahead in flight
-constexpr int kMidLdsBytes = kMidStages * kMidStageBytes;
 constexpr int kMidThreads = 256;
-static_assert(4 * kEpWaveBytes <= kMidLdsBytes, "the epilogue reuses the stages");
+// MB = 32-token blocks per wave: the tile is 128 MB tokens x one head.
+template <int MB>
+struct MidShape {
+  static constexpr int kTokens = 128 * MB;
+  static constexpr int kStageBytes = (kTokens + kHeadDim) * kMidRowPitch;  // X rows then W rows: 32 or 48 KB
+  static constexpr int kStages = MB == 1 ? 4 : 3;   // chunk c in stage c % kStages
+  static constexpr int kLdsBytes = kStages * kStageBytes;
+  static constexpr int kLoads = 4 * MB + 4;         // 1 KB wave loads per chunk and wave
+  static constexpr int kAhead = kStages - 1;        // chunks requested ahead of the one being multiplied
+  static_assert(4 * kEpWaveBytes <= kLdsBytes, "the epilogue reuses the stages");
+  static_assert(kLdsBytes <= 160 * 1024, "LDS of a compute unit");
+};
 
-template <typename S, int MODE>
+template <typename S, int MODE, int MB>
 __global__ __launch_bounds__(kMidThreads) void project_mid_kernel(ProjectKernelArgs p) {
   using M = Mfma<S>;
+  using Shape = MidShape<MB>;
+  constexpr int kStageBytes = Shape::kStageBytes, kStages = Shape::kStages, kLoads = Shape::kLoads;
   extern __shared__ __attribute__((aligned(16))) uint8_t mid_smem[];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int j = lane & 31, g = lane >> 5;
@@ -42,8 +52,8 @@ __global__ __launch_bounds__(kMidThreads) void project_mid_kernel(ProjectKernelA
   }
   const uint32_t K = p.K;
   const uint32_t n_chunks = K / kMidKc;
-  const uint32_t row0 = tm * kMidTokens;
-  const uint32_t rows_here = min(p.rows - row0, (uint32_t)kMidTokens);
+  const uint32_t row0 = tm * Shape::kTokens;
+  const uint32_t rows_here = min(p.rows - row0, (uint32_t)Shape::kTokens);
   // (descriptors as four plain words: base, base >> 32, bytes, flags; they go into inline asm)
   auto make_rsrc = [](uint64_t base, uint32_t bytes) {
     return u32x4{(uint32_t)base, (uint32_t)(base >> 32) & 0xffffu, bytes, (uint32_t)kBufFlags};
@@ -61,15 +71,15 @@ __global__ __launch_bounds__(kMidThreads) void project_mid_kernel(ProjectKernelA
   const u32x4 w_rsrc = make_rsrc(uniform64(wbase) + (uint64_t)hs * kHeadDim * K * 2, kHeadDim * K * 2);
 
   // staging: lane l of a wave instruction delivers its 16 bytes to M0 + 16 l, so a wave fills
-  // 1 KB = eight whole rows of a stage per instruction; thread -> row tid / 8 (+ 32 i: the 128
-  // X rows for i < 4, then the 128 W rows), LDS piece tid % 8.  The permutation of the pieces
+  // 1 KB = eight whole rows of a stage per instruction; thread -> row tid / 8 (+ 32 i: the
+  // X rows for i < 4 MB, then the 128 W rows), LDS piece tid % 8.  The permutation of the pieces
   // within a row (piece p of row r sits at p ^ ((r >> 1) & 7)) is applied on the memory side:
   // which piece of the line a lane asks for.  Eight lanes still fetch one whole 128-byte line.
   // Rows past the end of the activations read zeros.
   const uint32_t st_row = tid >> 3, st_piece = (tid & 7) ^ ((tid >> 4) & 7);
-  uint32_t src_off[4];
+  uint32_t src_off[4 * MB];
 #pragma unroll
-  for (int i = 0; i < 4; ++i) src_off[i] = (st_row + 32 * i) * K * 2 + st_piece * 16;
+  for (int i = 0; i < 4 * MB; ++i) src_off[i] = (st_row + 32 * i) * K * 2 + st_piece * 16;
   const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t*)mid_smem;
   const uint32_t st_wave = lds0 + (uint32_t)__builtin_amdgcn_readfirstlane(wave) * 1024;
   // Written as asm: the compiler's own form of this load makes it wait for every outstanding
@@ -84,69 +94,87 @@ __global__ __launch_bounds__(kMidThreads) void project_mid_kernel(ProjectKernelA
   // access, zeros into a stage nobody reads, and every iteration issues the same eight loads.
   const u32x4 none_rsrc = make_rsrc(uniform64(p.x), 0);
   auto load_piece = [&](uint32_t chunk, int i) {
-    const uint32_t to = st_wave + (chunk % kMidStages) * kMidStageBytes + 4096 * i;
+    const uint32_t to = st_wave + (chunk % kStages) * kStageBytes + 4096 * i;
     const bool real = chunk < n_chunks;
-    load_lds(real ? (i < 4 ? x_rsrc : w_rsrc) : none_rsrc, src_off[i & 3], chunk * (kMidKc * 2), to);
+    load_lds(real ? (i < 4 * MB ? x_rsrc : w_rsrc) : none_rsrc, src_off[i < 4 * MB ? i : i - 4 * MB],
+             chunk * (kMidKc * 2), to);
   };
 
-  f32x16 acc[4][1];  // [column block nb][token block]
+  f32x16 acc[4][MB];  // [column block nb][token block mb]
 #pragma unroll
   for (int nb = 0; nb < 4; ++nb)
 #pragma unroll
-    for (int r = 0; r < 16; ++r) acc[nb][0][r] = 0.0f;
+    for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[nb][mb][r] = 0.0f;
 
   // operand reads: lane (j, g) takes row j of a 32-row block, piece 2 step + g, permuted
   const uint32_t swz = (j >> 1) & 7;
-  const uint32_t x_row = lds0 + (wave * 32 + j) * kMidRowPitch;
-  const uint32_t w_row = lds0 + (kMidTokens + j) * kMidRowPitch;
-  // operands of one 16-wide step: the X block of this wave and the head's four W blocks
-  u32x4 ox[2], ow[2][4];
+  const uint32_t x_row = lds0 + (wave * 32 * MB + j) * kMidRowPitch;
+  const uint32_t w_row = lds0 + (Shape::kTokens + j) * kMidRowPitch;
+  // operands of one 16-wide step: the wave's MB X blocks (o < MB), then the head's four W blocks
+  constexpr int kOps = MB + 4;
+  u32x4 ops[2][kOps];
   auto read_operand = [&](auto set_, uint32_t stage, int st, int o) {
     constexpr int set = decltype(set_)::value;
     const uint32_t piece = ((2 * st + g) ^ swz) * 16;
-    if (o == 0)
-      ox[set] = *(const LdsVec4*)(x_row + stage + piece);
+    if (o < MB)
+      ops[set][o] = *(const LdsVec4*)(x_row + stage + 32 * o * kMidRowPitch + piece);
     else
-      ow[set][o - 1] = *(const LdsVec4*)(w_row + stage + 32 * (o - 1) * kMidRowPitch + piece);
+      ops[set][o] = *(const LdsVec4*)(w_row + stage + 32 * (o - MB) * kMidRowPitch + piece);
   };
 
-  // prologue: chunks 0, 1, 2 on their way; chunk 0 has landed in every wave's rows
+  // prologue: the first kAhead chunks on their way; chunk 0 has landed in every wave's rows
 #pragma unroll
-  for (int k = 0; k < kMidStages - 1; ++k)
+  for (int k = 0; k < Shape::kAhead; ++k)
 #pragma unroll
-    for (int i = 0; i < 8; ++i) load_piece(k, i);
-  asm volatile("s_waitcnt vmcnt(16)" ::: "memory");
+    for (int i = 0; i < kLoads; ++i) load_piece(k, i);
+  if constexpr (MB == 1)
+    asm volatile("s_waitcnt vmcnt(16)" ::: "memory");   // (kAhead - 1) * kLoads
+  else
+    asm volatile("s_waitcnt vmcnt(12)" ::: "memory");
   __syncthreads();
 #pragma unroll
-  for (int o = 0; o < 5; ++o) read_operand(std::integral_constant<int, 0>{}, 0, 0, o);
+  for (int o = 0; o < kOps; ++o) read_operand(std::integral_constant<int, 0>{}, 0, 0, o);
 
-  // One iteration = one chunk = four 16-wide steps of four MFMAs.  The operands of a step
-  // are read during the step before it, across chunks too.  During steps 0-1 chunk c + 3 is
-  // requested into the stage chunk c - 1 has left; after step 2 the wave waits for its own
-  // pieces of chunk c + 1 (requested two iterations ago: all but the 16 youngest loads) and
-  // meets the others at the one barrier of the iteration.  The barrier orders both hazards:
-  // the stage being refilled was last read for step 3 of chunk c - 1, and those reads had
-  // returned before the previous barrier; and chunk c + 1 is complete before the reads of
-  // its first step, issued during step 3.
+  // One iteration = one chunk = four 16-wide steps of 4 MB MFMAs.  The operands of a step
+  // are read during the step before it, across chunks too.  During steps 0-1 chunk c + kAhead
+  // is requested into the stage chunk c - 1 has left; after step 2 the wave waits for its own
+  // pieces of chunk c + 1 (all but the loads of the chunks after it) and meets the others at
+  // the one barrier of the iteration.  The barrier orders both hazards: the stage being
+  // refilled was last read for step 3 of chunk c - 1, and those reads had returned before the
+  // previous barrier; and chunk c + 1 is complete before the reads of its first step, issued
+  // during step 3.
+  constexpr int kPerStep = 4 * MB;
   for (uint32_t c = 0; c < n_chunks; ++c) {
-    const uint32_t cur = (c % kMidStages) * kMidStageBytes;
-    const uint32_t nxt = ((c + 1) % kMidStages) * kMidStageBytes;
+    const uint32_t cur = (c % kStages) * kStageBytes;
+    const uint32_t nxt = ((c + 1) % kStages) * kStageBytes;
     __builtin_amdgcn_sched_barrier(0);
-    static_for<16>([&](auto n_) {
+    static_for<4 * kPerStep>([&](auto n_) {
       constexpr int n = decltype(n_)::value;
-      constexpr int st = n >> 2, nb = n & 3;
+      constexpr int st = n / kPerStep, m = n % kPerStep;
+      constexpr int mb = m % MB, nb = m / MB;
       constexpr int set = st & 1;
-      acc[nb][0] = M::m32x32x16(ow[set][nb], ox[set], acc[nb][0]);
-      // five reads for the next step over this step's four MFMAs
+      acc[nb][mb] = M::m32x32x16(ops[set][MB + nb], ops[set][mb], acc[nb][mb]);
+      // the next step's MB + 4 operands, read over this step's MFMAs (two after the first)
       const uint32_t from = (st < 3) ? cur : nxt;
       constexpr int next_st = (st + 1) & 3;
-      read_operand(std::integral_constant<int, 1 - set>{}, from, next_st, nb == 0 ? 0 : nb + 1);
-      if constexpr (nb == 0) read_operand(std::integral_constant<int, 1 - set>{}, from, next_st, 1);
-      if constexpr (n < 8) load_piece(c + kMidStages - 1, n);
-      if constexpr (n == 11) {
+      if constexpr (m == 0) {
+        read_operand(std::integral_constant<int, 1 - set>{}, from, next_st, 0);
+        read_operand(std::integral_constant<int, 1 - set>{}, from, next_st, MB);
+      } else if constexpr (m < kOps - 1) {
+        // remaining X blocks first (MB == 2: block 1), then W blocks 1..3
+        constexpr int o = (m < MB) ? m : m + 1;
+        read_operand(std::integral_constant<int, 1 - set>{}, from, next_st, o);
+      }
+      if constexpr (n < kLoads) load_piece(c + Shape::kAhead, n);
+      if constexpr (n == 3 * kPerStep - 1) {
         // this wave's pieces of chunk c + 1 are in LDS, and its reads of this chunk's stage
         // have returned
-        asm volatile("s_waitcnt vmcnt(16) lgkmcnt(0)" ::: "memory");
+        if constexpr (MB == 1)
+          asm volatile("s_waitcnt vmcnt(16) lgkmcnt(0)" ::: "memory");
+        else
+          asm volatile("s_waitcnt vmcnt(12) lgkmcnt(0)" ::: "memory");
         __builtin_amdgcn_s_barrier();
       }
       __builtin_amdgcn_sched_barrier(0);
@@ -154,33 +182,47 @@ __global__ __launch_bounds__(kMidThreads) void project_mid_kernel(ProjectKernelA
   }
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the last (empty) requests still write LDS
   __syncthreads();
-  finish_head<S, MODE, 1>(p, acc, tn, row0 + 32 * wave, lds0 + wave * kEpWaveBytes, lane);
+  finish_head<S, MODE, MB>(p, acc, tn, row0 + 32 * MB * wave, lds0 + wave * kEpWaveBytes, lane);
 }
 
-}  // namespace
-
-hipError_t mid_prepare() {
-  const void* kernels[] = {
-      (const void*)project_mid_kernel<F16, kModeQkv>, (const void*)project_mid_kernel<BF16, kModeQkv>,
-      (const void*)project_mid_kernel<F16, kModeAdd>, (const void*)project_mid_kernel<BF16, kModeAdd>};
+template <int MB>
+hipError_t prepare_shape() {
+  const void* kernels[] = {(const void*)project_mid_kernel<F16, kModeQkv, MB>,
+                           (const void*)project_mid_kernel<BF16, kModeQkv, MB>,
+                           (const void*)project_mid_kernel<F16, kModeAdd, MB>,
+                           (const void*)project_mid_kernel<BF16, kModeAdd, MB>};
   for (const void* k : kernels) {
     const hipError_t e =
-        hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, kMidLdsBytes);
+        hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, MidShape<MB>::kLdsBytes);
     if (e != hipSuccess) return e;
   }
   return hipSuccess;
 }
 
-hipError_t launch_project_mid(ProjectKernelArgs p, int dtype, bool add, hipStream_t stream) {
-  p.tiles_m = (p.rows + kMidTokens - 1) / kMidTokens;
+template <int MB>
+hipError_t launch_shape(ProjectKernelArgs p, int dtype, bool add, hipStream_t stream) {
+  p.tiles_m = (p.rows + MidShape<MB>::kTokens - 1) / MidShape<MB>::kTokens;
   p.tiles_n = p.heads0 + 2 * p.heads_kv;
   const uint32_t blocks = p.tiles_m * p.tiles_n;
   auto go = [&](auto kernel) {
-    hipLaunchKernelGGL(kernel, dim3(blocks), dim3(kMidThreads), kMidLdsBytes, stream, p);
+    hipLaunchKernelGGL(kernel, dim3(blocks), dim3(kMidThreads), MidShape<MB>::kLdsBytes, stream, p);
     return hipGetLastError();
   };
-  if (add) return dtype == 0 ? go(project_mid_kernel<F16, kModeAdd>) : go(project_mid_kernel<BF16, kModeAdd>);
-  return dtype == 0 ? go(project_mid_kernel<F16, kModeQkv>) : go(project_mid_kernel<BF16, kModeQkv>);
+  if (add)
+    return dtype == 0 ? go(project_mid_kernel<F16, kModeAdd, MB>) : go(project_mid_kernel<BF16, kModeAdd, MB>);
+  return dtype == 0 ? go(project_mid_kernel<F16, kModeQkv, MB>) : go(project_mid_kernel<BF16, kModeQkv, MB>);
+}
+
+}  // namespace
+
+hipError_t mid_prepare() {
+  const hipError_t e = prepare_shape<1>();
+  return e != hipSuccess ? e : prepare_shape<2>();
+}
+
+hipError_t launch_project_mid(ProjectKernelArgs p, uint32_t token_blocks, int dtype, bool add,
+                              hipStream_t stream) {
+  return token_blocks == 2 ? launch_shape<2>(p, dtype, add, stream) : launch_shape<1>(p, dtype, add, stream);
 }
 
 }  // namespace proj

@@ -334,11 +334,12 @@ int ellm_matmul_add_run(ellm_matmul_add* handle, size_t position_index, size_t p
 int ellm_matmul_add_destroy(ellm_matmul_add* handle);
 
 /*
- * Which of the three projection kernels a call with `rows` activation rows
+ * Which projection kernel and tile shape a call with `rows` activation rows
  * ((position_interval - 1) * batch capacity + batch_size), `heads` output column groups
  * of 128 (attention_head_num + 2 * kv_head_num, or n / 128) and inner size k runs on the
- * current device: 0 = the weight-streaming kernel for at most 64 rows, 1 = 128-token x
- * one-head MFMA tiles, 2 = 256 x 256 MFMA tiles; -1 for sizes no handle accepts.  No
+ * current device: 0 = the weight-streaming kernel for at most 64 rows, 1 = MFMA tiles of
+ * 128 tokens x one head, 2 = tiles of 256 tokens x one head, 3 = tiles of 256 tokens x two
+ * heads; -1 for sizes no handle accepts.  No
  * counterpart in the reference (its MatMul3::run has one code path); it lets a test or a
  * harness see that its shapes reach every kernel.
  */

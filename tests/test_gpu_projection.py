@@ -74,7 +74,7 @@ def _weights(k, hq, hkv, dtype, seed):
             rand_storage((hkv * D, k), seed + 2, dtype, scale=s))
 
 
-FEW_ROWS, MID_TILES, TILES = 0, 1, 2     # ellm_projection_path
+FEW_ROWS, TILES_128, TILES_256X1, TILES_256X2 = 0, 1, 2, 3     # ellm_projection_path
 
 
 def _path(rows, heads, k):
@@ -85,11 +85,13 @@ def _path(rows, heads, k):
 
 CASES = [
     # interval, pitch, batch, k, hq, hkv, cap, p0, dtype
-    # 128-token x one-head tiles (more than 128 rows, too few for 256 x 256 tiles to fill the part)
+    # 128-token x one-head tiles (more than 64 rows, and no more tiles than compute units)
     (300, 1, 1, 256, 8, 2, 512, 17, orc.F16),      # three token tiles, the last partial
     (513, 1, 1, 192, 2, 2, 1024, 3, orc.BF16),     # five token tiles, bfloat16
-    (9, 100, 97, 2048, 32, 4, 64, 7, orc.F16),     # 897 rows of the benchmark model, sequences beyond batch_size skipped
     (33, 5, 4, 64, 3, 1, 64, 9, orc.BF16),         # one chunk of K, odd head count
+    # 256-token x one-head tiles
+    (9, 100, 97, 2048, 32, 4, 64, 7, orc.F16),     # 897 rows of the benchmark model, sequences beyond batch_size skipped
+    (79, 128, 101, 64, 3, 1, 128, 5, orc.BF16),    # 10085 rows: last tile partial, odd head count, one chunk of K
     # 256 x 256 tiles (many rows; K kept small so that the oracle stays quick)
     (2081, 8, 5, 64, 3, 1, 4096, 9, orc.F16),      # 16645 rows: last token tile partial, odd head count, batch < pitch
     (130, 128, 128, 128, 2, 2, 256, 3, orc.BF16),  # 16640 rows, bfloat16, two chunks of K
@@ -128,13 +130,14 @@ def test_matmul3_against_the_oracle(interval, pitch, batch, k, hq, hkv, cap, p0,
 
 def test_cases_reach_every_projection_kernel():
     seen = {_path((i - 1) * pitch + b, hq + 2 * hkv, k) for (i, pitch, b, k, hq, hkv, _, _, _) in CASES}
-    assert seen == {FEW_ROWS, MID_TILES, TILES}, seen
+    every = {FEW_ROWS, TILES_128, TILES_256X1, TILES_256X2}
+    assert seen == every, seen
     seen = {_path((i - 1) * pitch + b, n // D, k) for (i, pitch, b, k, n, _) in ADD_CASES}
-    assert seen == {FEW_ROWS, MID_TILES, TILES}, seen
+    assert seen == every, seen
     # the benchmark shapes: 32768 rows on the large tiles, the reference's serving shape
-    # (64 positions x 24 sequences, src/serving/start copy.rs:30) on the small ones
-    assert _path(32768, 40, 2048) == TILES and _path(32768, 16, 4096) == TILES
-    assert _path(64 * 24, 40, 2048) == MID_TILES and _path(64 * 24, 16, 4096) == MID_TILES
+    # (64 positions x 24 sequences, src/serving/start copy.rs:30) on the one-head tiles
+    assert _path(32768, 40, 2048) == TILES_256X2 and _path(32768, 16, 4096) == TILES_256X2
+    assert _path(64 * 24, 40, 2048) == TILES_256X1 and _path(64 * 24, 16, 4096) == TILES_128
     assert _path(16, 40, 2048) == FEW_ROWS
 
 
@@ -143,7 +146,7 @@ def test_matmul3_ragged_step_of_many_sequences():
     positions on the tile kernel."""
     dtype = orc.F16
     pitch, batch, k, hq, hkv, cap = 200, 150, 256, 3, 2, 96
-    assert _path(batch, hq + 2 * hkv, k) == MID_TILES
+    assert _path(batch, hq + 2 * hkv, k) == TILES_128
     hidden = rand_storage((1, pitch, k), 61, dtype)
     wq, wk, wv = _weights(k, hq, hkv, dtype, 62)
     rope = _rope_table(cap, dtype)
@@ -187,6 +190,8 @@ ADD_CASES = [
     (300, 1, 1, 512, 256, orc.F16),                # 128-token tiles
     (257, 2, 2, 128, 128, orc.F16),
     (65, 24, 20, 4096, 256, orc.BF16),             # 1556 rows of which 20 in 24 live, K of the benchmark model
+    (1250, 4, 4, 64, 1536, orc.F16),               # 256-token x one-head tiles: 5000 rows, last tile partial
+    (600, 12, 9, 128, 640, orc.BF16),              # same tiles: 7197 rows of which 9 in 12 live, bfloat16
     (4100, 4, 3, 64, 640, orc.F16),                # 256 x 256 tiles: 16399 rows, last tile partial, odd head count
     (2049, 8, 8, 192, 512, orc.BF16),              # 16392 rows, bfloat16, three chunks of K
     (3, 5, 4, 64, 384, orc.BF16),
