@@ -522,7 +522,7 @@ def main():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--skip-cpu", action="store_true")
-    ap.add_argument("--only", default="", help="decode | prefill | decode128k | chunk | mixed | mixed48 | kvwrite | tokenstep | layerstep | qkv | oproj | chunkproj | stepproj")
+    ap.add_argument("--only", default="", help="decode | prefill | decode128k | chunk | smallchunk | mixed | mixed48 | kvwrite | tokenstep | layerstep | qkv | oproj | chunkproj | stepproj")
     ap.add_argument("--prefill-zero-kv", action="store_true",
                     help="diagnostic for --only prefill: K and V all zero (the kernel issues the same "
                          "instructions; separates its cycle count from the clock the part sustains "
@@ -610,6 +610,18 @@ def main():
                          "frac": round(ck["kernel_tflops"] / MFMA_F16_PEAK_TFLOPS, 4),
                          "traffic": None},
         })
+    if args.only in ("", "smallchunk"):
+        # a short chunk of one sequence on a long cache: 8 row-block workgroups, so the key range
+        # is split over workgroups and merged by a second small launch
+        sc = bench_prefill(64, args.steps, min(args.warmup, 5), p0=8192)
+        also.append({
+            "workload": "chunk of 64 new tokens of one sequence on an 8192-token cache, 32q/4kv heads, fp16 "
+                        "(key range split over workgroups + merge launch)",
+            "metric": "prefill attn TFLOP/s", "value": round(sc["tflops"], 2), "unit": "TFLOP/s",
+            "ms_per_step": round(sc["ms_per_step"], 5), "steps": args.steps,
+            "kv_gbs": round(2 * 4 * (8192 + 64) * D * 2 / (sc["ms_per_step"] * 1e-3) / 1e9, 1),
+        })
+
     if args.only in ("", "mixed"):
         # one layer of BASELINE configs[4]: a 16384-token prefill and a single-token step over 32
         # sequences with cache lengths U{1024..131072}; the configuration runs this 48 times a step

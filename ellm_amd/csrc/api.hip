@@ -77,6 +77,10 @@ struct ellm_attn {
   float* ws2_ml;
   uint32_t* counters;
   ellm::DecodeWorkspace ws;
+  // chunk calls with few row blocks on a long cache split the key range: partial rows
+  float* part_o;
+  float* part_ml;
+  size_t part_rows;
 };
 
 struct ellm_kv_cache {
@@ -89,13 +93,13 @@ struct ellm_kv_cache {
 
 static hipError_t free_workspace(ellm_attn* h) {
   hipError_t first = hipSuccess;
-  void* ptrs[] = {h->ws_acc, h->ws_ml, h->ws2_acc, h->ws2_ml, h->counters};
+  void* ptrs[] = {h->ws_acc, h->ws_ml, h->ws2_acc, h->ws2_ml, h->counters, h->part_o, h->part_ml};
   for (void* p : ptrs) {
     if (!p) continue;
     hipError_t e = hipFree(p);
     if (e != hipSuccess && first == hipSuccess) first = e;
   }
-  h->ws_acc = h->ws_ml = h->ws2_acc = h->ws2_ml = nullptr;
+  h->ws_acc = h->ws_ml = h->ws2_acc = h->ws2_ml = h->part_o = h->part_ml = nullptr;
   h->counters = nullptr;
   return first;
 }
@@ -174,8 +178,10 @@ int ellm_attn_create(const ellm_attn_desc* d, ellm_attn** out_handle) {
   h->n_cu = n_cu;
   h->ws = ellm::decode_workspace((uint32_t)d->batch_size, (uint32_t)d->attention_head_num,
                                  (uint32_t)d->kv_head_num, (uint32_t)n_cu);
-  h->ws_acc = h->ws_ml = h->ws2_acc = h->ws2_ml = nullptr;
+  h->ws_acc = h->ws_ml = h->ws2_acc = h->ws2_ml = h->part_o = h->part_ml = nullptr;
   h->counters = nullptr;
+  h->part_rows = ellm::prefill_workspace_rows((uint32_t)d->max_position_interval, (uint32_t)d->batch_size,
+                                              (uint32_t)d->attention_head_num, (uint32_t)n_cu);
   hipError_t e = hipMalloc((void**)&h->ws_acc, h->ws.rows * 128 * sizeof(float));
   if (e == hipSuccess) e = hipMalloc((void**)&h->ws_ml, h->ws.rows * 2 * sizeof(float));
   if (e == hipSuccess) e = hipMalloc((void**)&h->ws2_acc, h->ws.rows2 * 128 * sizeof(float));
@@ -183,6 +189,8 @@ int ellm_attn_create(const ellm_attn_desc* d, ellm_attn** out_handle) {
   // arrival counters of the single-token kernel; they return to zero by themselves
   if (e == hipSuccess) e = hipMalloc((void**)&h->counters, h->ws.counters * sizeof(uint32_t));
   if (e == hipSuccess) e = hipMemset(h->counters, 0, h->ws.counters * sizeof(uint32_t));
+  if (e == hipSuccess && h->part_rows) e = hipMalloc((void**)&h->part_o, h->part_rows * 128 * sizeof(float));
+  if (e == hipSuccess && h->part_rows) e = hipMalloc((void**)&h->part_ml, h->part_rows * 2 * sizeof(float));
   if (e != hipSuccess) {
     (void)free_workspace(h);
     delete h;
@@ -222,6 +230,10 @@ static void fill_args(const ellm_attn* h, ellm::AttnArgs* a) {
   a->ws2_acc = h->ws2_acc;
   a->ws2_ml = h->ws2_ml;
   a->counters = h->counters;
+  a->prefill_part_o = h->part_o;
+  a->prefill_part_ml = h->part_ml;
+  a->prefill_part_rows = h->part_rows;
+  a->n_cu = (uint32_t)h->n_cu;
   a->positions = nullptr;
 }
 

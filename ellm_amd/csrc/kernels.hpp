@@ -37,7 +37,16 @@ struct AttnArgs {
   uint32_t* counters;  // arrival counters, zero between launches
   uint32_t split_len;  // keys per split, multiple of 64
   uint32_t n_split;
+  // chunk path, key range split over workgroups (may be null: never split): room for
+  // prefill_part_rows partial rows of 128 + 2 floats
+  float* prefill_part_o;
+  float* prefill_part_ml;
+  size_t prefill_part_rows;
+  uint32_t n_cu;
 };
+// Partial rows the chunk path's workspace holds for an operator of this shape (0: none needed).
+size_t prefill_workspace_rows(uint32_t max_interval, uint32_t batch_capacity, uint32_t n_q_heads,
+                              uint32_t n_cu);
 
 // Keys handled by one workgroup step of the single-token kernel.
 constexpr uint32_t kDecodeStepKeys = 64;

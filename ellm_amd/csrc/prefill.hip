@@ -52,6 +52,13 @@ struct PrefillKernelArgs {
   uint32_t position_index, interval;
   uint32_t negate_q;         // scale < 0: fold the sign into Q (exact) so that c > 0
   float c;                   // |scale| * log2(e), > 0
+  // Key range split over gridDim.y workgroups (few row blocks on a long cache): split s
+  // walks tiles [s * split_tiles, (s + 1) * split_tiles) and leaves, per query row, its
+  // unnormalised output row, running maximum (log2 units) and denominator in
+  // part_o [row][n_split][128] / part_ml [row][n_split][2] for prefill_merge_kernel.
+  uint32_t n_split, split_tiles;
+  float* part_o;
+  float* part_ml;
 };
 
 // ---------------------------------------------------------------------------
@@ -81,7 +88,7 @@ constexpr int kPpThreads = kPpWaves * kWave;
 constexpr int kLdsAhead = 8;  // LDS operand reads in flight ahead of their MFMA
 constexpr int kBufferFlags = 0x00020000;  // raw buffer of 32-bit data, no swizzle (word 3 of the descriptor)
 
-template <typename T>
+template <typename T, bool SPLIT>
 __global__ __launch_bounds__(kPpThreads, 2) void prefill_pingpong_kernel(PrefillKernelArgs p) {
   // K tiles [2][64][kKsPitch] then V tiles [3][64][kVsPitch]: V is staged one step
   // earlier than it is read, so that every operand of a matrix step is in LDS a whole
@@ -112,7 +119,11 @@ __global__ __launch_bounds__(kPpThreads, 2) void prefill_pingpong_kernel(Prefill
   const uint32_t S = p.interval, P0 = p.position_index;
   const uint32_t wg_last_tok = min(S, t_base + 32 * p.tblocks_per_wg) - 1;
   const uint32_t kmax = P0 + wg_last_tok;
-  const uint32_t n_tiles = kmax / kBK + 1;
+  const uint32_t all_tiles = kmax / kBK + 1;
+  // the tiles of this workgroup: all of them, or its share of the key range
+  const uint32_t kt0 = SPLIT ? blockIdx.y * p.split_tiles : 0u;
+  if (SPLIT && kt0 >= all_tiles) return;  // (prefill_merge_kernel derives the live splits the same way)
+  const uint32_t n_tiles = SPLIT ? min(all_tiles - kt0, p.split_tiles) : all_tiles;
 
   const uint32_t hg = wave % p.heads_per_wg, tb = wave / p.heads_per_wg;
   const uint32_t head = kvh * p.group + hgrp * p.heads_per_wg + hg;
@@ -170,8 +181,8 @@ __global__ __launch_bounds__(kPpThreads, 2) void prefill_pingpong_kernel(Prefill
   const uint32_t ks_store = lds0 + 2 * (ld_r * kKsPitch + 8 * ld_c);
   const uint32_t vs_store = lds0 + 2 * (2 * kKsHalves + ld_r * kVsPitch + 8 * ld_c);
   u32x4 stg[4];
-  auto load_piece = [&](uint32_t kt, int i) {  // kt must be wave-uniform to the compiler
-    const uint32_t off = kt * tile_bytes;
+  auto load_piece = [&](uint32_t kt, int i) {  // kt (relative to kt0) must be wave-uniform to the compiler
+    const uint32_t off = (kt0 + kt) * tile_bytes;
     // (written as a scalar min and subtract: a saturating subtract would be a vector instruction)
     const uint32_t left = valid_bytes - __builtin_amdgcn_readfirstlane(min(valid_bytes, off));
     const __amdgpu_buffer_rsrc_t rsrc =
@@ -305,7 +316,7 @@ __global__ __launch_bounds__(kPpThreads, 2) void prefill_pingpong_kernel(Prefill
   // Vector step kt = soft-max of tile kt: mask on the diagonal, row max, lazy
   // rescale of O^T, exponentials, packing, row sum.
   auto vector_step = [&](uint32_t kt) __attribute__((always_inline)) {
-    const uint32_t kb = kt * kBK;
+    const uint32_t kb = (kt0 + kt) * kBK;
     if (kb + kBK - 1 > first_pos) {  // tile crosses this row block's diagonal
 #pragma unroll
       for (int mb = 0; mb < 2; ++mb)
@@ -381,7 +392,20 @@ __global__ __launch_bounds__(kPpThreads, 2) void prefill_pingpong_kernel(Prefill
   }
 
 
-  {
+  if constexpr (SPLIT) {
+    const float l = sum_with_partner_half(l_run);
+    if (row_valid) {
+      const size_t part = (((size_t)tok * p.batch_pitch + seq) * p.n_q_heads + head) * p.n_split + blockIdx.y;
+      float* orow = p.part_o + part * kHeadDim;
+#pragma unroll
+      for (int db = 0; db < 4; ++db)
+#pragma unroll
+        for (int q4 = 0; q4 < 4; ++q4)
+          *(f32x4*)(orow + 32 * db + 8 * q4 + 4 * g) =
+              f32x4{oacc[db][4 * q4], oacc[db][4 * q4 + 1], oacc[db][4 * q4 + 2], oacc[db][4 * q4 + 3]};
+      if (g == 0) *(float2*)(p.part_ml + part * 2) = float2{m_run, l};
+    }
+  } else {
     const float l = sum_with_partner_half(l_run);
     if (row_valid) {
       const float inv = 1.0f / l;
@@ -401,6 +425,61 @@ __global__ __launch_bounds__(kPpThreads, 2) void prefill_pingpong_kernel(Prefill
             (m_run + fast_log2(l)) * kLn2;
     }
   }
+}
+
+// Folds the partial results of a split launch: G lanes per (query row, four columns) take
+// the row's splits in turn and combine through lane exchanges (with hundreds of splits and
+// few rows a thread walking them alone would be one long chain of memory round trips).
+// A row's live splits are those whose first tile is at or before the last key any row of
+// its workgroup sees, as in the kernel above; a split whose keys are all masked for this row
+// left (max = -inf, sum = 0) and weighs nothing.  Split 0 always holds key 0, so the maximum
+// is finite.
+template <typename T, int G>
+__global__ __launch_bounds__(256) void prefill_merge_kernel(PrefillKernelArgs p, uint32_t batch) {
+  const uint32_t quads = kHeadDim / 4;
+  const size_t items = (size_t)p.interval * batch * p.n_q_heads * quads;
+  const size_t gid = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const uint32_t sub = gid % G;
+  const bool valid = gid / G < items;
+  const size_t item = valid ? gid / G : 0;  // idle groups keep their lanes in the exchanges
+  const uint32_t dq = item % quads;
+  size_t r = item / quads;
+  const uint32_t head = r % p.n_q_heads;
+  r /= p.n_q_heads;
+  const uint32_t seq = r % batch;
+  const uint32_t tok = r / batch;
+  const uint32_t wg_tokens = 32 * p.tblocks_per_wg;
+  const uint32_t wg_last_tok = min(p.interval, (tok / wg_tokens + 1) * wg_tokens) - 1;
+  const uint32_t all_tiles = (p.position_index + wg_last_tok) / kBK + 1;
+  const uint32_t live = (all_tiles + p.split_tiles - 1) / p.split_tiles;
+  const size_t row = ((size_t)tok * p.batch_pitch + seq) * p.n_q_heads + head;
+  const float* ml = p.part_ml + row * p.n_split * 2;
+  const float* po = p.part_o + row * p.n_split * kHeadDim + 4 * dq;
+  float m = -INFINITY;
+  for (uint32_t s = sub; s < live; s += G) m = fmaxf(m, ml[2 * s]);
+#pragma unroll
+  for (int x = 1; x < G; x <<= 1) m = fmaxf(m, __shfl_xor(m, x));
+  float l = 0.0f;
+  f32x4 o = {0.0f, 0.0f, 0.0f, 0.0f};
+  for (uint32_t s = sub; s < live; s += G) {
+    const float ms = ml[2 * s];
+    const float w = (ms == -INFINITY) ? 0.0f : fast_exp2(ms - m);
+    l += w * ml[2 * s + 1];
+    o += w * *(const f32x4*)(po + (size_t)s * kHeadDim);
+  }
+#pragma unroll
+  for (int x = 1; x < G; x <<= 1) {
+    l += __shfl_xor(l, x);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) o[e] += __shfl_xor(o[e], x);
+  }
+  if (!valid || sub != 0) return;
+  const float inv = 1.0f / l;
+  u32x2 w;
+  w[0] = Mfma<T>::pack2(o[0] * inv, o[1] * inv);
+  w[1] = Mfma<T>::pack2(o[2] * inv, o[3] * inv);
+  *(u32x2*)(p.out + (size_t)tok * p.q_token_stride + ((size_t)seq * p.n_q_heads + head) * kHeadDim + 4 * dq) = w;
+  if (p.lse && dq == 0) p.lse[row] = (m + fast_log2(l)) * kLn2;
 }
 
 uint32_t gcd_u32(uint32_t a, uint32_t b) {
@@ -451,11 +530,59 @@ hipError_t launch_pingpong(const AttnArgs& a, hipStream_t stream) {
   } else {
     n_wg = p.combos * p.n_wg_tokens;
   }
-  hipLaunchKernelGGL((prefill_pingpong_kernel<T>), dim3(n_wg), dim3(kPpThreads), 0, stream, p);
-  return hipGetLastError();
+  // Few row blocks on a long cache: split the key range until there are about two
+  // workgroups per compute unit (four measured no faster), a split no shorter than eight
+  // tiles (each pays the pipeline's first and last step), as far as the workspace holds the
+  // partial rows.
+  p.n_split = 1;
+  p.split_tiles = 0;
+  p.part_o = a.prefill_part_o;
+  p.part_ml = a.prefill_part_ml;
+  const uint32_t base = p.combos * p.n_wg_tokens;
+  const uint32_t max_tiles = (a.position_index + a.position_interval - 1) / kBK + 1;
+  const size_t rows = (size_t)a.position_interval * a.batch_pitch * a.n_q_heads;
+  if (a.prefill_part_o && base < a.n_cu && max_tiles >= 16) {
+    uint32_t want = (2 * a.n_cu + base - 1) / base;
+    const size_t room = a.prefill_part_rows / rows;   // splits the workspace holds for every row
+    if (want > room) want = (uint32_t)room;
+    if (want > 1) {
+      uint32_t split_tiles = (max_tiles + want - 1) / want;
+      if (split_tiles < 8) split_tiles = 8;
+      p.split_tiles = split_tiles;
+      p.n_split = (max_tiles + split_tiles - 1) / split_tiles;
+    }
+  }
+  if (p.n_split <= 1) {
+    p.n_split = 1;
+    hipLaunchKernelGGL((prefill_pingpong_kernel<T, false>), dim3(n_wg), dim3(kPpThreads), 0, stream, p);
+    return hipGetLastError();
+  }
+  hipLaunchKernelGGL((prefill_pingpong_kernel<T, true>), dim3(n_wg, p.n_split), dim3(kPpThreads), 0, stream, p);
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return e;
+  const size_t items = (size_t)a.position_interval * a.batch * a.n_q_heads * (kHeadDim / 4);
+  auto merge = [&](auto kernel, size_t lanes) {
+    hipLaunchKernelGGL(kernel, dim3((uint32_t)((items * lanes + 255) / 256)), dim3(256), 0, stream, p, a.batch);
+    return hipGetLastError();
+  };
+  // lanes per item: more when there are many splits to walk, as long as the grid stays small
+  constexpr size_t kLanesMax = (size_t)1 << 21;
+  if (p.n_split > 32 && items * 64 <= kLanesMax) return merge(prefill_merge_kernel<T, 64>, 64);
+  if (p.n_split > 8 && items * 8 <= kLanesMax) return merge(prefill_merge_kernel<T, 8>, 8);
+  return merge(prefill_merge_kernel<T, 1>, 1);
 }
 
 }  // namespace
+
+// The key range is split only while the unsplit launch has fewer workgroups than compute
+// units, i.e. at most 256 n_cu query rows, and then into at most ~n_cu workgroups in all.
+size_t prefill_workspace_rows(uint32_t max_interval, uint32_t batch_capacity, uint32_t n_q_heads,
+                              uint32_t n_cu) {
+  if (max_interval < 2) return 0;  // single-token calls take the other kernel
+  const size_t rows = (size_t)max_interval * batch_capacity * n_q_heads;
+  const size_t cap = (size_t)256 * n_cu;
+  return rows * 256 < cap ? rows * 256 : cap;
+}
 
 hipError_t launch_prefill(const AttnArgs& a, hipStream_t stream) {
   if (a.dtype == 0) return launch_pingpong<F16>(a, stream);

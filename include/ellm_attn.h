@@ -97,7 +97,8 @@ typedef struct ellm_attn_desc {
 typedef struct ellm_attn ellm_attn;
 
 /* Validates the description and allocates the operator's own workspace (split
- * partial results for the single-token path).  Borrowed pointers are not owned. */
+ * partial results for the single-token path and, when max_position_interval > 1,
+ * for short chunks on long caches: at most 34 MB).  Borrowed pointers are not owned. */
 int ellm_attn_create(const ellm_attn_desc* desc, ellm_attn** out_handle);
 
 /* Frees the handle and its workspace only.  NULL is accepted. */
@@ -109,8 +110,9 @@ int ellm_attn_destroy(ellm_attn* handle);
  * position_interval) of the first batch_size sequences; the query at position p
  * attends to keys 0..=p of its own sequence (flash_attention.rs:57-58).
  * position_interval == 1 takes the split-KV single-token kernel, larger
- * intervals the tiled MFMA kernel.  Zero batch_size or position_interval is a
- * no-op returning ELLM_OK.
+ * intervals the tiled MFMA kernel (with the key range split over workgroups and
+ * a merge launch behind it when the call has too few query rows to fill the
+ * device).  Zero batch_size or position_interval is a no-op returning ELLM_OK.
  */
 int ellm_attn_run(ellm_attn* handle, size_t position_index, size_t position_interval,
                   size_t batch_size, void* stream);

@@ -40,6 +40,13 @@ PREFILL = [
     ("interval_2", 2, 2, 8, 2, 64, 61, 2),
     ("tile_edge_63_64_65", 1, 1, 8, 1, 256, 63, 66),
     ("qwen3_heads_2k", 1, 1, 32, 4, 2048, 0, 2048),
+    # few row blocks on a long cache: the key range is split over workgroups and merged
+    ("split_chunk_on_long_cache", 1, 1, 8, 1, 2304, 2000, 70),
+    ("split_batch_below_capacity_g4", 3, 2, 8, 2, 1600, 1500, 40),
+    ("split_interval_2", 2, 2, 8, 2, 4200, 4100, 2),
+    ("split_from_zero_later_splits_empty_for_early_rows", 1, 1, 8, 1, 1152, 0, 1100),
+    ("split_qwen3_chunk_64_on_8k", 1, 1, 32, 4, 8320, 8192, 64),
+    ("split_three_tokens_on_20k_forty_splits", 1, 1, 8, 1, 20480, 20000, 3),
 ]
 
 
