@@ -36,6 +36,8 @@ TRAFFIC_BYTES = {
     "decode128k": (264959 + 2523) * 1024,
     "prefill": (1363516 + 319881) * 1024,
     "kvwrite": (73808 + 65536) * 1024,
+    "qkv": (1130126 + 327680) * 1024,          # fetched past the L2s (mostly from the last-level cache) + written
+    "stepproj": (21383 + 1318) * 1024,
 }
 MFMA_F16_PEAK_TFLOPS = 2500.0  # MI355X dense fp16/bf16 MFMA, published
 D = 128
@@ -698,7 +700,8 @@ def main():
             "ms_per_step": round(pj["ms_per_step"], 4), "steps": pj_steps,
             "roofline": {"bound": "mfma", "achieved": round(pj["kernel_tflops"], 2),
                          "peak": MFMA_F16_PEAK_TFLOPS, "unit": "TFLOP/s",
-                         "frac": round(pj["kernel_tflops"] / MFMA_F16_PEAK_TFLOPS, 4), "traffic": None},
+                         "frac": round(pj["kernel_tflops"] / MFMA_F16_PEAK_TFLOPS, 4),
+                         "traffic": TRAFFIC_BYTES["qkv"]},
         })
     if args.only in ("", "oproj"):
         pj_steps = max(3, min(args.steps, 20))
@@ -743,7 +746,7 @@ def main():
             "roofline": {"bound": "hbm", "achieved": round(sp["qkv_bytes"] / (sp["qkv_kernel_ms"] * 1e-3) / 1e9, 1),
                          "peak": HBM_PEAK_GBS, "unit": "GB/s",
                          "frac": round(sp["qkv_bytes"] / (sp["qkv_kernel_ms"] * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
-                         "traffic": None},
+                         "traffic": TRAFFIC_BYTES["stepproj"]},
         })
 
     if args.only in ("", "layerstep"):
