@@ -169,3 +169,87 @@ def test_chunked_prefill_projection_feeds_attention():
     qkv.close()
     attn.close()
     cache.close()
+
+
+def test_recorded_chunk_step_on_a_long_cache_replays_like_eager():
+    """A prompt chunk's attention block (fused projection on one-head tiles -> chunk attention with
+    its key range split over workgroups and merged -> output projection) recorded once and
+    replayed with fresh activations: every replay equals the eager run of the same inputs bit
+    for bit, and the first one matches the oracle."""
+    import torch
+
+    import ellm_amd
+
+    dtype = orc.F16
+    b, hq, hkv, cap, hidden, p0, n = 2, 8, 2, 2048, 256, 1700, 70
+    scale = 1.0 / np.sqrt(D)
+    rope = _rope_table(cap, dtype)
+    wq = rand_storage((hq * D, hidden), 21, dtype, scale=hidden ** -0.5)
+    wk = rand_storage((hkv * D, hidden), 22, dtype, scale=hidden ** -0.5)
+    wv = rand_storage((hkv * D, hidden), 23, dtype, scale=hidden ** -0.5)
+    wo = rand_storage((hidden, hq * D), 24, dtype, scale=(hq * D) ** -0.5)
+    k0 = rand_storage((b, hkv, cap, D), 25, dtype)
+    v0 = rand_storage((b, hkv, cap, D), 26, dtype)
+    lib = ellm_amd.load_library()
+    assert lib.ellm_projection_path(n * b, hq + 2 * hkv, hidden) in (1, 2)
+
+    cache = ellm_amd.KVCache(1, b, hkv, cap, ellm_amd.DTYPE_F16)
+    kt, vt = cache.layer_tensors(0, torch.float16)
+    _, _, strides = cache.layer(0)
+    x = torch.zeros((n, b, hidden), dtype=torch.float16, device="cuda")
+    q = torch.zeros((n, b, hq, D), dtype=torch.float16, device="cuda")
+    att = torch.zeros_like(q)
+    res = torch.zeros((n, b, hidden), dtype=torch.float16, device="cuda")
+    out = torch.zeros_like(res)
+    dev = [to_dev(a, dtype) for a in (wq, wk, wv, rope, wo)]
+    qkv = ellm_amd.MatMul3(x, dev[0], q, dev[1], kt, dev[2], vt, dev[3], D, b, hq, hkv, strides, cap)
+    attn = ellm_amd.Attention(q, kt, vt, att, b, hq, hkv, D, strides, scale, sequence_capacity=cap,
+                              max_position_interval=n)
+    oproj = ellm_amd.MatMulAdd(att.view(n, b, hq * D), dev[4], res, out)
+
+    def step(stream):
+        qkv.run(p0, n, b, stream=stream)
+        attn.run(p0, n, b, stream=stream)
+        oproj.run(p0, n, b, stream=stream)
+
+    def fresh(i):
+        kt.copy_(to_dev(k0, dtype))
+        vt.copy_(to_dev(v0, dtype))
+        x.copy_(to_dev(rand_storage((n, b, hidden), 100 + i, dtype), dtype))
+        res.copy_(to_dev(rand_storage((n, b, hidden), 200 + i, dtype), dtype))
+        out.zero_()
+        att.zero_()
+
+    stream = torch.cuda.Stream()
+    eager = []
+    for i in range(3):
+        fresh(i)
+        torch.cuda.synchronize()
+        step(stream)
+        stream.synchronize()
+        eager.append((att.clone(), out.clone(), kt.clone()))
+    with ellm_amd.StepGraph(stream) as graph:
+        step(stream)
+    for i in range(3):
+        fresh(i)
+        torch.cuda.synchronize()
+        graph.launch()
+        stream.synchronize()
+        for got, want in zip((att, out, kt), eager[i]):
+            assert torch.equal(got, want), i
+    # the first inputs against the oracle: projection rows, then attention over the cache they wrote
+    fresh(0)
+    torch.cuda.synchronize()
+    graph.launch()
+    stream.synchronize()
+    gq, gatt = to_host(q, dtype), to_host(att, dtype)
+    sk, sv = (orc.to_storage(to_host(t, dtype), dtype) for t in (kt, vt))
+    want, _ = orc.attention(orc.to_storage(gq, dtype), sk, sv, scale, dtype, position_index=p0)
+    assert compare(gatt, orc.from_storage(want, dtype), dtype)["ok"]
+    want_out = orc.matmul_add(orc.to_storage(gatt, dtype).reshape(n, b, hq * D), wo,
+                              rand_storage((n, b, hidden), 200, dtype), dtype, batch_size=b)
+    assert compare_ulps(to_host(out, dtype), orc.from_storage(want_out, dtype), dtype)["ok"]
+    graph.close()
+    for op in (qkv, attn, oproj):
+        op.close()
+    cache.close()
