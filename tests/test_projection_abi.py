@@ -110,3 +110,21 @@ def test_matmul_add_run_range_checks():
     assert lib.ellm_matmul_add_run(h, 0, 1, 5, None) == OUT_OF_RANGE
     assert lib.ellm_matmul_add_run(h, 0, 0, 4, None) == OK
     assert lib.ellm_matmul_add_destroy(h) == OK
+
+
+def test_projection_path_rule():
+    """ellm_projection_path without a device (256 compute units assumed): the few-rows kernel up
+    to 64 rows when K suits it, then the smallest one-head tile whose workgroups fit the part in
+    one round, then the 256 x 256 tiles; sizes no handle accepts give -1."""
+    lib = ellm_amd.load_library()
+    path = lib.ellm_projection_path
+    few, t128, t256, big = 0, 1, 2, 3
+    assert path(1, 40, 2048) == few and path(64, 40, 2048) == few
+    assert path(65, 40, 2048) == t128                 # one 128-token tile per head
+    assert path(16, 40, 64) == t128                   # K too short for the streaming kernel's waves
+    assert path(6 * 128, 40, 2048) == t128 and path(6 * 128 + 1, 40, 2048) == t256
+    assert path(6 * 256, 40, 2048) == t256 and path(6 * 256 + 1, 40, 2048) == big
+    assert path(16 * 128, 16, 4096) == t128 and path(16 * 256, 16, 4096) == t256
+    assert path(16 * 256 + 1, 16, 4096) == big and path(32768, 40, 2048) == big
+    assert path(0, 40, 2048) == -1 and path(16, 0, 2048) == -1 and path(16, 40, 0) == -1
+    assert path(1 << 40, 40, 2048) == -1 and path(16, 40, 1 << 20) == -1
