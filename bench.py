@@ -625,7 +625,7 @@ def main():
         })
 
     if args.only in ("", "mixed"):
-        # one layer of BASELINE configs[4]: a 16384-token prefill and a single-token step over 32
+        # one layer of the mixed-step configuration: a 16384-token prefill and a single-token step over 32
         # sequences with cache lengths U{1024..131072}; the configuration runs this 48 times a step
         mx_steps = max(3, min(args.steps, 10))
         mp = bench_prefill(16384, mx_steps, min(args.warmup, 2))
