@@ -490,6 +490,57 @@ def bench_layer_step(layers, batch, length, steps, warmup, hidden=2048, hq=32, h
     return {"eager_ms": eager_ms, "graph_ms": graph_ms, "kv_bytes": kv_bytes, "w_bytes": w_bytes}
 
 
+def bench_chunk_block(positions, batch, p0, steps, warmup, hidden=2048, hq=32, hkv=4):
+    """The attention block of one layer for a prompt chunk of `positions` tokens x `batch` sequences
+    on caches that already hold `p0` tokens: fused Q/K/V projection (K/V written into the cache at
+    p0..), chunk attention over 0..p0 + positions, output projection + residual."""
+    import torch
+
+    import ellm_amd
+
+    dt = torch.float16
+    cap = p0 + positions
+    scale = 1.0 / D ** 0.5
+    cache = ellm_amd.KVCache(1, batch, hkv, cap, ellm_amd.DTYPE_F16)
+    kt, vt = cache.layer_tensors(0, dt)
+    kt.normal_()
+    vt.normal_()
+    _, _, strides = cache.layer(0)
+    j = torch.arange(D // 2, device="cuda", dtype=torch.float64)
+    ang = torch.arange(cap, device="cuda", dtype=torch.float64)[:, None] * (1.0e6 ** (-2.0 * j / D))[None, :]
+    rope = torch.stack((torch.cos(ang), torch.sin(ang)), dim=-1).reshape(cap, D).to(dt)
+    x = _dev_normal((positions, batch, hidden), dt, 701)
+    y = torch.zeros_like(x)
+    q = torch.zeros((positions, batch, hq, D), dtype=dt, device="cuda")
+    att = torch.zeros_like(q)
+    w = [_dev_normal((h * D, hidden), dt, 702 + i, scale=hidden ** -0.5) for i, h in enumerate((hq, hkv, hkv))]
+    wo = _dev_normal((hidden, hq * D), dt, 705, scale=(hq * D) ** -0.5)
+    qkv = ellm_amd.MatMul3(x, w[0], q, w[1], kt, w[2], vt, rope, D, batch, hq, hkv, strides, cap)
+    attn = ellm_amd.Attention(q, kt, vt, att, batch, hq, hkv, D, strides, scale, sequence_capacity=cap,
+                              max_position_interval=positions)
+    oproj = ellm_amd.MatMulAdd(att.view(positions, batch, hq * D), wo, x, y)
+    parts = {}
+    for name, fn in (("qkv", lambda i: qkv.run(p0, positions, batch)),
+                     ("attention", lambda i: attn.run(p0, positions, batch)),
+                     ("output", lambda i: oproj.run(p0, positions, batch))):
+        per, _ = _time_steps(fn, steps, warmup)
+        parts[name] = sum(per) / len(per)
+
+    def block(_i):
+        qkv.run(p0, positions, batch)
+        attn.run(p0, positions, batch)
+        oproj.run(p0, positions, batch)
+
+    _, block_ms = _time_steps(block, steps, warmup)
+    for op in (qkv, attn, oproj):
+        op.close()
+    cache.close()
+    rows = positions * batch
+    flops = (2 * rows * hidden * (hq + 2 * hkv) * D + 2 * rows * hidden * hq * D
+             + 4 * D * hq * batch * (positions * p0 + positions * (positions + 1) / 2))
+    return {"block_ms": block_ms, "parts_ms": parts, "flops": flops}
+
+
 def cpu_baseline_decode(batch, length, hq=32, hkv=4, budget_s=1.5):
     """The CPU oracle on the full single-token workload (all host cores), repeated for about
     `budget_s` seconds of wall time (x 16 threads: 20-odd core-seconds of CPU work)."""
@@ -524,7 +575,7 @@ def main():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--skip-cpu", action="store_true")
-    ap.add_argument("--only", default="", help="decode | prefill | decode128k | chunk | smallchunk | mixed | mixed48 | kvwrite | tokenstep | layerstep | qkv | oproj | chunkproj | stepproj")
+    ap.add_argument("--only", default="", help="decode | prefill | decode128k | chunk | smallchunk | mixed | mixed48 | kvwrite | tokenstep | layerstep | qkv | oproj | chunkproj | chunkblock | stepproj")
     ap.add_argument("--prefill-zero-kv", action="store_true",
                     help="diagnostic for --only prefill: K and V all zero (the kernel issues the same "
                          "instructions; separates its cycle count from the clock the part sustains "
@@ -730,6 +781,19 @@ def main():
             "roofline": {"bound": "mfma", "achieved": round(cq["kernel_tflops"], 2),
                          "peak": MFMA_F16_PEAK_TFLOPS, "unit": "TFLOP/s",
                          "frac": round(cq["kernel_tflops"] / MFMA_F16_PEAK_TFLOPS, 4), "traffic": None},
+        })
+
+    if args.only in ("", "chunkblock"):
+        cb = bench_chunk_block(64, 24, 4096, min(args.steps, 30), min(args.warmup, 5))
+        also.append({
+            "workload": "attention block of one layer for a prompt chunk of 64 positions x 24 sequences (the "
+                        "reference's serving shape) on caches of 4096 tokens: fused Q/K/V projection (K/V into the "
+                        "cache) + chunk attention + output projection with residual, fp16, three launches",
+            "metric": "attention-block ms per chunk", "value": round(cb["block_ms"], 5), "unit": "ms",
+            "steps": min(args.steps, 30),
+            "qkv_ms": round(cb["parts_ms"]["qkv"], 5), "attention_ms": round(cb["parts_ms"]["attention"], 5),
+            "output_ms": round(cb["parts_ms"]["output"], 5),
+            "tflops": round(cb["flops"] / (cb["block_ms"] * 1e-3) / 1e12, 1),
         })
 
     if args.only in ("", "stepproj"):
