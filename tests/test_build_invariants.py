@@ -1,0 +1,42 @@
+"""Properties of the generated code that the sources rely on but cannot state themselves,
+checked on the compiler's assembly listing (no GPU needed)."""
+import os
+import re
+import shutil
+import subprocess
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+CSRC = os.path.join(ROOT, "ellm_amd", "csrc")
+HIPCC = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
+FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fno-strict-aliasing", "-Xclang", "-target-feature",
+         "-Xclang", "-packed-fp32-ops", "-Wno-int-to-pointer-cast", "--cuda-device-only", "-S"]
+
+
+def _listing(name, tmp_path):
+    if not os.path.exists(HIPCC):
+        pytest.skip("no hipcc")
+    out = tmp_path / (name + ".s")
+    subprocess.run([HIPCC, *FLAGS, "-o", str(out), os.path.join(CSRC, name)], check=True,
+                   capture_output=True, timeout=600)
+    return out.read_text()
+
+
+def test_one_head_tile_kernels_leave_m0_to_the_inline_asm(tmp_path):
+    """project_mid.hip sets M0 (the LDS address of a direct-to-LDS load) inside inline asm that
+    cannot declare the write; that is sound only while the compiler keeps nothing of its own in
+    M0, i.e. never indexes registers through it in these kernels."""
+    text = _listing("project_mid.hip", tmp_path)
+    code = [l.split(";")[0] for l in text.splitlines()]
+    uses = [l for l in code if re.search(r"\bm0\b", l)]
+    assert uses and all(re.fullmatch(r"\s*s_mov_b32 m0, s\d+\s*", l) for l in uses), \
+        [l for l in uses if not re.fullmatch(r"\s*s_mov_b32 m0, s\d+\s*", l)][:5]
+    assert not any("movrel" in l or "s_set_gpr_idx" in l for l in code)
+
+
+@pytest.mark.parametrize("name", ["project_mid.hip", "prefill.hip", "decode.hip"])
+def test_hot_kernels_do_not_spill(name, tmp_path):
+    text = _listing(name, tmp_path)
+    sizes = [int(x) for x in re.findall(r"\.private_segment_fixed_size:\s*(\d+)", text)]
+    assert sizes and all(v == 0 for v in sizes), sizes
