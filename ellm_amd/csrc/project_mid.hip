@@ -27,6 +27,10 @@ struct MidShape {
   static constexpr int kLdsBytes = kStages * kStageBytes;
   static constexpr int kLoads = 4 * MB + 4;         // 1 KB wave loads per chunk and wave
   static constexpr int kAhead = kStages - 1;        // chunks requested ahead of the one being multiplied
+  // loads a wave still has outstanding when its pieces of the next chunk must have landed: the
+  // chunks requested after that one (the literal in the kernel's s_waitcnt)
+  static constexpr int kMayBePending = (kAhead - 1) * kLoads;
+  static_assert(kMayBePending == (MB == 1 ? 16 : 12), "s_waitcnt vmcnt literals in project_mid_kernel");
   static_assert(4 * kEpWaveBytes <= kLdsBytes, "the epilogue reuses the stages");
   static_assert(kLdsBytes <= 160 * 1024, "LDS of a compute unit");
 };
@@ -130,7 +134,7 @@ __global__ __launch_bounds__(kMidThreads) void project_mid_kernel(ProjectKernelA
 #pragma unroll
     for (int i = 0; i < kLoads; ++i) load_piece(k, i);
   if constexpr (MB == 1)
-    asm volatile("s_waitcnt vmcnt(16)" ::: "memory");   // (kAhead - 1) * kLoads
+    asm volatile("s_waitcnt vmcnt(16)" ::: "memory");   // Shape::kMayBePending
   else
     asm volatile("s_waitcnt vmcnt(12)" ::: "memory");
   __syncthreads();
