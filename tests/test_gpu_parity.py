@@ -156,6 +156,10 @@ def test_unusual_scales(scale):
     v = rand_storage((1, 2, 128, D), 18, dtype)
     _check(f"scale {scale} prefill", q, k, v, scale, dtype, p0=30)
     _check(f"scale {scale} decode", q[:1], k, v, scale, dtype, p0=127)
+    # the same through the split chunk path (few rows on a long cache) and its merge
+    k2 = rand_storage((1, 2, 1600, D), 27, dtype, scale=0.3)
+    v2 = rand_storage((1, 2, 1600, D), 28, dtype)
+    _check(f"scale {scale} split chunk", q, k2, v2, scale, dtype, p0=1500)
 
 
 def test_garbage_beyond_the_position_does_not_leak():
@@ -175,6 +179,25 @@ def test_garbage_beyond_the_position_does_not_leak():
     c1, _ = gpu_attention(q[:1], k, v, 0.09, dtype, position_index=p0 + s - 1)
     d1, _ = gpu_attention(q[:1], k2, v2, 0.09, dtype, position_index=p0 + s - 1)
     assert np.array_equal(c1, d1)
+
+
+def test_garbage_beyond_the_position_does_not_leak_into_split_chunks():
+    """The split chunk path: workgroups of later key ranges see rows whose every key is masked,
+    and the cache beyond the last position holds NaN / Inf."""
+    dtype = orc.F16
+    s, p0, cap = 40, 1400, 2048
+    q = rand_storage((s, 1, 8, D), 22, dtype)
+    k = rand_storage((1, 2, cap, D), 23, dtype)
+    v = rand_storage((1, 2, cap, D), 24, dtype)
+    clean, clean_lse = gpu_attention(q, k, v, 0.09, dtype, position_index=p0)
+    k2, v2 = k.copy(), v.copy()
+    bad = np.array([0x7e00, 0x7c00, 0xfc00, 0x7bff], dtype=np.uint16)      # NaN, +Inf, -Inf, 65504
+    k2[:, :, p0 + s:] = bad[np.arange(k2[:, :, p0 + s:].size) % 4].reshape(k2[:, :, p0 + s:].shape)
+    v2[:, :, p0 + s:] = bad[(np.arange(v2[:, :, p0 + s:].size) + 1) % 4].reshape(v2[:, :, p0 + s:].shape)
+    dirty, dirty_lse = gpu_attention(q, k2, v2, 0.09, dtype, position_index=p0)
+    assert np.array_equal(clean, dirty) and np.array_equal(clean_lse, dirty_lse)
+    want, want_lse = orc.attention(q, k, v, 0.09, dtype, position_index=p0)
+    assert compare(clean, orc.from_storage(want, dtype), dtype)["ok"]
 
 
 def test_causality_rows_ignore_later_keys():
