@@ -253,3 +253,69 @@ def test_recorded_chunk_step_on_a_long_cache_replays_like_eager():
     for op in (qkv, attn, oproj):
         op.close()
     cache.close()
+
+
+def test_recorded_long_chunk_uses_the_large_projection_tiles():
+    """A chunk long enough for the 256 x 256 projection tiles (the one kernel here that needs
+    per-wave scratch memory), recorded and replayed: equal to the eager run bit for bit."""
+    import torch
+
+    import ellm_amd
+
+    dtype = orc.F16
+    n, b, hq, hkv, hidden = 5700, 1, 8, 2, 64
+    cap = n
+    lib = ellm_amd.load_library()
+    assert lib.ellm_projection_path(n, hq + 2 * hkv, hidden) == 3
+    rope = _rope_table(cap, dtype)
+    w = [rand_storage((h * D, hidden), 31 + i, dtype, scale=hidden ** -0.5) for i, h in enumerate((hq, hkv, hkv))]
+    cache = ellm_amd.KVCache(1, b, hkv, cap, ellm_amd.DTYPE_F16)
+    kt, vt = cache.layer_tensors(0, torch.float16)
+    _, _, strides = cache.layer(0)
+    x = torch.zeros((n, b, hidden), dtype=torch.float16, device="cuda")
+    q = torch.zeros((n, b, hq, D), dtype=torch.float16, device="cuda")
+    att = torch.zeros_like(q)
+    dev = [to_dev(a, dtype) for a in (*w, rope)]
+    qkv = ellm_amd.MatMul3(x, dev[0], q, dev[1], kt, dev[2], vt, dev[3], D, b, hq, hkv, strides, cap)
+    attn = ellm_amd.Attention(q, kt, vt, att, b, hq, hkv, D, strides, 1.0 / np.sqrt(D), sequence_capacity=cap,
+                              max_position_interval=n)
+    stream = torch.cuda.Stream()
+
+    def step():
+        qkv.run(0, n, b, stream=stream)
+        attn.run(0, n, b, stream=stream)
+
+    def fresh(i):
+        x.copy_(to_dev(rand_storage((n, b, hidden), 300 + i, dtype), dtype))
+        for t in (q, att, kt, vt):
+            t.zero_()
+
+    eager = []
+    for i in range(2):
+        fresh(i)
+        torch.cuda.synchronize()
+        step()
+        stream.synchronize()
+        eager.append((q.clone(), att.clone(), kt.clone(), vt.clone()))
+    with ellm_amd.StepGraph(stream) as graph:
+        step()
+    for i in range(2):
+        fresh(i)
+        torch.cuda.synchronize()
+        graph.launch()
+        stream.synchronize()
+        for got, want in zip((q, att, kt, vt), eager[i]):
+            assert torch.equal(got, want), i
+    # a few rows of the projection against the oracle (rows as sequences of a one-token call)
+    rows = np.array([0, 255, 256, 4095, 5699], dtype=np.uint32)
+    hid = rand_storage((n, b, hidden), 301, dtype)[rows, 0][None]
+    oq = np.zeros((1, len(rows), hq, D), dtype=np.uint16)
+    okc = np.zeros((len(rows), hkv, cap, D), dtype=np.uint16)
+    ovc = np.zeros_like(okc)
+    assert orc.matmul3(np.ascontiguousarray(hid), *w, oq, okc, ovc, rope, (hkv * cap * D, cap * D, D, 1), cap, 0, 1,
+                       dtype, positions=rows) == 0
+    assert compare_ulps(to_host(q, dtype)[rows, 0], orc.from_storage(oq, dtype)[0], dtype)["ok"]
+    graph.close()
+    qkv.close()
+    attn.close()
+    cache.close()
