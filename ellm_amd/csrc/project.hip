@@ -202,7 +202,8 @@ __global__ __launch_bounds__(kProjThreads) void project_kernel(ProjectKernelArgs
     __builtin_amdgcn_s_barrier();
   }
 
-  finish_head<S, MODE, 4>(p, acc, 2 * tn + wn, row0 + wm * 128, lds0 + wave * kEpWaveBytes, lane);
+  const HeadRows<4> head = prepare_head<S, MODE, 4>(p, 2 * tn + wn, row0 + wm * 128, lane);
+  finish_head<S, MODE, 4>(p, acc, head, lds0 + wave * kEpWaveBytes, lane);
 }
 
 }  // namespace

@@ -26,42 +26,74 @@ constexpr int kEpWaveBytes = 32 * kEpPitch + 32 * 8;  // 32 rows and their desti
 // (table or residual) of token block mb + 1 is requested before block mb is worked on.
 // One code path: a head that is not normalised and rotated runs the same arithmetic
 // with scale 1 and the rotation (cos, sin) = (1, 0), which leaves every value as it is.
-template <typename S, int MODE, int MB>
-__device__ __forceinline__ void finish_head(const ProjectKernelArgs& p, f32x16 (&acc)[4][MB],
-                                            uint32_t hh, uint32_t first_row, uint32_t ep_rows,
-                                            int lane) {
-  using M = Mfma<S>;
-  const int j = lane & 31, g = lane >> 5;
-  const uint32_t heads_total = p.heads0 + 2 * p.heads_kv;
-  if (hh >= heads_total) return;
-  const uint32_t seg = (hh < p.heads0) ? 0u : (hh < p.heads0 + p.heads_kv ? 1u : 2u);
-  const uint32_t hs = hh - (seg == 0 ? 0u : (seg == 1 ? p.heads0 : p.heads0 + p.heads_kv));
-  const bool finalize = MODE == kModeQkv && ((seg == 1) || (seg == 0 && p.finalize0));
-  uint16_t* const dst = (seg == 0) ? p.out0 : (seg == 1 ? p.k_out : p.v_out);
+// Where the rows of one head x 32 MB tokens go and what is combined with them, plus the extra
+// operand of token block 0, already requested: a kernel with registers to spare calls
+// prepare_head() ahead of its main loop, so that neither the positions nor the first table /
+// residual rows are waited for after it.
+template <int MB>
+struct HeadRows {
   uint16_t* out_row[MB];
   const uint16_t* ext_row[MB];
   bool live[MB];
+  bool present;    // false: the head lies beyond the last one (odd head count), nothing to do
+  bool finalize;   // normalise + rotate
+  u32x2 ext0[16];
+};
+
+template <typename S, int MODE, int MB>
+__device__ __forceinline__ HeadRows<MB> prepare_head(const ProjectKernelArgs& p, uint32_t hh,
+                                                     uint32_t first_row, int lane) {
+  using M = Mfma<S>;
+  HeadRows<MB> h;
+  const int j = lane & 31, g = lane >> 5;
+  const uint32_t heads_total = p.heads0 + 2 * p.heads_kv;
+  h.present = hh < heads_total;
+  const uint32_t seg = (hh < p.heads0) ? 0u : (hh < p.heads0 + p.heads_kv ? 1u : 2u);
+  const uint32_t hs = hh - (seg == 0 ? 0u : (seg == 1 ? p.heads0 : p.heads0 + p.heads_kv));
+  h.finalize = MODE == kModeQkv && ((seg == 1) || (seg == 0 && p.finalize0));
+  uint16_t* const dst = (seg == 0) ? p.out0 : (seg == 1 ? p.k_out : p.v_out);
 #pragma unroll
   for (int mb = 0; mb < MB; ++mb) {
     const uint32_t R = first_row + 32 * mb + j;
     const uint32_t t = R / p.batch_pitch, b = R % p.batch_pitch;
-    live[mb] = R < p.rows && b < p.batch;
+    h.live[mb] = h.present && R < p.rows && b < p.batch;
     uint32_t pos = t;
     if (p.positions)
-      pos += live[mb] ? min(p.positions[b], p.max_start) : 0u;
+      pos += h.live[mb] ? min(p.positions[b], p.max_start) : 0u;
     else
       pos += p.position_index;
     const size_t col = hs * kHeadDim;
     if (seg == 0)
-      out_row[mb] = dst + (size_t)R * p.ld0 + col;
+      h.out_row[mb] = dst + (size_t)R * p.ld0 + col;
     else
-      out_row[mb] = dst + (size_t)b * p.kv_stride_seq + (size_t)hs * p.kv_stride_head +
-                    (size_t)pos * p.kv_stride_pos;
+      h.out_row[mb] = dst + (size_t)b * p.kv_stride_seq + (size_t)hs * p.kv_stride_head +
+                      (size_t)pos * p.kv_stride_pos;
     if (MODE == kModeQkv)
-      ext_row[mb] = p.rope + (size_t)pos * p.rope_pos_stride + (size_t)hs * p.rope_head_stride + 4 * g;
+      h.ext_row[mb] = p.rope + (size_t)pos * p.rope_pos_stride + (size_t)hs * p.rope_head_stride + 4 * g;
     else
-      ext_row[mb] = p.residual + (size_t)R * p.ld0 + col + 4 * g;
+      h.ext_row[mb] = p.residual + (size_t)R * p.ld0 + col + 4 * g;
   }
+  const uint32_t one_zero = M::pack2(1.0f, 0.0f);
+  if ((MODE == kModeAdd || h.finalize) && h.live[0]) {
+#pragma unroll
+    for (int i = 0; i < 16; ++i) h.ext0[i] = *(const u32x2*)(h.ext_row[0] + 32 * (i >> 2) + 8 * (i & 3));
+  } else {
+#pragma unroll
+    for (int i = 0; i < 16; ++i) h.ext0[i] = u32x2{one_zero, one_zero};
+  }
+  return h;
+}
+
+template <typename S, int MODE, int MB>
+__device__ __forceinline__ void finish_head(const ProjectKernelArgs& p, f32x16 (&acc)[4][MB],
+                                            const HeadRows<MB>& h, uint32_t ep_rows, int lane) {
+  using M = Mfma<S>;
+  const int j = lane & 31, g = lane >> 5;
+  if (!h.present) return;
+  const bool finalize = h.finalize;
+  const auto& out_row = h.out_row;
+  const auto& ext_row = h.ext_row;
+  const auto& live = h.live;
   const uint32_t ep_table = ep_rows + 32 * kEpPitch;
   const uint32_t one_zero = M::pack2(1.0f, 0.0f);
   u32x2 ext[2][16];
@@ -74,7 +106,8 @@ __device__ __forceinline__ void finish_head(const ProjectKernelArgs& p, f32x16 (
       for (int i = 0; i < 16; ++i) ext[set][i] = u32x2{one_zero, one_zero};
     }
   };
-  fetch_ext(std::integral_constant<int, 0>{}, 0);
+#pragma unroll
+  for (int i = 0; i < 16; ++i) ext[0][i] = h.ext0[i];
   static_for<MB>([&](auto mb_) {
     constexpr int mb = decltype(mb_)::value;
     constexpr int set = mb & 1;

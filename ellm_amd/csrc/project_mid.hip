@@ -133,6 +133,9 @@ __global__ __launch_bounds__(kMidThreads) void project_mid_kernel(ProjectKernelA
   for (int k = 0; k < Shape::kAhead; ++k)
 #pragma unroll
     for (int i = 0; i < kLoads; ++i) load_piece(k, i);
+  // (requested behind the first chunks, used after the loop: destinations, positions and the
+  // first rows of the rotary table or the residual)
+  const HeadRows<MB> head = prepare_head<S, MODE, MB>(p, tn, row0 + 32 * MB * wave, lane);
   if constexpr (MB == 1)
     asm volatile("s_waitcnt vmcnt(16)" ::: "memory");   // Shape::kMayBePending
   else
@@ -186,7 +189,7 @@ __global__ __launch_bounds__(kMidThreads) void project_mid_kernel(ProjectKernelA
   }
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the last (empty) requests still write LDS
   __syncthreads();
-  finish_head<S, MODE, MB>(p, acc, tn, row0 + 32 * MB * wave, lds0 + wave * kEpWaveBytes, lane);
+  finish_head<S, MODE, MB>(p, acc, head, lds0 + wave * kEpWaveBytes, lane);
 }
 
 template <int MB>
