@@ -106,6 +106,7 @@ ABI_SYMBOLS = {
     "ellm_attn_destroy": (ctypes.c_int, [_vp]),
     "ellm_attn_run": (ctypes.c_int, [_vp, _sz, _sz, _sz, _vp]),
     "ellm_attn_run_ragged": (ctypes.c_int, [_vp, _vp, _sz, _sz, _vp]),
+    "ellm_attn_run_noalloc": (ctypes.c_int, [ctypes.POINTER(AttnDesc), _vp, _sz, _sz, _vp]),
     "ellm_kv_create": (ctypes.c_int, [ctypes.POINTER(KvDesc), _pvp]),
     "ellm_kv_destroy": (ctypes.c_int, [_vp]),
     "ellm_kv_layer": (ctypes.c_int, [_vp, _sz, _pvp, _pvp, ctypes.POINTER(_sz * 4)]),

@@ -113,6 +113,13 @@ class Attention:
         check(self._lib.ellm_attn_run_ragged(self._handle, _positions_ptr(positions, batch_size),
                                              int(max_position), batch_size, _stream_ptr(stream)))
 
+    def run_noalloc(self, position, batch_size, positions=None, stream=None):
+        """The single-token step through ellm_attn_run_noalloc: this operator's description,
+        the library's static device scratch instead of the handle's workspace."""
+        pos_ptr = _positions_ptr(positions, batch_size) if positions is not None else None
+        check(self._lib.ellm_attn_run_noalloc(ctypes.byref(self.desc), pos_ptr, int(position),
+                                              batch_size, _stream_ptr(stream)))
+
     def close(self):
         if self._handle:
             check(self._lib.ellm_attn_destroy(self._handle))

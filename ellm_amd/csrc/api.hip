@@ -67,6 +67,72 @@ int ellm::set_error(int status, const char* fmt, ...) {
   return status;
 }
 
+int ellm::validate_attn_desc(const ellm_attn_desc* d) {
+  if (!d) return fail(ELLM_ERR_INVALID_ARGUMENT, "null descriptor");
+  if (!d->q || !d->k || !d->v || !d->out)
+    return fail(ELLM_ERR_INVALID_ARGUMENT, "q, k, v and out must be non-null device pointers");
+  if (!aligned16(d->q) || !aligned16(d->k) || !aligned16(d->v) || !aligned16(d->out))
+    return fail(ELLM_ERR_INVALID_ARGUMENT, "q, k, v and out must be 16-byte aligned");
+  if (d->dtype != ELLM_DTYPE_F16 && d->dtype != ELLM_DTYPE_BF16)
+    return fail(ELLM_ERR_INVALID_ARGUMENT, "dtype %d is neither ELLM_DTYPE_F16 nor ELLM_DTYPE_BF16",
+                d->dtype);
+  if (d->head_size != 128)
+    return fail(ELLM_ERR_UNSUPPORTED, "head_size %zu: only 128 is supported", d->head_size);
+  if (d->batch_size == 0 || d->attention_head_num == 0 || d->kv_head_num == 0)
+    return fail(ELLM_ERR_INVALID_ARGUMENT, "batch_size, attention_head_num, kv_head_num must be > 0");
+  if (d->attention_head_num % d->kv_head_num != 0)
+    return fail(ELLM_ERR_INVALID_ARGUMENT, "attention_head_num %zu is not a multiple of kv_head_num %zu",
+                d->attention_head_num, d->kv_head_num);
+  if (d->kv_strides[3] != 1)
+    return fail(ELLM_ERR_INVALID_ARGUMENT, "kv_strides[3] must be 1 (head dimension contiguous)");
+  for (int i = 0; i < 3; ++i)
+    if (d->kv_strides[i] == 0 || d->kv_strides[i] % 8 != 0)
+      return fail(ELLM_ERR_INVALID_ARGUMENT,
+                  "kv_strides[%d] = %zu must be a non-zero multiple of 8 elements", i,
+                  d->kv_strides[i]);
+  if (d->kv_strides[2] < d->head_size)
+    return fail(ELLM_ERR_INVALID_ARGUMENT, "kv_strides[2] = %zu is smaller than head_size",
+                d->kv_strides[2]);
+  if (d->sequence_capacity == 0 || d->sequence_capacity > 0x7fffffffu)
+    return fail(ELLM_ERR_INVALID_ARGUMENT, "sequence_capacity %zu out of range", d->sequence_capacity);
+  if (d->sequence_capacity * d->kv_strides[2] > 0x7fffffffu)
+    return fail(ELLM_ERR_UNSUPPORTED,
+                "a K/V plane spans %zu elements; offsets inside a plane are 32-bit (max 2^31 - 1)",
+                d->sequence_capacity * d->kv_strides[2]);
+  if (d->max_position_interval == 0 || d->max_position_interval > d->sequence_capacity)
+    return fail(ELLM_ERR_INVALID_ARGUMENT,
+                "max_position_interval %zu must be in 1..sequence_capacity", d->max_position_interval);
+  if (d->batch_size > 65535 || d->attention_head_num > 65535)
+    return fail(ELLM_ERR_UNSUPPORTED, "batch_size and attention_head_num are limited to 65535");
+  if (!(d->inverse_sqrt_head == d->inverse_sqrt_head))
+    return fail(ELLM_ERR_INVALID_ARGUMENT, "inverse_sqrt_head is NaN");
+  return ELLM_OK;
+}
+
+void ellm::attn_args_from_desc(const ellm_attn_desc& d, ellm::AttnArgs* a) {
+  a->q = d.q;
+  a->k = d.k;
+  a->v = d.v;
+  a->out = d.out;
+  a->lse = d.lse;
+  a->batch_pitch = (uint32_t)d.batch_size;
+  a->n_q_heads = (uint32_t)d.attention_head_num;
+  a->n_kv_heads = (uint32_t)d.kv_head_num;
+  a->group = a->n_q_heads / a->n_kv_heads;
+  a->kv_stride_seq = d.kv_strides[0];
+  a->kv_stride_head = d.kv_strides[1];
+  a->kv_stride_pos = d.kv_strides[2];
+  a->scale = d.inverse_sqrt_head;
+  a->dtype = d.dtype;
+  a->capacity = (uint32_t)d.sequence_capacity;
+  a->ws_acc = a->ws_ml = a->ws2_acc = a->ws2_ml = nullptr;
+  a->counters = nullptr;
+  a->prefill_part_o = a->prefill_part_ml = nullptr;
+  a->prefill_part_rows = 0;
+  a->n_cu = 0;
+  a->positions = nullptr;
+}
+
 struct ellm_attn {
   ellm_attn_desc desc;
   int device;
@@ -129,47 +195,12 @@ int ellm_device_count(void) {
 int ellm_attn_create(const ellm_attn_desc* d, ellm_attn** out_handle) {
   if (!d || !out_handle) return fail(ELLM_ERR_INVALID_ARGUMENT, "null descriptor or handle pointer");
   *out_handle = nullptr;
-  if (!d->q || !d->k || !d->v || !d->out)
-    return fail(ELLM_ERR_INVALID_ARGUMENT, "q, k, v and out must be non-null device pointers");
-  if (!aligned16(d->q) || !aligned16(d->k) || !aligned16(d->v) || !aligned16(d->out))
-    return fail(ELLM_ERR_INVALID_ARGUMENT, "q, k, v and out must be 16-byte aligned");
-  if (d->dtype != ELLM_DTYPE_F16 && d->dtype != ELLM_DTYPE_BF16)
-    return fail(ELLM_ERR_INVALID_ARGUMENT, "dtype %d is neither ELLM_DTYPE_F16 nor ELLM_DTYPE_BF16",
-                d->dtype);
-  if (d->head_size != 128)
-    return fail(ELLM_ERR_UNSUPPORTED, "head_size %zu: only 128 is supported", d->head_size);
-  if (d->batch_size == 0 || d->attention_head_num == 0 || d->kv_head_num == 0)
-    return fail(ELLM_ERR_INVALID_ARGUMENT, "batch_size, attention_head_num, kv_head_num must be > 0");
-  if (d->attention_head_num % d->kv_head_num != 0)
-    return fail(ELLM_ERR_INVALID_ARGUMENT, "attention_head_num %zu is not a multiple of kv_head_num %zu",
-                d->attention_head_num, d->kv_head_num);
-  if (d->kv_strides[3] != 1)
-    return fail(ELLM_ERR_INVALID_ARGUMENT, "kv_strides[3] must be 1 (head dimension contiguous)");
-  for (int i = 0; i < 3; ++i)
-    if (d->kv_strides[i] == 0 || d->kv_strides[i] % 8 != 0)
-      return fail(ELLM_ERR_INVALID_ARGUMENT,
-                  "kv_strides[%d] = %zu must be a non-zero multiple of 8 elements", i,
-                  d->kv_strides[i]);
-  if (d->kv_strides[2] < d->head_size)
-    return fail(ELLM_ERR_INVALID_ARGUMENT, "kv_strides[2] = %zu is smaller than head_size",
-                d->kv_strides[2]);
-  if (d->sequence_capacity == 0 || d->sequence_capacity > 0x7fffffffu)
-    return fail(ELLM_ERR_INVALID_ARGUMENT, "sequence_capacity %zu out of range", d->sequence_capacity);
-  if (d->sequence_capacity * d->kv_strides[2] > 0x7fffffffu)
-    return fail(ELLM_ERR_UNSUPPORTED,
-                "a K/V plane spans %zu elements; offsets inside a plane are 32-bit (max 2^31 - 1)",
-                d->sequence_capacity * d->kv_strides[2]);
-  if (d->max_position_interval == 0 || d->max_position_interval > d->sequence_capacity)
-    return fail(ELLM_ERR_INVALID_ARGUMENT,
-                "max_position_interval %zu must be in 1..sequence_capacity", d->max_position_interval);
-  if (d->batch_size > 65535 || d->attention_head_num > 65535)
-    return fail(ELLM_ERR_UNSUPPORTED, "batch_size and attention_head_num are limited to 65535");
-  if (!(d->inverse_sqrt_head == d->inverse_sqrt_head))
-    return fail(ELLM_ERR_INVALID_ARGUMENT, "inverse_sqrt_head is NaN");
+  if (int st = ellm::validate_attn_desc(d)) return st;
 
   int device = 0, n_cu = 0;
   int st = ellm::current_gfx950_device(&device, &n_cu);
   if (st != ELLM_OK) return st;
+  ellm::prepare_static_scratch();
 
   ellm_attn* h = new (std::nothrow) ellm_attn;
   if (!h) return fail(ELLM_ERR_HIP, "out of host memory");
@@ -209,22 +240,7 @@ int ellm_attn_destroy(ellm_attn* h) {
 }
 
 static void fill_args(const ellm_attn* h, ellm::AttnArgs* a) {
-  const ellm_attn_desc& d = h->desc;
-  a->q = d.q;
-  a->k = d.k;
-  a->v = d.v;
-  a->out = d.out;
-  a->lse = d.lse;
-  a->batch_pitch = (uint32_t)d.batch_size;
-  a->n_q_heads = (uint32_t)d.attention_head_num;
-  a->n_kv_heads = (uint32_t)d.kv_head_num;
-  a->group = a->n_q_heads / a->n_kv_heads;
-  a->kv_stride_seq = d.kv_strides[0];
-  a->kv_stride_head = d.kv_strides[1];
-  a->kv_stride_pos = d.kv_strides[2];
-  a->scale = d.inverse_sqrt_head;
-  a->dtype = d.dtype;
-  a->capacity = (uint32_t)d.sequence_capacity;
+  ellm::attn_args_from_desc(h->desc, a);
   a->ws_acc = h->ws_acc;
   a->ws_ml = h->ws_ml;
   a->ws2_acc = h->ws2_acc;
@@ -234,7 +250,6 @@ static void fill_args(const ellm_attn* h, ellm::AttnArgs* a) {
   a->prefill_part_ml = h->part_ml;
   a->prefill_part_rows = h->part_rows;
   a->n_cu = (uint32_t)h->n_cu;
-  a->positions = nullptr;
 }
 
 static int run_decode(ellm_attn* h, ellm::AttnArgs* a, uint32_t max_position, hipStream_t stream) {
@@ -323,6 +338,7 @@ int ellm_kv_create(const ellm_kv_desc* d, ellm_kv_cache** out_cache) {
   int device = 0, n_cu = 0;
   int st = ellm::current_gfx950_device(&device, &n_cu);
   if (st != ELLM_OK) return st;
+  ellm::prepare_static_scratch();
 
   ellm_kv_cache* c = new (std::nothrow) ellm_kv_cache;
   if (!c) return fail(ELLM_ERR_HIP, "out of host memory");

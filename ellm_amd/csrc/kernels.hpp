@@ -5,6 +5,8 @@
 #include <stddef.h>
 #include <stdint.h>
 
+struct ellm_attn_desc;
+
 namespace ellm {
 
 // Everything a launch needs; filled by the C ABI after validation.
@@ -132,6 +134,15 @@ int current_gfx950_device(int* device, int* n_cu);
 // ELLM_OK when `device` (the one a handle was created on) is the calling thread's current
 // device; a handle's workspace and the caller's buffers live on that device only.
 int check_current_device(int device);
+
+// The checks ellm_attn_create applies to a description (status + message recorded), and the
+// shape part of AttnArgs taken from a checked description (workspace pointers left null).
+int validate_attn_desc(const ellm_attn_desc* d);
+void attn_args_from_desc(const ellm_attn_desc& d, AttnArgs* a);
+
+// Looks up, once per device, the address of the current device's copy of the static scratch
+// that ellm_attn_run_noalloc uses (noalloc.hip).
+void prepare_static_scratch();
 
 // Records the message ellm_last_error_string() returns on this thread; returns status.
 int set_error(int status, const char* fmt, ...) __attribute__((format(printf, 2, 3)));

@@ -128,6 +128,32 @@ int ellm_attn_run(ellm_attn* handle, size_t position_index, size_t position_inte
 int ellm_attn_run_ragged(ellm_attn* handle, const uint32_t* positions, size_t max_position,
                          size_t batch_size, void* stream);
 
+/*
+ * The single-token step of ellm_attn_run / ellm_attn_run_ragged (position_interval == 1)
+ * without a handle and without any allocation.  No counterpart in the reference: it is
+ * for callers that cannot call hipMalloc — code under HIP graph capture, tight serving
+ * loops, harnesses that forbid allocation.  The description is read on every call (q, k,
+ * v, out, lse, strides, scale as for ellm_attn_create; max_position_interval is ignored
+ * beyond its range check); nothing is created and nothing needs destroying.
+ *   positions == NULL : every sequence attends to keys 0..=position;
+ *   positions != NULL : device uint32[batch_size], one position per sequence, each
+ *                       clamped to `position` (their upper bound, which sizes the launch).
+ * Same kernel and split plan as the handle's path, so the results are bit-identical.
+ * The split partials and arrival counters live in a static device array of 5,074,944
+ * bytes that every device the library runs on holds until the process ends; the call
+ * uses the current device's copy.  Limit: sequences x query heads x splits <= 8192
+ * partial rows, which covers GQA groups of up to 16 query heads on a 256-unit part;
+ * larger shapes return ELLM_ERR_OUT_OF_RANGE and must use a handle.  Every call on a
+ * device shares that device's array: calls that overlap on one device (two streams, or
+ * two graphs replayed at once) race; calls in stream order do not.  It calls no
+ * hipMalloc / hipFree and launches kernels only (the counters are cleared by a small
+ * fill kernel), so it may be recorded into a graph; the first call on a device looks up
+ * the array's address (any ellm_attn_create / ellm_kv_create on that device has done so
+ * already).
+ */
+int ellm_attn_run_noalloc(const ellm_attn_desc* desc, const uint32_t* positions, size_t position,
+                          size_t batch_size, void* stream);
+
 /* ------------------------------------------------------------------------ *
  * Key/value cache: one allocation, [layer][sequence][kv_head][position][128],
  * for keys and one for values, written in place at token coordinates.
