@@ -54,35 +54,55 @@ def _dev_normal(shape, dtype, seed, scale=1.0):
     return x.to(dtype)
 
 
-def _time_steps(fn, steps, warmup):
-    """W untimed steps, then exactly K steps between two synchronisation points.
+MIN_TIMED_MS = 100.0   # a measurement repeats its K-step pass until this much has been timed
+MAX_PASSES = 400
+_last_passes = 0
 
-    Returns ([average launch duration in ms], host-clock ms per step).  The host clock
-    brackets the first K-step pass with torch.cuda.synchronize() on both sides.  The
-    launch duration comes from a second K-step pass bracketed by two HIP events on the
-    launch stream (the library launches on torch's current stream, where the events
-    are recorded too): one step of either workload is a single kernel launch and the
-    launches run back to back, so elapsed / K is that kernel's average duration
-    (an event pair around every single launch adds several microseconds of
-    command-processor work per step and overstates a 50 us kernel by 10 %)."""
+
+def _time_steps(fn, steps, warmup, min_ms=None):
+    """W untimed steps, then passes of exactly K steps each, every pass between two
+    synchronisation points, repeated until MIN_TIMED_MS of device time has been measured
+    (a 20-step pass of a 47 us kernel is 1 ms: one preemption or clock ramp moves it by
+    several per cent).  Returns ([median launch duration in ms], median host-clock ms per step).
+
+    Per pass the host clock brackets the K steps with torch.cuda.synchronize() on both sides,
+    and two HIP events recorded on the launch stream (the library launches on torch's current
+    stream, where the events are recorded too) bracket the same K launches: one step of a
+    single-kernel workload is one launch and the launches run back to back, so elapsed / K
+    is that kernel's average duration (an event pair around every single launch adds several
+    microseconds of command-processor work per step and overstates a 50 us kernel by 10 %).
+    The number of passes of the last call is left in _last_passes."""
+    import statistics
+
     import torch
 
+    global _last_passes
+    if min_ms is None:
+        min_ms = MIN_TIMED_MS
     for i in range(warmup):
         fn(i)
     torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for i in range(steps):
-        fn(warmup + i)
-    torch.cuda.synchronize()
-    step_ms = (time.perf_counter() - t0) * 1e3 / steps
-    start = torch.cuda.Event(enable_timing=True)
-    stop = torch.cuda.Event(enable_timing=True)
-    start.record()
-    for i in range(steps):
-        fn(warmup + i)
-    stop.record()
-    torch.cuda.synchronize()
-    return [start.elapsed_time(stop) / steps], step_ms
+    host, dev, total = [], [], 0.0
+    n = warmup
+    while True:
+        start = torch.cuda.Event(enable_timing=True)
+        stop = torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        start.record()
+        for i in range(steps):
+            fn(n + i)
+        stop.record()
+        torch.cuda.synchronize()
+        host.append((time.perf_counter() - t0) * 1e3 / steps)
+        ms = start.elapsed_time(stop)
+        dev.append(ms / steps)
+        total += ms
+        n += steps
+        if total >= min_ms or len(dev) >= MAX_PASSES:
+            break
+    _last_passes = len(dev)
+    return [statistics.median(dev)], statistics.median(host)
 
 
 def bench_decode(batch, length, steps, warmup, hq=32, hkv=4, copies=4):
@@ -113,6 +133,7 @@ def bench_decode(batch, length, steps, warmup, hq=32, hkv=4, copies=4):
         "kernel_ms": kern_ms,
         "gbs": alg_bytes / (step_ms * 1e-3) / 1e9,
         "kernel_gbs": alg_bytes / (kern_ms * 1e-3) / 1e9,
+        "passes": _last_passes,
     }
 
 
@@ -128,9 +149,10 @@ def bench_prefill(seq, steps, warmup, hq=32, hkv=4, dtype_name="f16", p0=0, zero
     g.manual_seed(5)
     qs = torch.rand((1, 1, hq, 1), generator=g, device="cuda") * 1.5 + 0.5   # per-head scale U[0.5, 2]
     ks = torch.rand((1, hkv, 1, 1), generator=g, device="cuda") * 1.5 + 0.5
+    vs = torch.rand((1, hkv, 1, 1), generator=g, device="cuda") * 1.5 + 0.5
     q = (_dev_normal((seq, 1, hq, D), torch.float32, 11) * qs).to(dt)
     k = (_dev_normal((1, hkv, cap, D), torch.float32, 12) * ks).to(dt)
-    v = (_dev_normal((1, hkv, cap, D), torch.float32, 13) * ks).to(dt)
+    v = (_dev_normal((1, hkv, cap, D), torch.float32, 13) * vs).to(dt)
     if zero_kv:  # diagnostic: same instruction stream, operands that toggle nothing
         k.zero_()
         v.zero_()
@@ -148,6 +170,7 @@ def bench_prefill(seq, steps, warmup, hq=32, hkv=4, dtype_name="f16", p0=0, zero
         "kernel_ms": kern_ms,
         "tflops": flops / (step_ms * 1e-3) / 1e12,
         "kernel_tflops": flops / (kern_ms * 1e-3) / 1e12,
+        "passes": _last_passes,
     }
 
 
@@ -541,32 +564,202 @@ def bench_chunk_block(positions, batch, p0, steps, warmup, hidden=2048, hq=32, h
     return {"block_ms": block_ms, "parts_ms": parts, "flops": flops}
 
 
-def cpu_baseline_decode(batch, length, hq=32, hkv=4, budget_s=1.5):
-    """The CPU oracle on the full single-token workload (all host cores), repeated for about
-    `budget_s` seconds of wall time (x 16 threads: 20-odd core-seconds of CPU work)."""
+def _host_info():
+    """CPU model, logical cores of the machine, and the threads the CPU baselines use: one per
+    core this process may run on, at most the CPU share the environment states
+    (OMP_NUM_THREADS, which a shared GPU box sets to its per-GPU share of the host)."""
+    model = "unknown"
+    try:
+        with open("/proc/cpuinfo") as f:
+            for line in f:
+                if line.startswith("model name"):
+                    model = line.split(":", 1)[1].strip()
+                    break
+    except OSError:
+        pass
+    try:
+        allowed = len(os.sched_getaffinity(0))
+    except AttributeError:
+        allowed = os.cpu_count() or 1
+    share = os.environ.get("OMP_NUM_THREADS", "")
+    cores = min(allowed, int(share)) if share.isdigit() and int(share) > 0 else allowed
+    return {"cpu_model": model, "host_cores": os.cpu_count() or 1, "cores": max(1, cores)}
+
+
+def _cpu_normal(shape, dtype_name, seed):
+    """N(0,1) on the host in the storage type, as a numpy array of bit patterns."""
     import numpy as np
+    import torch
+
+    g = torch.Generator()
+    g.manual_seed(seed)
+    dt = torch.float16 if dtype_name == "f16" else torch.bfloat16
+    x = torch.randn(shape, generator=g, dtype=torch.float32).to(dt)
+    a = x.view(torch.int16).numpy()
+    return a.view(np.float16) if dtype_name == "f16" else a.view(np.uint16)
+
+
+def cpu_baseline_decode(batch, length, hq=32, hkv=4, budget_s=1.5):
+    """The CPU oracle on the full single-token workload, repeated for about `budget_s` seconds
+    of wall time (x the threads: 20-odd core-seconds of CPU work); one pinned thread per core
+    with the reference's static split and barrier (src/serving/start.rs:43-77)."""
     import oracle_lib as orc
 
-    cores = min(os.cpu_count() or 1, 16)
-    rng = np.random.default_rng(1)
-    q = rng.standard_normal((1, batch, hq, D), dtype=np.float32).astype(np.float16)
-    k = rng.standard_normal((batch, hkv, length, D), dtype=np.float32).astype(np.float16)
-    v = rng.standard_normal((batch, hkv, length, D), dtype=np.float32).astype(np.float16)
+    host = _host_info()
+    cores = host["cores"]
+    q = _cpu_normal((1, batch, hq, D), "f16", 1)
+    k = _cpu_normal((batch, hkv, length, D), "f16", 2)
+    v = _cpu_normal((batch, hkv, length, D), "f16", 3)
+    import numpy as np
     out = np.zeros_like(q)
     op = orc.Operator(q, k, v, out, None, batch, hq, hkv, D, [hkv * length * D, length * D, D, 1],
                       1.0 / D ** 0.5, orc.F16)
-    t1 = op.run_threads(length - 1, 1, batch, cores, pin=False)
+    t1 = op.run_threads(length - 1, 1, batch, cores, pin=True)
     repeats = max(1, min(200, int(budget_s / max(t1, 1e-3))))
-    t = op.run_threads(length - 1, 1, batch, cores, pin=False, repeats=repeats) / repeats
+    t = op.run_threads(length - 1, 1, batch, cores, pin=True, repeats=repeats) / repeats
     alg_bytes = 2 * batch * hkv * length * D * 2 + 2 * batch * hq * D * 2
     return {
         "value": alg_bytes / t / 1e9,
         "unit": "GB/s",
         "cores": cores,
         "kind": "port",
+        "pinned": True,
         "sample": f"full workload ({batch} seq x {length} keys x {hq} heads), {repeats} passes, "
-                  f"{t * 1e3:.1f} ms per pass, one thread per core with the reference's static split",
+                  f"{t * 1e3:.1f} ms per pass, one pinned thread per core with the reference's static split",
     }
+
+
+def _cpu_sampled_rows(op, position_index, pick_rows, row_macs, cores, budget_s, positions=None):
+    """Times the oracle on a seeded sample of (token, sequence, head) rows sized for about
+    `budget_s` seconds of wall time: a pilot of 2 rows per thread gives the rate, then the
+    sample.  pick_rows(n) -> uint32 [n, 3]; row_macs(rows) -> multiply-adds of those rows.
+    Returns (seconds, multiply-adds of the sample, rows)."""
+    pilot = pick_rows(2 * cores)
+    _, _, t0 = op.run_rows(position_index, pilot, cores, positions=positions, pin=True)
+    rate = row_macs(pilot) / max(t0, 1e-4)
+    n = int(min(200000, max(4 * cores, rate * budget_s / (row_macs(pilot) / len(pilot)))))
+    rows = pick_rows(n)
+    _, _, t = op.run_rows(position_index, rows, cores, positions=positions, pin=True)
+    return t, row_macs(rows), len(rows)
+
+
+def cpu_baseline_chunk(seq, p0, hq, hkv, dtype_name, budget_s=1.5, seed=17):
+    """The CPU oracle on a seeded subset of the (token, head) rows of a causal chunk of `seq`
+    tokens on a cache that already holds `p0`, extrapolated to the whole chunk by the count of
+    multiply-adds (a row at position p costs 2 x 128 x (p + 1) of them); the full chunk is
+    10^12 to 10^13 multiply-adds, hours of CPU time."""
+    import numpy as np
+    import oracle_lib as orc
+
+    host = _host_info()
+    cores = host["cores"]
+    cap = p0 + seq
+    code = orc.F16 if dtype_name == "f16" else orc.BF16
+    k = _cpu_normal((1, hkv, cap, D), dtype_name, seed)
+    v = _cpu_normal((1, hkv, cap, D), dtype_name, seed + 1)
+    q = np.zeros((seq, 1, hq, D), dtype=k.dtype)       # untouched pages cost nothing
+    out = np.zeros((1, 1, hq, D), dtype=k.dtype)       # run_rows returns its own rows
+    op = orc.Operator(q, k, v, out, None, 1, hq, hkv, D, [hkv * cap * D, cap * D, D, 1],
+                      1.0 / D ** 0.5, code)
+    rng = np.random.default_rng(seed)
+    qrow = _cpu_normal((D,), dtype_name, seed + 2)
+
+    def pick_rows(n):
+        rows = np.stack((rng.integers(0, seq, size=n), np.zeros(n, dtype=np.int64),
+                         rng.integers(0, hq, size=n)), axis=1).astype(np.uint32)
+        q[rows[:, 0], 0, rows[:, 2]] = qrow
+        return rows
+
+    def row_macs(rows):
+        return float(2 * D * (p0 + rows[:, 0].astype(np.float64) + 1).sum())
+
+    t, macs, n = _cpu_sampled_rows(op, p0, pick_rows, row_macs, cores, budget_s)
+    full_macs = 2.0 * D * hq * (seq * p0 + seq * (seq + 1) / 2)
+    factor = full_macs / macs
+    return {
+        "value": 2 * full_macs / (t * factor) / 1e12,
+        "unit": "TFLOP/s",
+        "cores": cores,
+        "kind": "port",
+        "pinned": True,
+        "sample": f"{n} seeded (token, head) rows of the {seq}-token chunk, {macs / 1e9:.2f} of "
+                  f"{full_macs / 1e9:.0f} G multiply-adds in {t:.2f} s on {cores} pinned threads; the whole "
+                  f"chunk extrapolated by multiply-add count (x {factor:.0f}) would take {t * factor:.0f} s",
+        "extrapolation_factor": factor,
+        "seconds_extrapolated": t * factor,
+    }
+
+
+def cpu_baseline_ragged_decode(lengths, hq=32, hkv=4, sample_seqs=4, seed=19):
+    """The CPU oracle on a single-token step over `sample_seqs` of the drawn sequences (all their
+    query heads), extrapolated to all of them by cached-token count."""
+    import numpy as np
+    import oracle_lib as orc
+
+    host = _host_info()
+    cores = host["cores"]
+    rng = np.random.default_rng(seed)
+    chosen = np.sort(rng.choice(len(lengths), size=min(sample_seqs, len(lengths)), replace=False))
+    lens = np.asarray(lengths)[chosen]
+    cap = int(lens.max())
+    b = len(chosen)
+    k = _cpu_normal((b, hkv, cap, D), "f16", seed)
+    v = _cpu_normal((b, hkv, cap, D), "f16", seed + 1)
+    q = _cpu_normal((1, b, hq, D), "f16", seed + 2)
+    out = np.zeros_like(q)
+    op = orc.Operator(q, k, v, out, None, b, hq, hkv, D, [hkv * cap * D, cap * D, D, 1],
+                      1.0 / D ** 0.5, orc.F16)
+    pos = (lens - 1).astype(np.uint32)
+    t = op.run_threads(0, 1, b, cores, positions=pos, pin=True)
+    factor = float(np.sum(lengths)) / float(lens.sum())
+    nbytes = float(2 * hkv * D * 2 * np.sum(lengths) + 2 * len(lengths) * hq * D * 2)
+    return {
+        "value": nbytes / (t * factor) / 1e9,
+        "unit": "GB/s",
+        "cores": cores,
+        "kind": "port",
+        "pinned": True,
+        "sample": f"{b} of the {len(lengths)} sequences (cache lengths {lens.tolist()}), all {hq} heads, "
+                  f"{t * 1e3:.0f} ms on {cores} pinned threads; extrapolated by cached-token count (x {factor:.2f})",
+        "extrapolation_factor": factor,
+        "seconds_extrapolated": t * factor,
+    }
+
+
+def bench_mfma_stream(mode, dtype_name, n_cu, seconds=0.6, zeros=False, per_cu=1):
+    """What a pure stream of v_mfma_f32_32x32x16 sustains on N(0,1) operands on this box now
+    (libellm_diag.so: one wave per SIMD, four accumulators, no global memory access in the loop;
+    mode 0 register operands, mode 1 the A operand re-read from LDS for every MFMA, mode 2 the
+    same plus the vector instructions of a soft-max of that tile shape in the same wave)."""
+    import ctypes
+
+    import torch
+
+    path = os.path.join(ROOT, "ellm_amd", "lib", "libellm_diag.so")
+    lib = ctypes.CDLL(path)
+    fn = lib.ellm_diag_mfma_stream
+    fn.restype = ctypes.c_int
+    fn.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int,
+                   ctypes.c_int, ctypes.c_void_p, ctypes.POINTER(ctypes.c_double)]
+    dt = torch.float16 if dtype_name == "f16" else torch.bfloat16
+    ops = _dev_normal((16, 256, 8), dt, 91)
+    if zeros:   # the same instruction stream on operands that toggle nothing: what the schedule allows
+        ops.zero_()
+    n_wg = n_cu * per_cu     # per_cu = 2: two waves per SIMD, so one wave's vector work overlaps the other's MFMAs
+    sink = torch.zeros((n_wg * 256,), dtype=torch.float32, device="cuda")
+    flops = ctypes.c_double()
+    iters = 4000      # 128000 MFMAs a wave: ~2.5 ms a launch
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+    def launch(_i):
+        rc = fn(mode, 0 if dtype_name == "f16" else 1, ops.data_ptr(), sink.data_ptr(), n_wg, iters // per_cu, stream,
+                ctypes.byref(flops))
+        if rc:
+            raise RuntimeError(f"ellm_diag_mfma_stream returned {rc}")
+
+    # long enough for the part's power management to settle on its sustained clock
+    per, _ = _time_steps(launch, 40, 40, min_ms=seconds * 1e3)
+    return flops.value / (per[0] * 1e-3) / 1e12
 
 
 def main():
@@ -608,11 +801,22 @@ def main():
 
     also = []
     dec = None
+    host = _host_info()
     if args.only in ("", "decode"):
         dec = bench_decode(16, 8192, args.steps, args.warmup)
     if args.only in ("", "prefill"):
         pf_steps = max(3, min(args.steps, 10))
         pf = bench_prefill(32768, pf_steps, min(args.warmup, 2), zero_kv=args.prefill_zero_kv)
+        # the ceiling this box gives any MFMA kernel on dense random fp16 operands, timed right
+        # after the kernel it is compared with
+        n_cu = torch.cuda.get_device_properties(0).multi_processor_count
+        stream_reg = bench_mfma_stream(0, "f16", n_cu)
+        stream_lds = bench_mfma_stream(1, "f16", n_cu)
+        stream_mix = bench_mfma_stream(2, "f16", n_cu, per_cu=2)
+        stream_mix0 = bench_mfma_stream(2, "f16", n_cu, seconds=0.3, zeros=True, per_cu=2)
+        stream_reg0 = bench_mfma_stream(0, "f16", n_cu, seconds=0.3, zeros=True)
+        stream_lds0 = bench_mfma_stream(1, "f16", n_cu, seconds=0.3, zeros=True)
+        pf_cpu = None if args.skip_cpu else cpu_baseline_chunk(32768, 0, 32, 4, "f16")
         also.append({
             "workload": "prefill: 1 seq x 32768 tokens, 32q/4kv heads, fp16, causal"
                         + (" [DIAGNOSTIC: K = V = 0]" if args.prefill_zero_kv else ""),
@@ -622,6 +826,21 @@ def main():
                          "peak": MFMA_F16_PEAK_TFLOPS, "unit": "TFLOP/s",
                          "frac": round(pf["kernel_tflops"] / MFMA_F16_PEAK_TFLOPS, 4),
                          "traffic": TRAFFIC_BYTES["prefill"]},
+            "passes": pf["passes"],
+            "mfma_stream_on_n01_fp16": {
+                "what": "pure v_mfma_f32_32x32x16_f16 stream on N(0,1) operands, one wave per SIMD on every "
+                        "compute unit, no memory access in the loop, timed in this run (libellm_diag.so)",
+                "register_operands_tflops": round(stream_reg, 1),
+                "a_operand_from_lds_tflops": round(stream_lds, 1),
+                "lds_fed_with_softmax_vector_mix_tflops": round(stream_mix, 1),
+                "same_streams_on_zero_operands_tflops": [round(stream_reg0, 1), round(stream_lds0, 1),
+                                                         round(stream_mix0, 1)],
+                "kernel_frac_of_mix_stream": round(pf["kernel_tflops"] / stream_mix, 4),
+                "frac_of_published_peak": round(stream_reg / MFMA_F16_PEAK_TFLOPS, 4),
+                "kernel_frac_of_register_stream": round(pf["kernel_tflops"] / stream_reg, 4),
+                "kernel_frac_of_lds_fed_stream": round(pf["kernel_tflops"] / stream_lds, 4),
+            },
+            "cpu_baseline": pf_cpu,
         })
     if args.only in ("", "decode128k"):
         d128 = bench_decode(1, 131072, args.steps, args.warmup)
@@ -633,6 +852,7 @@ def main():
                          "peak": HBM_PEAK_GBS, "unit": "GB/s",
                          "frac": round(d128["kernel_gbs"] / HBM_PEAK_GBS, 4),
                          "traffic": TRAFFIC_BYTES["decode128k"]},
+            "passes": d128["passes"],
         })
 
         # the batch of configs[1] at the full cache length: 4.3 GB of K/V a step, far beyond
@@ -653,6 +873,7 @@ def main():
         ck_steps = max(3, min(args.steps, 5))
         ck = bench_prefill(8192, ck_steps, min(args.warmup, 1), hq=64, hkv=8, dtype_name="bf16",
                            p0=120000)
+        ck_cpu = None if args.skip_cpu else cpu_baseline_chunk(8192, 120000, 64, 8, "bf16")
         also.append({
             "workload": "chunked prefill: 8192 new tokens on a 120000-token cache, 64q/8kv heads, "
                         "bf16 (BASELINE configs[3])",
@@ -662,6 +883,8 @@ def main():
                          "peak": MFMA_F16_PEAK_TFLOPS, "unit": "TFLOP/s",
                          "frac": round(ck["kernel_tflops"] / MFMA_F16_PEAK_TFLOPS, 4),
                          "traffic": None},
+            "passes": ck["passes"],
+            "cpu_baseline": ck_cpu,
         })
     if args.only in ("", "smallchunk"):
         # a short chunk of one sequence on a long cache: 8 row-block workgroups, so the key range
@@ -683,6 +906,16 @@ def main():
         md = bench_ragged_decode(32, 1024, 131072, mx_steps, min(args.warmup, 2))
         mq = bench_qkv_projection(16384, mx_steps, min(args.warmup, 2))
         msp = bench_step_projections(32, mx_steps, min(args.warmup, 2))
+        mx_cpu = None
+        if not args.skip_cpu:
+            import numpy as np
+            lengths = np.random.default_rng(7).integers(1024, 131072 + 1, size=32)   # as bench_ragged_decode
+            cp = cpu_baseline_chunk(16384, 0, 32, 4, "f16", budget_s=1.0)
+            cd = cpu_baseline_ragged_decode(lengths)
+            mx_cpu = {"value": round((cp["seconds_extrapolated"] + cd["seconds_extrapolated"]) * 1e3, 1),
+                      "unit": "ms", "cores": cp["cores"], "kind": "port", "pinned": True,
+                      "sample": "prefill side: " + cp["sample"] + "; single-token side: " + cd["sample"],
+                      "prefill_tflops": cp["value"], "decode_gbs": cd["value"]}
         also.append({
             "workload": "mixed step, one of 48 layers (BASELINE configs[4]), kernel by kernel: Q/K/V projection + "
                         "attention of a 16384-token prefill, Q/K/V projection + attention of one new token of 32 "
@@ -701,6 +934,7 @@ def main():
             "roofline": {"bound": "hbm", "achieved": round(md["kernel_gbs"], 1),
                          "peak": HBM_PEAK_GBS, "unit": "GB/s",
                          "frac": round(md["kernel_gbs"] / HBM_PEAK_GBS, 4), "traffic": None},
+            "cpu_baseline": mx_cpu,
         })
 
     if args.only in ("", "mixed48"):
@@ -854,6 +1088,9 @@ def main():
                      "unit": "GB/s", "frac": round(dec["kernel_gbs"] / HBM_PEAK_GBS, 4),
                      "traffic": TRAFFIC_BYTES["decode"]},
         "cpu_baseline": cpu,
+        "passes": dec["passes"],
+        "cpu_model": host["cpu_model"],
+        "host_cores": host["host_cores"],
         "also": also,
     }
     print(json.dumps(line))

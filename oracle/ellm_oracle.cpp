@@ -340,6 +340,33 @@ struct Barrier {
   }
 };
 
+// src/serving/start.rs:43-61 pins worker i to core i (core_affinity::set_for_current).  Here:
+// the i-th core of the set the process was allowed to run on when the pool started, so
+// that a process confined to a share of a machine pins inside its share.
+struct CoreSet {
+  std::vector<int> cores;
+  CoreSet() {
+#if defined(__linux__)
+    cpu_set_t set;
+    CPU_ZERO(&set);
+    if (sched_getaffinity(0, sizeof(set), &set) == 0)
+      for (int c = 0; c < CPU_SETSIZE; ++c)
+        if (CPU_ISSET(c, &set)) cores.push_back(c);
+#endif
+  }
+  void pin_current(size_t tid) const {
+#if defined(__linux__)
+    if (cores.empty()) return;
+    cpu_set_t set;
+    CPU_ZERO(&set);
+    CPU_SET(cores[tid % cores.size()], &set);
+    pthread_setaffinity_np(pthread_self(), sizeof(set), &set);
+#else
+    (void)tid;
+#endif
+  }
+};
+
 }  // namespace
 
 extern "C" {
@@ -447,17 +474,11 @@ double ellm_oracle_attention_run_threads(const ellm_oracle_attn* op, size_t posi
   Barrier barrier(n_threads);
   std::atomic<int> err{0};
   std::vector<std::thread> pool;
+  const CoreSet cores;
   const auto t0 = std::chrono::steady_clock::now();
   for (size_t tid = 0; tid < n_threads; ++tid) {
     pool.emplace_back([&, tid]() {
-#if defined(__linux__)
-      if (pin) {
-        cpu_set_t set;
-        CPU_ZERO(&set);
-        CPU_SET((int)tid, &set);
-        pthread_setaffinity_np(pthread_self(), sizeof(set), &set);
-      }
-#endif
+      if (pin) cores.pin_current(tid);
       for (size_t r = 0; r < repeats; ++r) {
         if (ellm_oracle_attention_run(op, position_index, position_interval, batch_size, positions,
                                       n_threads, tid))
@@ -474,36 +495,49 @@ double ellm_oracle_attention_run_threads(const ellm_oracle_attn* op, size_t posi
 
 // Selected (token, sequence, head) rows only: the bounded sample used when the
 // full problem is too large for the CPU.  rows = n triples (token_in_chunk,
-// sequence, head).  Work is split over threads by the same assign().
-double ellm_oracle_attention_rows_threads(const ellm_oracle_attn* op, size_t position_index,
-                                          const uint32_t* rows, size_t n_rows, void* out_rows,
-                                          float* lse_rows, size_t n_threads) {
+// sequence, head).  Work is split over threads by the same assign().  `positions` (may be
+// null) gives per-sequence positions as in ellm_oracle_attention_run; `pin` pins thread i
+// to the i-th core the process may run on.
+double ellm_oracle_attention_rows_threads_ex(const ellm_oracle_attn* op, size_t position_index,
+                                             const uint32_t* positions, const uint32_t* rows,
+                                             size_t n_rows, void* out_rows, float* lse_rows,
+                                             size_t n_threads, int pin) {
   if (!op || n_threads == 0) return -1.0;
   const size_t heads = op->attention_head_num;
   const size_t group = heads / op->kv_head_num;
   const size_t max_stride = op->batch_capacity * heads;
   std::vector<std::thread> pool;
+  const CoreSet cores;
   const auto t0 = std::chrono::steady_clock::now();
   for (size_t tid = 0; tid < n_threads; ++tid) {
     pool.emplace_back([&, tid]() {
+      if (pin) cores.pin_current(tid);
       size_t begin, end;
       if (!assign(n_rows, n_threads, tid, &begin, &end)) return;
       for (size_t r = begin; r < end; ++r) {
         const size_t high = rows[3 * r], row = rows[3 * r + 1], col = rows[3 * r + 2];
         const size_t index = (high * max_stride + row * heads + col) * op->head_size;
         const size_t kv_index = row * op->kv_strides[0] + (col / group) * op->kv_strides[1];
+        const size_t position = positions ? (size_t)positions[row] : position_index + high;
         flash_attention_row(elem_ptr(op->q, index, op->dtype),
                             elem_ptr(op->k, kv_index, op->dtype),
                             elem_ptr(op->v, kv_index, op->dtype),
                             elem_ptr(out_rows, r * op->head_size, op->dtype),
                             lse_rows ? lse_rows + r : nullptr, op->inverse_sqrt_head,
-                            op->head_size, op->kv_strides[2], position_index + high, op->dtype);
+                            op->head_size, op->kv_strides[2], position, op->dtype);
       }
     });
   }
   for (auto& t : pool) t.join();
   const auto t1 = std::chrono::steady_clock::now();
   return std::chrono::duration<double>(t1 - t0).count();
+}
+
+double ellm_oracle_attention_rows_threads(const ellm_oracle_attn* op, size_t position_index,
+                                          const uint32_t* rows, size_t n_rows, void* out_rows,
+                                          float* lse_rows, size_t n_threads) {
+  return ellm_oracle_attention_rows_threads_ex(op, position_index, nullptr, rows, n_rows, out_rows,
+                                               lse_rows, n_threads, 0);
 }
 
 void ellm_oracle_rms_norm_f32(const float* in, float* out, size_t n, float eps) {

@@ -62,6 +62,9 @@ def load():
     lib.ellm_oracle_attention_rows_threads.restype = ctypes.c_double
     lib.ellm_oracle_attention_rows_threads.argtypes = [
         ctypes.POINTER(OracleAttn), sz, vp, sz, vp, vp, sz]
+    lib.ellm_oracle_attention_rows_threads_ex.restype = ctypes.c_double
+    lib.ellm_oracle_attention_rows_threads_ex.argtypes = [
+        ctypes.POINTER(OracleAttn), sz, vp, vp, sz, vp, vp, sz, ctypes.c_int]
     lib.ellm_oracle_f32_to_f16.restype = ctypes.c_uint16
     lib.ellm_oracle_f32_to_f16.argtypes = [f]
     lib.ellm_oracle_f16_to_f32.restype = f
@@ -276,15 +279,18 @@ class Operator:
             raise RuntimeError("oracle rejected the arguments")
         return t
 
-    def run_rows(self, position_index, rows, n_threads):
-        """rows: uint32 [n, 3] of (token_in_chunk, sequence, head). Returns (out_rows, lse, secs)."""
+    def run_rows(self, position_index, rows, n_threads, positions=None, pin=False):
+        """rows: uint32 [n, 3] of (token_in_chunk, sequence, head); positions: optional uint32
+        per-sequence positions (single-token steps). Returns (out_rows, lse, secs)."""
         rows = np.ascontiguousarray(rows, dtype=np.uint32)
         n = rows.shape[0]
         out = np.zeros((n, self.desc.head_size), dtype=storage_np_dtype(self.desc.dtype))
         lse = np.zeros(n, dtype=np.float32)
-        t = load().ellm_oracle_attention_rows_threads(ctypes.byref(self.desc), position_index,
-                                                      _ptr(rows), n, _ptr(out), _ptr(lse),
-                                                      n_threads)
+        if positions is not None:
+            positions = np.ascontiguousarray(positions, dtype=np.uint32)
+        t = load().ellm_oracle_attention_rows_threads_ex(ctypes.byref(self.desc), position_index,
+                                                         _ptr(positions), _ptr(rows), n, _ptr(out),
+                                                         _ptr(lse), n_threads, int(pin))
         if t < 0:
             raise RuntimeError("oracle rejected the arguments")
         return out, lse, t

@@ -155,3 +155,19 @@ def test_host_mirrors_refuse_host_memory_and_wrong_types():
     with pytest.raises(TypeError, match="device"):
         ellm_amd.MatMul3(x, w, q, w, kv, w, kv, torch.zeros((16, 128), dtype=torch.float16), 128, 1,
                          1, 1, [16 * 128, 16 * 128, 128, 1], 16)
+
+
+def test_diagnostic_library_exports_its_declared_symbol():
+    """libellm_diag.so (the MFMA-stream measurement aid bench.py uses) loads without a GPU and
+    exports what include/ellm_diag.h declares; it rejects bad arguments before any launch."""
+    header = open(os.path.join(ROOT, "include", "ellm_diag.h")).read()
+    header = re.sub(r"/\*.*?\*/", "", header, flags=re.S)
+    declared = set(re.findall(r"\b(ellm_[a-z_0-9]+)\s*\(", header))
+    assert declared == {"ellm_diag_mfma_stream"}
+    lib = ctypes.CDLL(os.path.join(ROOT, "ellm_amd", "lib", "libellm_diag.so"))
+    fn = lib.ellm_diag_mfma_stream
+    fn.restype = ctypes.c_int
+    fn.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int,
+                   ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p]
+    assert fn(0, 0, None, None, 1, 1, None, None) == 1
+    assert fn(7, 0, 0x1000, 0x1000, 1, 1, None, None) == 1

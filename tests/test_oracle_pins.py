@@ -327,6 +327,19 @@ def test_selected_rows_equal_the_full_run():
         assert np.array_equal(got[i], whole[t, b, h]) and got_lse[i] == lse[t, b, h]
 
 
+def test_selected_rows_with_per_sequence_positions_and_pinned_threads_equal_the_full_run():
+    B, hq, hkv, cap = 3, 4, 2, 20
+    q, k, v = _rand((1, B, hq, D), 83), _rand((B, hkv, cap, D), 84), _rand((B, hkv, cap, D), 85)
+    pos = np.array([3, 19, 11], dtype=np.uint32)
+    whole, lse = orc.attention(q, k, v, 0.2, orc.F32, positions=pos)
+    op = orc.Operator(q, k, v, np.zeros_like(q), None, B, hq, hkv, D,
+                      [hkv * cap * D, cap * D, D, 1], 0.2, orc.F32)
+    rows = np.array([[0, b, h] for b in range(B) for h in (0, 3)], dtype=np.uint32)
+    got, got_lse, _ = op.run_rows(0, rows, 3, positions=pos, pin=True)
+    for i, (t, b, h) in enumerate(rows):
+        assert np.array_equal(got[i], whole[t, b, h]) and got_lse[i] == lse[t, b, h]
+
+
 # ---- independent library and committed vectors -------------------------------------------
 
 def test_matches_torch_sdpa():
