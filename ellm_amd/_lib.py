@@ -53,6 +53,26 @@ class KvDesc(ctypes.Structure):
     ]
 
 
+class KvRaggedDesc(ctypes.Structure):
+    _fields_ = [
+        ("layers", ctypes.c_size_t),
+        ("sequences", ctypes.c_size_t),
+        ("kv_head_num", ctypes.c_size_t),
+        ("head_size", ctypes.c_size_t),
+        ("capacities", ctypes.POINTER(ctypes.c_size_t)),
+        ("dtype", ctypes.c_int),
+    ]
+
+
+class KvSeqTable(ctypes.Structure):
+    _fields_ = [
+        ("seq_offsets", ctypes.c_void_p),
+        ("seq_capacity", ctypes.c_void_p),
+        ("seq_capacity_host", ctypes.POINTER(ctypes.c_size_t)),
+        ("sequences", ctypes.c_size_t),
+    ]
+
+
 class MatMul3Desc(ctypes.Structure):
     _fields_ = [
         ("hidden", ctypes.c_void_p),
@@ -108,6 +128,12 @@ ABI_SYMBOLS = {
     "ellm_attn_run_ragged": (ctypes.c_int, [_vp, _vp, _sz, _sz, _vp]),
     "ellm_attn_run_noalloc": (ctypes.c_int, [ctypes.POINTER(AttnDesc), _vp, _sz, _sz, _vp]),
     "ellm_kv_create": (ctypes.c_int, [ctypes.POINTER(KvDesc), _pvp]),
+    "ellm_kv_create_ragged": (ctypes.c_int, [ctypes.POINTER(KvRaggedDesc), _pvp]),
+    "ellm_kv_layer_ragged": (ctypes.c_int, [_vp, _sz, _sz, _pvp, _pvp, ctypes.POINTER(_sz * 4),
+                                            ctypes.POINTER(KvSeqTable)]),
+    "ellm_attn_create_ragged": (ctypes.c_int, [ctypes.POINTER(AttnDesc), ctypes.POINTER(KvSeqTable), _pvp]),
+    "ellm_matmul3_create_ragged": (ctypes.c_int, [ctypes.POINTER(MatMul3Desc), ctypes.POINTER(KvSeqTable),
+                                                  _pvp]),
     "ellm_kv_destroy": (ctypes.c_int, [_vp]),
     "ellm_kv_layer": (ctypes.c_int, [_vp, _sz, _pvp, _pvp, ctypes.POINTER(_sz * 4)]),
     "ellm_kv_append": (ctypes.c_int, [_vp, _sz, _sz, _sz, _sz, _vp, _vp, _sz, _vp]),

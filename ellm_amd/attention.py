@@ -13,7 +13,7 @@ computes with torch.
 import ctypes
 
 from . import _lib
-from ._lib import AttnDesc, KvDesc, check, load_library
+from ._lib import AttnDesc, KvDesc, KvRaggedDesc, KvSeqTable, check, load_library
 
 
 def _dtype_code(t):
@@ -67,16 +67,22 @@ class Attention:
 
     def __init__(self, q, k, v, out, batch_size, attention_head_num, kv_head_num, head_size,
                  kv_strides, inverse_sqrt_head, lse=None, sequence_capacity=None,
-                 max_position_interval=None):
+                 max_position_interval=None, seq_table=None):
+        """seq_table: a KVCache.layer_ragged(...) view, for a cache whose sequences have different
+        capacities (then kv_strides[0] and sequence_capacity are not used)."""
         import torch
 
         self._lib = load_library()
-        self._keep = (q, k, v, out, lse)
-        cap = int(sequence_capacity if sequence_capacity is not None else k.shape[2])
+        self._keep = (q, k, v, out, lse, seq_table)
         interval = int(max_position_interval if max_position_interval is not None else q.shape[0])
         rows = interval * batch_size * attention_head_num
-        kv_span = ((batch_size - 1) * int(kv_strides[0]) + (kv_head_num - 1) * int(kv_strides[1])
-                   + (cap - 1) * int(kv_strides[2]) + head_size)
+        if seq_table is not None:
+            cap = max(seq_table.capacities[:batch_size])
+            kv_span = seq_table.span_elems(batch_size, kv_head_num, int(kv_strides[1]))
+        else:
+            cap = int(sequence_capacity if sequence_capacity is not None else k.shape[2])
+            kv_span = ((batch_size - 1) * int(kv_strides[0]) + (kv_head_num - 1) * int(kv_strides[1])
+                       + (cap - 1) * int(kv_strides[2]) + head_size)
         d = AttnDesc()
         d.q = _device_buffer("q", q, rows * head_size)
         d.out = _device_buffer("out", out, rows * head_size, q.dtype)
@@ -95,7 +101,11 @@ class Attention:
         d.max_position_interval = interval
         self.desc = d
         self._handle = ctypes.c_void_p()
-        check(self._lib.ellm_attn_create(ctypes.byref(d), ctypes.byref(self._handle)))
+        if seq_table is not None:
+            check(self._lib.ellm_attn_create_ragged(ctypes.byref(d), ctypes.byref(seq_table.table),
+                                                    ctypes.byref(self._handle)))
+        else:
+            check(self._lib.ellm_attn_create(ctypes.byref(d), ctypes.byref(self._handle)))
 
     @classmethod
     def new(cls, *args, **kwargs):
@@ -132,15 +142,72 @@ class Attention:
             pass
 
 
-class KVCache:
-    """[layer][sequence][kv_head][position][128] keys and values in one allocation each."""
+class RaggedLayerView:
+    """One layer of a cache with per-sequence capacities, from sequence `first_sequence` on:
+    base addresses, strides and the sequence table to hand to Attention / MatMul3."""
 
-    def __init__(self, layers, sequences, kv_head_num, capacity, dtype_code, head_size=128):
+    def __init__(self, cache, k, v, strides, table, first_sequence):
+        self.cache, self.k, self.v, self.strides, self.table = cache, k, v, strides, table
+        self.first_sequence = first_sequence
+        self.capacities = [int(table.seq_capacity_host[i]) for i in range(table.sequences)]
+        self.offsets = cache.offsets[first_sequence:]
+
+    def span_elems(self, batch_size, kv_head_num, head_stride):
+        """Elements from the layer base that the first batch_size sequences' planes reach."""
+        return max(self.offsets[i] + (kv_head_num - 1) * head_stride + self.capacities[i] * 128
+                   for i in range(batch_size))
+
+
+class KVCache:
+    """Keys and values of every layer in one allocation each: [layer][sequence][kv_head]
+    [position][128] with one capacity, or (KVCache.ragged) [layer][kv_head][sequence: its own
+    positions][128] with a capacity per sequence."""
+
+    def __init__(self, layers, sequences, kv_head_num, capacity, dtype_code, head_size=128,
+                 capacities=None):
         self._lib = load_library()
-        d = KvDesc(layers, sequences, kv_head_num, head_size, capacity, dtype_code)
-        self.desc = d
         self._handle = ctypes.c_void_p()
-        check(self._lib.ellm_kv_create(ctypes.byref(d), ctypes.byref(self._handle)))
+        self.capacities = None
+        if capacities is None:
+            d = KvDesc(layers, sequences, kv_head_num, head_size, capacity, dtype_code)
+            self.desc = d
+            check(self._lib.ellm_kv_create(ctypes.byref(d), ctypes.byref(self._handle)))
+            return
+        caps = (ctypes.c_size_t * len(capacities))(*[int(c) for c in capacities])
+        rd = KvRaggedDesc(layers, len(capacities), kv_head_num, head_size, caps, dtype_code)
+        self.desc = KvDesc(layers, len(capacities), kv_head_num, head_size, max(capacities), dtype_code)
+        self.capacities = [int(c) for c in capacities]
+        self.offsets = [128 * sum(self.capacities[:i]) for i in range(len(capacities))]
+        self.layer_elems = 128 * sum(self.capacities) * kv_head_num
+        check(self._lib.ellm_kv_create_ragged(ctypes.byref(rd), ctypes.byref(self._handle)))
+
+    @classmethod
+    def ragged(cls, layers, capacities, kv_head_num, dtype_code, head_size=128):
+        return cls(layers, len(capacities), kv_head_num, 0, dtype_code, head_size, capacities=capacities)
+
+    def layer_ragged(self, layer, first_sequence=0):
+        k, v = ctypes.c_void_p(), ctypes.c_void_p()
+        strides = (ctypes.c_size_t * 4)()
+        table = KvSeqTable()
+        check(self._lib.ellm_kv_layer_ragged(self._handle, layer, first_sequence, ctypes.byref(k),
+                                             ctypes.byref(v), ctypes.byref(strides), ctypes.byref(table)))
+        return RaggedLayerView(self, k.value, v.value, list(strides), table, first_sequence)
+
+    def layer_flat_tensors(self, layer, torch_dtype):
+        """One layer's K and V of a cache with per-sequence capacities as flat torch tensors
+        [kv_head, positions of all sequences, 128]."""
+        import torch
+
+        view = self.layer_ragged(layer)
+        total = sum(self.capacities)
+        shape = (self.desc.kv_head_num, total, self.desc.head_size)
+
+        def wrap(ptr):
+            iface = {"shape": (self.layer_elems,), "typestr": "<i2", "data": (ptr, False), "version": 2}
+            holder = type("DevBuf", (), {"__cuda_array_interface__": iface})()
+            return torch.as_tensor(holder, device="cuda").view(torch_dtype).view(shape)
+
+        return wrap(view.k), wrap(view.v)
 
     def layer(self, layer):
         k, v = ctypes.c_void_p(), ctypes.c_void_p()

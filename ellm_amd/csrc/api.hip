@@ -6,6 +6,7 @@
 #include <cstdio>
 #include <cstring>
 #include <new>
+#include <vector>
 
 #include "../../include/ellm_attn.h"
 #include "kernels.hpp"
@@ -131,6 +132,8 @@ void ellm::attn_args_from_desc(const ellm_attn_desc& d, ellm::AttnArgs* a) {
   a->prefill_part_rows = 0;
   a->n_cu = 0;
   a->positions = nullptr;
+  a->seq_offsets = nullptr;
+  a->seq_caps = nullptr;
 }
 
 struct ellm_attn {
@@ -147,14 +150,48 @@ struct ellm_attn {
   float* part_o;
   float* part_ml;
   size_t part_rows;
+  // sequences of different capacities (ellm_attn_create_ragged): device tables (borrowed from
+  // the cache) and a host copy of the capacities for the range checks; empty / null otherwise
+  const size_t* seq_offsets;
+  const uint32_t* seq_caps;
+  std::vector<size_t> caps_host;
 };
 
 struct ellm_kv_cache {
-  ellm_kv_desc desc;
+  ellm_kv_desc desc;   // capacity = the largest per-sequence capacity
   int device;
   void* k;
   void* v;
   size_t layer_elems;  // elements per layer
+  // plane of (sequence s, head h) = layer base + offset(s) + h x stride_head.  One capacity for
+  // all: [sequence][kv_head][position][128], offset(s) = s x stride_seq, no tables.  Per-sequence
+  // capacities: [kv_head][sequence: its positions][128], offset(s) = 128 x (positions of the
+  // sequences before s), kept in a device table (and capacities beside it).
+  size_t stride_seq, stride_head;
+  bool ragged;
+  std::vector<size_t> caps_host;      // [sequences]
+  std::vector<size_t> offsets_host;   // [sequences], elements
+  size_t* seq_offsets_dev;            // ragged only
+  uint32_t* seq_caps_dev;             // ragged only
+  ellm::KvLayout layout(size_t first_sequence = 0) const {
+    ellm::KvLayout l;
+    l.stride_seq = stride_seq;
+    l.stride_head = stride_head;
+    l.seq_offsets = ragged ? seq_offsets_dev + first_sequence : nullptr;
+    l.seq_caps = ragged ? seq_caps_dev + first_sequence : nullptr;
+    return l;
+  }
+  // the smallest / largest capacity among sequences [0, n)
+  size_t min_cap(size_t n) const {
+    size_t m = caps_host[0];
+    for (size_t i = 1; i < n; ++i) m = caps_host[i] < m ? caps_host[i] : m;
+    return m;
+  }
+  size_t max_cap(size_t n) const {
+    size_t m = caps_host[0];
+    for (size_t i = 1; i < n; ++i) m = caps_host[i] > m ? caps_host[i] : m;
+    return m;
+  }
 };
 
 static hipError_t free_workspace(ellm_attn* h) {
@@ -192,9 +229,29 @@ int ellm_device_count(void) {
   return usable;
 }
 
-int ellm_attn_create(const ellm_attn_desc* d, ellm_attn** out_handle) {
+static int attn_create(const ellm_attn_desc* d, const ellm_kv_seq_table* table, ellm_attn** out_handle) {
   if (!d || !out_handle) return fail(ELLM_ERR_INVALID_ARGUMENT, "null descriptor or handle pointer");
   *out_handle = nullptr;
+  ellm_attn_desc local;
+  if (table) {
+    if (!table->seq_offsets || !table->seq_capacity || !table->seq_capacity_host)
+      return fail(ELLM_ERR_INVALID_ARGUMENT, "the sequence table has a null member");
+    if (d->batch_size == 0 || d->batch_size > table->sequences)
+      return fail(ELLM_ERR_OUT_OF_RANGE, "batch_size %zu, the sequence table has %zu entries", d->batch_size,
+                  table->sequences);
+    // sequence_capacity is the largest capacity among the operator's sequences; kv_strides[0]
+    // has no meaning (the table gives every sequence's offset) and only has to pass the checks
+    local = *d;
+    size_t cap = 0;
+    for (size_t i = 0; i < d->batch_size; ++i) {
+      if (table->seq_capacity_host[i] == 0)
+        return fail(ELLM_ERR_INVALID_ARGUMENT, "sequence %zu of the table has capacity 0", i);
+      cap = table->seq_capacity_host[i] > cap ? table->seq_capacity_host[i] : cap;
+    }
+    local.sequence_capacity = cap;
+    if (local.kv_strides[0] == 0) local.kv_strides[0] = 8;
+    d = &local;
+  }
   if (int st = ellm::validate_attn_desc(d)) return st;
 
   int device = 0, n_cu = 0;
@@ -207,6 +264,13 @@ int ellm_attn_create(const ellm_attn_desc* d, ellm_attn** out_handle) {
   h->desc = *d;
   h->device = device;
   h->n_cu = n_cu;
+  h->seq_offsets = nullptr;
+  h->seq_caps = nullptr;
+  if (table) {
+    h->seq_offsets = table->seq_offsets;
+    h->seq_caps = table->seq_capacity;
+    h->caps_host.assign(table->seq_capacity_host, table->seq_capacity_host + d->batch_size);
+  }
   h->ws = ellm::decode_workspace((uint32_t)d->batch_size, (uint32_t)d->attention_head_num,
                                  (uint32_t)d->kv_head_num, (uint32_t)n_cu);
   h->ws_acc = h->ws_ml = h->ws2_acc = h->ws2_ml = h->part_o = h->part_ml = nullptr;
@@ -231,6 +295,16 @@ int ellm_attn_create(const ellm_attn_desc* d, ellm_attn** out_handle) {
   return ELLM_OK;
 }
 
+int ellm_attn_create(const ellm_attn_desc* d, ellm_attn** out_handle) {
+  return attn_create(d, nullptr, out_handle);
+}
+
+int ellm_attn_create_ragged(const ellm_attn_desc* d, const ellm_kv_seq_table* table,
+                            ellm_attn** out_handle) {
+  if (!table) return fail(ELLM_ERR_INVALID_ARGUMENT, "null sequence table");
+  return attn_create(d, table, out_handle);
+}
+
 int ellm_attn_destroy(ellm_attn* h) {
   if (!h) return ELLM_OK;
   hipError_t e = free_workspace(h);
@@ -250,6 +324,8 @@ static void fill_args(const ellm_attn* h, ellm::AttnArgs* a) {
   a->prefill_part_ml = h->part_ml;
   a->prefill_part_rows = h->part_rows;
   a->n_cu = (uint32_t)h->n_cu;
+  a->seq_offsets = h->seq_offsets;
+  a->seq_caps = h->seq_caps;
 }
 
 static int run_decode(ellm_attn* h, ellm::AttnArgs* a, uint32_t max_position, hipStream_t stream) {
@@ -281,6 +357,10 @@ int ellm_attn_run(ellm_attn* h, size_t position_index, size_t position_interval,
     return fail(ELLM_ERR_OUT_OF_RANGE,
                 "positions [%zu, %zu) do not fit the sequence capacity %zu", position_index,
                 position_index + position_interval, d.sequence_capacity);
+  for (size_t i = 0; i < batch_size && i < h->caps_host.size(); ++i)
+    if (position_index + position_interval > h->caps_host[i])
+      return fail(ELLM_ERR_OUT_OF_RANGE, "positions [%zu, %zu) do not fit sequence %zu, whose capacity is %zu",
+                  position_index, position_index + position_interval, i, h->caps_host[i]);
   ellm::AttnArgs a;
   fill_args(h, &a);
   a.position_index = (uint32_t)position_index;
@@ -316,23 +396,32 @@ int ellm_attn_run_ragged(ellm_attn* h, const uint32_t* positions, size_t max_pos
 
 /* ---- K/V cache ---------------------------------------------------------- */
 
-int ellm_kv_create(const ellm_kv_desc* d, ellm_kv_cache** out_cache) {
-  if (!d || !out_cache) return fail(ELLM_ERR_INVALID_ARGUMENT, "null descriptor or cache pointer");
-  *out_cache = nullptr;
-  if (d->dtype != ELLM_DTYPE_F16 && d->dtype != ELLM_DTYPE_BF16)
-    return fail(ELLM_ERR_INVALID_ARGUMENT, "dtype %d is neither ELLM_DTYPE_F16 nor ELLM_DTYPE_BF16",
-                d->dtype);
-  if (d->head_size != 128)
-    return fail(ELLM_ERR_UNSUPPORTED, "head_size %zu: only 128 is supported", d->head_size);
-  if (d->layers == 0 || d->sequences == 0 || d->kv_head_num == 0 || d->capacity == 0)
+// Shared by the two create functions: caps = positions per plane of every sequence;
+// uniform -> [sequence][kv_head][position][128] with one capacity, else
+// [kv_head][sequence: its own positions][128] with offset / capacity tables on the device.
+static int kv_create(size_t layers, size_t kv_head_num, size_t head_size, int dtype,
+                     const std::vector<size_t>& caps, bool ragged, ellm_kv_cache** out_cache) {
+  if (dtype != ELLM_DTYPE_F16 && dtype != ELLM_DTYPE_BF16)
+    return fail(ELLM_ERR_INVALID_ARGUMENT, "dtype %d is neither ELLM_DTYPE_F16 nor ELLM_DTYPE_BF16", dtype);
+  if (head_size != 128)
+    return fail(ELLM_ERR_UNSUPPORTED, "head_size %zu: only 128 is supported", head_size);
+  const size_t sequences = caps.size();
+  if (layers == 0 || sequences == 0 || kv_head_num == 0)
     return fail(ELLM_ERR_INVALID_ARGUMENT, "layers, sequences, kv_head_num and capacity must be > 0");
-  if (d->capacity > 0x7fffffffu || d->sequences > 65535 || d->kv_head_num > 65535)
+  if (sequences > 65535 || kv_head_num > 65535)
     return fail(ELLM_ERR_UNSUPPORTED, "capacity / sequences / kv_head_num too large");
-  // capacity, sequences and kv_head_num are bounded above; layers is not
-  size_t layer_elems = d->sequences * d->kv_head_num;
+  size_t total = 0, largest = 0;   // positions of all sequences of one head
+  for (size_t cap : caps) {
+    if (cap == 0) return fail(ELLM_ERR_INVALID_ARGUMENT, "layers, sequences, kv_head_num and capacity must be > 0");
+    if (cap > 0x7fffffffu / 128) return fail(ELLM_ERR_UNSUPPORTED, "capacity / sequences / kv_head_num too large");
+    total += cap;   // at most 65535 x 2^24
+    largest = cap > largest ? cap : largest;
+  }
+  // sequences, capacities and kv_head_num are bounded above; layers is not
+  size_t layer_elems = total * head_size;
   size_t bytes = 0;
-  if (__builtin_mul_overflow(layer_elems, d->capacity * d->head_size, &layer_elems) ||
-      __builtin_mul_overflow(layer_elems, d->layers, &bytes) ||
+  if (__builtin_mul_overflow(layer_elems, kv_head_num, &layer_elems) ||
+      __builtin_mul_overflow(layer_elems, layers, &bytes) ||
       __builtin_mul_overflow(bytes, (size_t)2, &bytes))
     return fail(ELLM_ERR_UNSUPPORTED, "the cache's size in bytes does not fit 64 bits");
   int device = 0, n_cu = 0;
@@ -342,17 +431,46 @@ int ellm_kv_create(const ellm_kv_desc* d, ellm_kv_cache** out_cache) {
 
   ellm_kv_cache* c = new (std::nothrow) ellm_kv_cache;
   if (!c) return fail(ELLM_ERR_HIP, "out of host memory");
-  c->desc = *d;
+  c->desc = ellm_kv_desc{layers, sequences, kv_head_num, head_size, largest, dtype};
   c->device = device;
   c->layer_elems = layer_elems;
+  c->ragged = ragged;
+  c->caps_host = caps;
+  c->offsets_host.resize(sequences);
   c->k = c->v = nullptr;
+  c->seq_offsets_dev = nullptr;
+  c->seq_caps_dev = nullptr;
+  if (ragged) {
+    c->stride_seq = 0;
+    c->stride_head = total * head_size;
+    size_t at = 0;
+    for (size_t i = 0; i < sequences; ++i) {
+      c->offsets_host[i] = at * head_size;
+      at += caps[i];
+    }
+  } else {
+    c->stride_seq = kv_head_num * largest * head_size;
+    c->stride_head = largest * head_size;
+    for (size_t i = 0; i < sequences; ++i) c->offsets_host[i] = i * c->stride_seq;
+  }
   hipError_t e = hipMalloc(&c->k, bytes);
   if (e == hipSuccess) e = hipMalloc(&c->v, bytes);
   if (e == hipSuccess) e = hipMemset(c->k, 0, bytes);
   if (e == hipSuccess) e = hipMemset(c->v, 0, bytes);
+  if (e == hipSuccess && ragged) {
+    std::vector<uint32_t> caps32(caps.begin(), caps.end());
+    e = hipMalloc((void**)&c->seq_offsets_dev, sequences * sizeof(size_t));
+    if (e == hipSuccess) e = hipMalloc((void**)&c->seq_caps_dev, sequences * sizeof(uint32_t));
+    if (e == hipSuccess)
+      e = hipMemcpy(c->seq_offsets_dev, c->offsets_host.data(), sequences * sizeof(size_t), hipMemcpyHostToDevice);
+    if (e == hipSuccess)
+      e = hipMemcpy(c->seq_caps_dev, caps32.data(), sequences * sizeof(uint32_t), hipMemcpyHostToDevice);
+  }
   if (e != hipSuccess) {
     if (c->k) (void)hipFree(c->k);
     if (c->v) (void)hipFree(c->v);
+    if (c->seq_offsets_dev) (void)hipFree(c->seq_offsets_dev);
+    if (c->seq_caps_dev) (void)hipFree(c->seq_caps_dev);
     delete c;
     return fail_hip(e, "K/V cache allocation");
   }
@@ -360,10 +478,39 @@ int ellm_kv_create(const ellm_kv_desc* d, ellm_kv_cache** out_cache) {
   return ELLM_OK;
 }
 
+int ellm_kv_create(const ellm_kv_desc* d, ellm_kv_cache** out_cache) {
+  if (!d || !out_cache) return fail(ELLM_ERR_INVALID_ARGUMENT, "null descriptor or cache pointer");
+  *out_cache = nullptr;
+  if (d->sequences > 65535) return fail(ELLM_ERR_UNSUPPORTED, "capacity / sequences / kv_head_num too large");
+  if (d->capacity > 0x7fffffffu) return fail(ELLM_ERR_UNSUPPORTED, "capacity / sequences / kv_head_num too large");
+  // (a size that cannot be allocated must be refused before the per-sequence vectors are built)
+  size_t probe = 0;
+  if (__builtin_mul_overflow(d->sequences * (d->kv_head_num > 65535 ? 65535 : d->kv_head_num),
+                             d->capacity * 128, &probe) ||
+      __builtin_mul_overflow(probe, d->layers, &probe) || __builtin_mul_overflow(probe, (size_t)2, &probe))
+    return fail(ELLM_ERR_UNSUPPORTED, "the cache's size in bytes does not fit 64 bits");
+  if (d->head_size != 128)
+    return fail(ELLM_ERR_UNSUPPORTED, "head_size %zu: only 128 is supported", d->head_size);
+  const std::vector<size_t> caps(d->sequences, d->capacity);
+  return kv_create(d->layers, d->kv_head_num, d->head_size, d->dtype, caps, false, out_cache);
+}
+
+int ellm_kv_create_ragged(const ellm_kv_ragged_desc* d, ellm_kv_cache** out_cache) {
+  if (!d || !out_cache) return fail(ELLM_ERR_INVALID_ARGUMENT, "null descriptor or cache pointer");
+  *out_cache = nullptr;
+  if (!d->capacities) return fail(ELLM_ERR_INVALID_ARGUMENT, "null capacities");
+  if (d->sequences == 0 || d->sequences > 65535)
+    return fail(d->sequences ? ELLM_ERR_UNSUPPORTED : ELLM_ERR_INVALID_ARGUMENT, "sequences %zu out of range", d->sequences);
+  const std::vector<size_t> caps(d->capacities, d->capacities + d->sequences);
+  return kv_create(d->layers, d->kv_head_num, d->head_size, d->dtype, caps, true, out_cache);
+}
+
 int ellm_kv_destroy(ellm_kv_cache* c) {
   if (!c) return ELLM_OK;
   hipError_t e1 = hipFree(c->k);
   hipError_t e2 = hipFree(c->v);
+  if (c->seq_offsets_dev) (void)hipFree(c->seq_offsets_dev);
+  if (c->seq_caps_dev) (void)hipFree(c->seq_caps_dev);
   delete c;
   if (e1 != hipSuccess) return fail_hip(e1, "hipFree");
   if (e2 != hipSuccess) return fail_hip(e2, "hipFree");
@@ -372,14 +519,39 @@ int ellm_kv_destroy(ellm_kv_cache* c) {
 
 int ellm_kv_layer(const ellm_kv_cache* c, size_t layer, void** k, void** v, size_t kv_strides[4]) {
   if (!c || !k || !v || !kv_strides) return fail(ELLM_ERR_INVALID_ARGUMENT, "null argument");
+  if (c->ragged)
+    return fail(ELLM_ERR_INVALID_ARGUMENT,
+                "this cache has per-sequence capacities: no single sequence stride exists, use ellm_kv_layer_ragged");
   if (layer >= c->desc.layers)
     return fail(ELLM_ERR_OUT_OF_RANGE, "layer %zu of %zu", layer, c->desc.layers);
   *k = (char*)c->k + layer * c->layer_elems * 2;
   *v = (char*)c->v + layer * c->layer_elems * 2;
-  kv_strides[0] = c->desc.kv_head_num * c->desc.capacity * c->desc.head_size;
-  kv_strides[1] = c->desc.capacity * c->desc.head_size;
+  kv_strides[0] = c->stride_seq;
+  kv_strides[1] = c->stride_head;
   kv_strides[2] = c->desc.head_size;
   kv_strides[3] = 1;
+  return ELLM_OK;
+}
+
+int ellm_kv_layer_ragged(const ellm_kv_cache* c, size_t layer, size_t first_sequence, void** k, void** v,
+                         size_t kv_strides[4], ellm_kv_seq_table* table) {
+  if (!c || !k || !v || !kv_strides || !table) return fail(ELLM_ERR_INVALID_ARGUMENT, "null argument");
+  if (!c->ragged)
+    return fail(ELLM_ERR_INVALID_ARGUMENT, "this cache has one capacity for every sequence: use ellm_kv_layer");
+  if (layer >= c->desc.layers)
+    return fail(ELLM_ERR_OUT_OF_RANGE, "layer %zu of %zu", layer, c->desc.layers);
+  if (first_sequence >= c->desc.sequences)
+    return fail(ELLM_ERR_OUT_OF_RANGE, "first_sequence %zu of %zu", first_sequence, c->desc.sequences);
+  *k = (char*)c->k + layer * c->layer_elems * 2;
+  *v = (char*)c->v + layer * c->layer_elems * 2;
+  kv_strides[0] = c->layer_elems;   // not used with a table (every sequence has its own offset)
+  kv_strides[1] = c->stride_head;
+  kv_strides[2] = c->desc.head_size;
+  kv_strides[3] = 1;
+  table->seq_offsets = c->seq_offsets_dev + first_sequence;
+  table->seq_capacity = c->seq_caps_dev + first_sequence;
+  table->seq_capacity_host = c->caps_host.data() + first_sequence;
+  table->sequences = c->desc.sequences - first_sequence;
   return ELLM_OK;
 }
 
@@ -397,17 +569,17 @@ int ellm_kv_append(ellm_kv_cache* c, size_t layer, size_t position_index, size_t
   if (batch_size > c->desc.sequences || src_batch_pitch < batch_size)
     return fail(ELLM_ERR_OUT_OF_RANGE, "batch_size %zu exceeds the cache's %zu sequences or the source pitch %zu",
                 batch_size, c->desc.sequences, src_batch_pitch);
-  if (position_index >= c->desc.capacity || n_tokens > c->desc.capacity - position_index)
+  const size_t room = c->min_cap(batch_size);   // the shortest of the sequences written
+  if (position_index >= room || n_tokens > room - position_index)
     return fail(ELLM_ERR_OUT_OF_RANGE, "positions [%zu, %zu) do not fit the capacity %zu",
-                position_index, position_index + n_tokens, c->desc.capacity);
+                position_index, position_index + n_tokens, room);
   if (n_tokens > 0xffffffffu / 2 || src_batch_pitch > 65535)
     return fail(ELLM_ERR_UNSUPPORTED, "n_tokens or src_batch_pitch too large");
   void* k = (char*)c->k + layer * c->layer_elems * 2;
   void* v = (char*)c->v + layer * c->layer_elems * 2;
   hipError_t e = ellm::launch_kv_append(k, v, k_src, v_src, (uint32_t)n_tokens, (uint32_t)batch_size,
                                         (uint32_t)src_batch_pitch, (uint32_t)c->desc.kv_head_num,
-                                        (uint32_t)c->desc.capacity, (uint32_t)position_index,
-                                        (hipStream_t)stream);
+                                        c->layout(), (uint32_t)position_index, (hipStream_t)stream);
   if (e != hipSuccess) return fail_hip(e, "kv append launch");
   return ELLM_OK;
 }
@@ -430,10 +602,12 @@ int ellm_kv_append_norm_rope(ellm_kv_cache* c, size_t layer, size_t position_ind
     return fail(ELLM_ERR_OUT_OF_RANGE, "batch_size %zu exceeds the cache's %zu sequences or the source pitch %zu",
                 batch_size, c->desc.sequences, src_batch_pitch);
   // with per-sequence positions the highest start is max_position (entries above it are clamped)
+  // (a cache with per-sequence capacities also bounds each sequence's rows on the device)
   const size_t first = positions ? max_position : position_index;
-  if (first >= c->desc.capacity || n_tokens > c->desc.capacity - first)
+  const size_t room = positions ? c->max_cap(batch_size) : c->min_cap(batch_size);
+  if (first >= room || n_tokens > room - first)
     return fail(ELLM_ERR_OUT_OF_RANGE, "positions [%zu, %zu) do not fit the capacity %zu", first,
-                first + n_tokens, c->desc.capacity);
+                first + n_tokens, room);
   if (first + n_tokens > rope_positions)
     return fail(ELLM_ERR_OUT_OF_RANGE, "positions [%zu, %zu) are beyond the %zu rows of the rotary table",
                 first, first + n_tokens, rope_positions);
@@ -443,7 +617,7 @@ int ellm_kv_append_norm_rope(ellm_kv_cache* c, size_t layer, size_t position_ind
   void* v = (char*)c->v + layer * c->layer_elems * 2;
   hipError_t e = ellm::launch_kv_append_norm_rope(
       k, v, k_src, v_src, rope, positions, (uint32_t)n_tokens, (uint32_t)batch_size,
-      (uint32_t)src_batch_pitch, (uint32_t)c->desc.kv_head_num, (uint32_t)c->desc.capacity,
+      (uint32_t)src_batch_pitch, (uint32_t)c->desc.kv_head_num, c->layout(),
       (uint32_t)position_index, (uint32_t)max_position, eps, c->desc.dtype, (hipStream_t)stream);
   if (e != hipSuccess) return fail_hip(e, "kv append (norm + rope) launch");
   return ELLM_OK;

@@ -142,6 +142,12 @@ __device__ __forceinline__ u32x2 gather_column(uint32_t r0, uint32_t r1, uint32_
   return o;
 }
 
+// Element offset of the first K/V plane of a sequence: sequence x stride, or, for a cache
+// whose sequences have different capacities, the sequence's entry of an offset table.
+__device__ __forceinline__ size_t seq_plane_offset(const size_t* table, size_t stride, uint32_t seq) {
+  return table ? table[seq] : (size_t)seq * stride;
+}
+
 constexpr float kLog2e = 1.4426950408889634f;
 constexpr float kLn2 = 0.6931471805599453f;
 

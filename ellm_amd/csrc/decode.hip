@@ -44,6 +44,8 @@ struct DecodeKernelArgs {
   uint16_t* out;
   float* lse;
   const uint32_t* positions;
+  const size_t* seq_offsets;   // per-sequence plane offsets (null: sequence x kv_stride_seq)
+  const uint32_t* seq_caps;    // per-sequence capacities (null: none to clamp to)
   float* ws_acc;
   float* ws_ml;
   float* ws2_acc;      // cluster partials [sequence][query head][n_cluster_max][128]
@@ -125,6 +127,7 @@ __global__ __launch_bounds__(kDecWaves* kWave, 4) void decode_split_kernel(
 
   uint32_t pos = p.position;
   if (p.positions) pos = min(p.positions[seq], p.position);
+  if (p.seq_caps) pos = min(pos, p.seq_caps[seq] - 1);
   const uint32_t len = pos + 1;
   const uint32_t k_begin = split * p.split_len;
   const uint32_t k_end = min(len, k_begin + p.split_len);
@@ -133,8 +136,9 @@ __global__ __launch_bounds__(kDecWaves* kWave, 4) void decode_split_kernel(
   // not counted: the merge below derives the live split count from the length.
   if (k_begin >= len) return;
 
-  const uint16_t* kplane = p.k + seq * p.kv_stride_seq + kvh * p.kv_stride_head;
-  const uint16_t* vplane = p.v + seq * p.kv_stride_seq + kvh * p.kv_stride_head;
+  const size_t plane = seq_plane_offset(p.seq_offsets, p.kv_stride_seq, seq) + kvh * p.kv_stride_head;
+  const uint16_t* kplane = p.k + plane;
+  const uint16_t* vplane = p.v + plane;
 
   // Query heads of this group as the B operand of S^T = K.Q^T:
   // lane (head c, group g) holds q[head][32 s + 8 g + 0..7] for s = 0..3.
@@ -464,6 +468,8 @@ hipError_t launch_decode(const AttnArgs& a, hipStream_t stream) {
   p.out = (uint16_t*)a.out;
   p.lse = a.lse;
   p.positions = a.positions;
+  p.seq_offsets = a.seq_offsets;
+  p.seq_caps = a.seq_caps;
   p.ws_acc = a.ws_acc;
   p.ws_ml = a.ws_ml;
   p.ws2_acc = a.ws2_acc;

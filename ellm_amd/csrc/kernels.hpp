@@ -31,6 +31,10 @@ struct AttnArgs {
   uint32_t position_interval;
   uint32_t batch;
   const uint32_t* positions;  // device, per sequence; null = position_index for all
+  // caches whose sequences differ in capacity (both null otherwise): per-sequence element
+  // offset of the first plane (replaces sequence x kv_stride_seq) and positions per plane
+  const size_t* seq_offsets;
+  const uint32_t* seq_caps;
   // single-token path workspace
   float* ws_acc;  // [sequence][query head][split][128]
   float* ws_ml;   // [sequence][query head][split][2]  (max in log2 units, sum)
@@ -73,9 +77,17 @@ bool decode_plan_fits(const DecodeWorkspace& w, uint32_t batch, uint32_t n_q_hea
 hipError_t launch_decode(const AttnArgs& a, hipStream_t stream);
 hipError_t launch_prefill(const AttnArgs& a, hipStream_t stream);
 
+// Where the rows of a cache layer live: plane of (sequence, head) at
+// seq_plane_offset(seq_offsets, stride_seq, sequence) + head x stride_head, rows 128 apart;
+// seq_caps (may be null) bounds the positions written per sequence on the device.
+struct KvLayout {
+  size_t stride_seq, stride_head;
+  const size_t* seq_offsets;
+  const uint32_t* seq_caps;
+};
 hipError_t launch_kv_append(void* k_dst, void* v_dst, const void* k_src, const void* v_src,
                             uint32_t n_tokens, uint32_t batch, uint32_t src_batch_pitch,
-                            uint32_t n_kv_heads, uint32_t capacity, uint32_t position_index,
+                            uint32_t n_kv_heads, const KvLayout& layout, uint32_t position_index,
                             hipStream_t stream);
 
 // Same, with RMS norm and rotary rotation of the key rows; rope: [positions][128] of
@@ -85,7 +97,7 @@ hipError_t launch_kv_append_norm_rope(void* k_dst, void* v_dst, const void* k_sr
                                       const void* v_src, const void* rope,
                                       const uint32_t* positions, uint32_t n_tokens, uint32_t batch,
                                       uint32_t src_batch_pitch, uint32_t n_kv_heads,
-                                      uint32_t capacity, uint32_t position_index,
+                                      const KvLayout& layout, uint32_t position_index,
                                       uint32_t max_start, float eps, int dtype,
                                       hipStream_t stream);
 
@@ -109,6 +121,8 @@ struct ProjectArgs {
   void* v_out;
   const void* rope;
   const uint32_t* positions;
+  const size_t* seq_offsets;   // as in AttnArgs (null: sequence x kv_stride_seq)
+  const uint32_t* seq_caps;
   size_t kv_stride_seq, kv_stride_head, kv_stride_pos;
   uint32_t rope_pos_stride, rope_head_stride;
   uint32_t K, rows, batch_pitch, batch, heads0, heads_kv;

@@ -12,7 +12,7 @@ namespace {
 __global__ __launch_bounds__(256) void kv_append_kernel(
     uint16_t* __restrict__ k_dst, uint16_t* __restrict__ v_dst, const uint16_t* __restrict__ k_src,
     const uint16_t* __restrict__ v_src, uint32_t n_tokens, uint32_t batch, uint32_t src_batch_pitch,
-    uint32_t n_kv_heads, uint32_t capacity, uint32_t position_index) {
+    uint32_t n_kv_heads, KvLayout layout, uint32_t position_index) {
   // one thread per 16-byte chunk; 16 chunks per 128-element row
   const size_t total = (size_t)n_tokens * batch * n_kv_heads * 16;
   for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total;
@@ -24,8 +24,8 @@ __global__ __launch_bounds__(256) void kv_append_kernel(
     const uint32_t b = r % batch;
     const uint32_t t = r / batch;
     const size_t src = (((size_t)t * src_batch_pitch + b) * n_kv_heads + h) * kHeadDim + 8 * c;
-    const size_t dst =
-        (((size_t)b * n_kv_heads + h) * capacity + position_index + t) * kHeadDim + 8 * c;
+    const size_t dst = seq_plane_offset(layout.seq_offsets, layout.stride_seq, b) +
+                       (size_t)h * layout.stride_head + (size_t)(position_index + t) * kHeadDim + 8 * c;
     store16(k_dst + dst, load16(k_src + src));
     store16(v_dst + dst, load16(v_src + src));
   }
@@ -50,7 +50,7 @@ __global__ __launch_bounds__(256) void kv_append_norm_rope_kernel(
     uint16_t* __restrict__ k_dst, uint16_t* __restrict__ v_dst, const uint16_t* __restrict__ k_src,
     const uint16_t* __restrict__ v_src, const uint16_t* __restrict__ rope,
     const uint32_t* __restrict__ positions, uint32_t n_tokens, uint32_t batch,
-    uint32_t src_batch_pitch, uint32_t n_kv_heads, uint32_t capacity, uint32_t position_index,
+    uint32_t src_batch_pitch, uint32_t n_kv_heads, KvLayout layout, uint32_t position_index,
     uint32_t max_start, float eps) {
 #pragma clang fp contract(off)
   const uint32_t c = threadIdx.x & 15;
@@ -69,7 +69,11 @@ __global__ __launch_bounds__(256) void kv_append_norm_rope_kernel(
     const uint32_t start = positions ? min(positions[b], max_start) : position_index;
     const uint32_t pos = start + t;
     const size_t src = (((size_t)t * src_batch_pitch + b) * n_kv_heads + h) * kHeadDim + 8 * c;
-    const size_t dst = (((size_t)b * n_kv_heads + h) * capacity + pos) * kHeadDim + 8 * c;
+    // (per-sequence capacities, where the cache has them, bound the row written: a start
+    // position beyond a short sequence's planes must not reach into its neighbour's)
+    const uint32_t pos_dst = layout.seq_caps ? min(pos, layout.seq_caps[b] - 1) : pos;
+    const size_t dst = seq_plane_offset(layout.seq_offsets, layout.stride_seq, b) +
+                       (size_t)h * layout.stride_head + (size_t)pos_dst * kHeadDim + 8 * c;
     const u32x4 kraw = load16(k_src + src);
     const u32x4 vraw = load16(v_src + src);
     const u32x4 rraw = load16(rope + (size_t)pos * kHeadDim + 8 * c);
@@ -127,7 +131,7 @@ hipError_t launch_kv_append_norm_rope(void* k_dst, void* v_dst, const void* k_sr
                                       const void* v_src, const void* rope,
                                       const uint32_t* positions, uint32_t n_tokens, uint32_t batch,
                                       uint32_t src_batch_pitch, uint32_t n_kv_heads,
-                                      uint32_t capacity, uint32_t position_index,
+                                      const KvLayout& layout, uint32_t position_index,
                                       uint32_t max_start, float eps, int dtype,
                                       hipStream_t stream) {
   const size_t rows = (size_t)n_tokens * batch * n_kv_heads;
@@ -138,7 +142,7 @@ hipError_t launch_kv_append_norm_rope(void* k_dst, void* v_dst, const void* k_sr
     hipLaunchKernelGGL(kernel, dim3((uint32_t)blocks), dim3(256), 0, stream, (uint16_t*)k_dst,
                        (uint16_t*)v_dst, (const uint16_t*)k_src, (const uint16_t*)v_src,
                        (const uint16_t*)rope, positions, n_tokens, batch, src_batch_pitch,
-                       n_kv_heads, capacity, position_index, max_start, eps);
+                       n_kv_heads, layout, position_index, max_start, eps);
   };
   if (dtype == 0)
     go(kv_append_norm_rope_kernel<Mfma<F16>>);
@@ -149,7 +153,7 @@ hipError_t launch_kv_append_norm_rope(void* k_dst, void* v_dst, const void* k_sr
 
 hipError_t launch_kv_append(void* k_dst, void* v_dst, const void* k_src, const void* v_src,
                             uint32_t n_tokens, uint32_t batch, uint32_t src_batch_pitch,
-                            uint32_t n_kv_heads, uint32_t capacity, uint32_t position_index,
+                            uint32_t n_kv_heads, const KvLayout& layout, uint32_t position_index,
                             hipStream_t stream) {
   const size_t total = (size_t)n_tokens * batch * n_kv_heads * 16;
   if (total == 0) return hipSuccess;
@@ -157,7 +161,7 @@ hipError_t launch_kv_append(void* k_dst, void* v_dst, const void* k_src, const v
   if (blocks > 65536) blocks = 65536;
   hipLaunchKernelGGL(kv_append_kernel, dim3((uint32_t)blocks), dim3(256), 0, stream,
                      (uint16_t*)k_dst, (uint16_t*)v_dst, (const uint16_t*)k_src,
-                     (const uint16_t*)v_src, n_tokens, batch, src_batch_pitch, n_kv_heads, capacity,
+                     (const uint16_t*)v_src, n_tokens, batch, src_batch_pitch, n_kv_heads, layout,
                      position_index);
   return hipGetLastError();
 }

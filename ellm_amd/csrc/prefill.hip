@@ -41,6 +41,7 @@ struct PrefillKernelArgs {
   float* lse;
   size_t q_token_stride;  // elements between consecutive tokens of Q/O
   size_t kv_stride_seq, kv_stride_head, kv_stride_pos;
+  const size_t* seq_offsets;  // per-sequence plane offsets (null: sequence x kv_stride_seq)
   uint32_t batch_pitch;
   uint32_t n_q_heads, n_kv_heads, group;
   uint32_t heads_per_wg;     // query heads stacked in one workgroup
@@ -145,8 +146,9 @@ __global__ __launch_bounds__(kPpThreads, 2) void prefill_pingpong_kernel(Prefill
   }
   const float c = p.c;
 
-  const uint16_t* kplane = p.k + seq * p.kv_stride_seq + kvh * p.kv_stride_head;
-  const uint16_t* vplane = p.v + seq * p.kv_stride_seq + kvh * p.kv_stride_head;
+  const size_t plane_at = seq_plane_offset(p.seq_offsets, p.kv_stride_seq, seq) + kvh * p.kv_stride_head;
+  const uint16_t* kplane = p.k + plane_at;
+  const uint16_t* vplane = p.v + plane_at;
 
   // staging: the 256 threads of a group move one 64 x 128 tile, four 16-byte pieces
   // each (rows ld_r + 16 i, columns 8 ld_c ..), K and V alike: V sits in LDS row by
@@ -504,6 +506,7 @@ hipError_t launch_pingpong(const AttnArgs& a, hipStream_t stream) {
   p.kv_stride_seq = a.kv_stride_seq;
   p.kv_stride_head = a.kv_stride_head;
   p.kv_stride_pos = a.kv_stride_pos;
+  p.seq_offsets = a.seq_offsets;
   p.batch_pitch = a.batch_pitch;
   p.n_q_heads = a.n_q_heads;
   p.n_kv_heads = a.n_kv_heads;

@@ -237,6 +237,8 @@ hipError_t launch_project(const ProjectArgs& a, hipStream_t stream) {
   p.v_out = (uint16_t*)a.v_out;
   p.rope = (const uint16_t*)a.rope;
   p.positions = a.positions;
+  p.seq_offsets = a.seq_offsets;
+  p.seq_caps = a.seq_caps;
   p.kv_stride_seq = a.kv_stride_seq;
   p.kv_stride_head = a.kv_stride_head;
   p.kv_stride_pos = a.kv_stride_pos;

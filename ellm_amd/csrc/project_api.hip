@@ -5,6 +5,7 @@
 
 #include <cmath>
 #include <new>
+#include <vector>
 
 #include "../../include/ellm_attn.h"
 #include "kernels.hpp"
@@ -19,6 +20,10 @@ struct ellm_matmul3 {
   int device;
   float* ws;
   uint32_t* counters;
+  // destination with per-sequence capacities (ellm_matmul3_create_ragged); null / empty otherwise
+  const size_t* seq_offsets;
+  const uint32_t* seq_caps;
+  std::vector<size_t> caps_host;
 };
 struct ellm_matmul_add {
   ellm_matmul_add_desc d;
@@ -61,9 +66,24 @@ int free_small_workspace(float* ws, uint32_t* counters) {
 
 extern "C" {
 
-int ellm_matmul3_create(const ellm_matmul3_desc* d, ellm_matmul3** out_handle) {
+static int matmul3_create(const ellm_matmul3_desc* d, const ellm_kv_seq_table* table,
+                          ellm_matmul3** out_handle) {
   if (!d || !out_handle) return ellm::set_error(ELLM_ERR_INVALID_ARGUMENT, "null descriptor or handle pointer");
   *out_handle = nullptr;
+  ellm_matmul3_desc local;
+  if (table) {
+    if (!table->seq_offsets || !table->seq_capacity || !table->seq_capacity_host)
+      return ellm::set_error(ELLM_ERR_INVALID_ARGUMENT, "the sequence table has a null member");
+    if (d->batch_size == 0 || d->batch_size > table->sequences)
+      return ellm::set_error(ELLM_ERR_OUT_OF_RANGE, "batch_size %zu, the sequence table has %zu entries",
+                             d->batch_size, table->sequences);
+    local = *d;
+    size_t cap = 0;
+    for (size_t i = 0; i < d->batch_size; ++i)
+      cap = table->seq_capacity_host[i] > cap ? table->seq_capacity_host[i] : cap;
+    local.sequence_capacity = cap;   // the largest: per-sequence checks follow at run time
+    d = &local;
+  }
   const void* ptrs[] = {d->hidden, d->q_weight, d->k_weight, d->v_weight, d->q_state,
                         d->k_state, d->v_state, d->rope};
   for (const void* p : ptrs) {
@@ -97,6 +117,13 @@ int ellm_matmul3_create(const ellm_matmul3_desc* d, ellm_matmul3** out_handle) {
   ellm_matmul3* h = new (std::nothrow) ellm_matmul3;
   if (!h) return ellm::set_error(ELLM_ERR_HIP, "out of host memory");
   h->d = *d;
+  h->seq_offsets = nullptr;
+  h->seq_caps = nullptr;
+  if (table) {
+    h->seq_offsets = table->seq_offsets;
+    h->seq_caps = table->seq_capacity;
+    h->caps_host.assign(table->seq_capacity_host, table->seq_capacity_host + d->batch_size);
+  }
   const int rc = alloc_small_workspace((uint32_t)(d->attention_head_num + 2 * d->kv_head_num),
                                        (uint32_t)d->hidden_size, &h->device, &h->ws, &h->counters);
   if (rc != ELLM_OK) {
@@ -105,6 +132,16 @@ int ellm_matmul3_create(const ellm_matmul3_desc* d, ellm_matmul3** out_handle) {
   }
   *out_handle = h;
   return ELLM_OK;
+}
+
+int ellm_matmul3_create(const ellm_matmul3_desc* d, ellm_matmul3** out_handle) {
+  return matmul3_create(d, nullptr, out_handle);
+}
+
+int ellm_matmul3_create_ragged(const ellm_matmul3_desc* d, const ellm_kv_seq_table* table,
+                               ellm_matmul3** out_handle) {
+  if (!table) return ellm::set_error(ELLM_ERR_INVALID_ARGUMENT, "null sequence table");
+  return matmul3_create(d, table, out_handle);
 }
 
 int ellm_matmul3_destroy(ellm_matmul3* h) {
@@ -127,6 +164,10 @@ static int matmul3_launch(ellm_matmul3* h, size_t position_index, size_t positio
   const size_t last = (positions ? max_start : position_index) + position_interval - 1;
   if (last >= d.sequence_capacity)
     return ellm::set_error(ELLM_ERR_OUT_OF_RANGE, "position %zu is outside the cache (capacity %zu)", last, d.sequence_capacity);
+  if (!positions)   // one shared range: it must fit every sequence written (per-sequence starts are clamped on the device)
+    for (size_t i = 0; i < batch_size && i < h->caps_host.size(); ++i)
+      if (last >= h->caps_host[i])
+        return ellm::set_error(ELLM_ERR_OUT_OF_RANGE, "position %zu is outside sequence %zu (capacity %zu)", last, i, h->caps_host[i]);
   const size_t heads_max = d.attention_head_num > d.kv_head_num ? d.attention_head_num : d.kv_head_num;
   if (last * d.rope_position_stride + (heads_max - 1) * d.rope_head_stride + 128 > d.rope_elems)
     return ellm::set_error(ELLM_ERR_OUT_OF_RANGE, "position %zu is outside the rotary table (%zu elements)", last, d.rope_elems);
@@ -141,6 +182,8 @@ static int matmul3_launch(ellm_matmul3* h, size_t position_index, size_t positio
   a.v_out = d.v_state;
   a.rope = d.rope;
   a.positions = positions;
+  a.seq_offsets = h->seq_offsets;
+  a.seq_caps = h->seq_caps;
   a.kv_stride_seq = d.kv_strides[0];
   a.kv_stride_head = d.kv_strides[1];
   a.kv_stride_pos = d.kv_strides[2];

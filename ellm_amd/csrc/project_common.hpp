@@ -21,6 +21,8 @@ struct ProjectKernelArgs {
   uint16_t* v_out;
   const uint16_t* rope;
   const uint32_t* positions;
+  const size_t* seq_offsets;   // per-sequence plane offsets (null: sequence x kv_stride_seq)
+  const uint32_t* seq_caps;    // per-sequence capacities (null: none to clamp to)
   size_t kv_stride_seq, kv_stride_head, kv_stride_pos;  // elements
   uint32_t ld0;
   uint32_t rope_pos_stride, rope_head_stride;           // elements
@@ -31,6 +33,14 @@ struct ProjectKernelArgs {
   uint32_t finalize0;        // segment 0 rows are normalised and rotated
   float eps;
 };
+
+// Element offset of the K/V row of (sequence b, kv head hs, position pos) in k_out / v_out.
+__device__ __forceinline__ size_t kv_row_offset(const ProjectKernelArgs& p, uint32_t b, uint32_t hs,
+                                                uint32_t pos) {
+  if (p.seq_caps) pos = min(pos, p.seq_caps[b] - 1);
+  return seq_plane_offset(p.seq_offsets, p.kv_stride_seq, b) + (size_t)hs * p.kv_stride_head +
+         (size_t)pos * p.kv_stride_pos;
+}
 
 template <int N, typename F>
 __device__ __forceinline__ void static_for(F&& f) {

@@ -66,8 +66,7 @@ __device__ __forceinline__ HeadRows<MB> prepare_head(const ProjectKernelArgs& p,
     if (seg == 0)
       h.out_row[mb] = dst + (size_t)R * p.ld0 + col;
     else
-      h.out_row[mb] = dst + (size_t)b * p.kv_stride_seq + (size_t)hs * p.kv_stride_head +
-                      (size_t)pos * p.kv_stride_pos;
+      h.out_row[mb] = dst + (h.live[mb] ? kv_row_offset(p, b, hs, pos) : (size_t)0);
     if (MODE == kModeQkv)
       h.ext_row[mb] = p.rope + (size_t)pos * p.rope_pos_stride + (size_t)hs * p.rope_head_stride + 4 * g;
     else

@@ -115,8 +115,7 @@ __global__ __launch_bounds__((NTB == 2 || NB == 2) ? 512 : 1024) void project_sm
             off = (size_t)R * p.ld0 + hs * kHeadDim + kGroupCols * cg + 4 * c4;
           } else {
             const uint32_t pos = t + (p.positions ? min(p.positions[b], p.max_start) : p.position_index);
-            off = (size_t)b * p.kv_stride_seq + (size_t)hs * p.kv_stride_head +
-                  (size_t)pos * p.kv_stride_pos + kGroupCols * cg + 4 * c4;
+            off = kv_row_offset(p, b, hs, pos) + kGroupCols * cg + 4 * c4;
           }
           if (MODE == kModeAdd) {
             const u32x2 rs = *(const u32x2*)(p.residual + off);
@@ -257,7 +256,7 @@ __global__ __launch_bounds__((NTB == 2 || NB == 2) ? 512 : 1024) void project_sm
       if (seg == 0)
         off = (size_t)R * p.ld0 + hs * kHeadDim + 8 * c8;
       else
-        off = (size_t)b * p.kv_stride_seq + (size_t)hs * p.kv_stride_head + (size_t)pos * p.kv_stride_pos + 8 * c8;
+        off = kv_row_offset(p, b, hs, pos) + 8 * c8;
       const u32x4 packed = {M::pack2(o[0], o[1]), M::pack2(o[2], o[3]), M::pack2(o[4], o[5]), M::pack2(o[6], o[7])};
       store16(dst + off, packed);
     }

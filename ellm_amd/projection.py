@@ -22,15 +22,20 @@ class MatMul3:
     def __init__(self, hidden, q_weight, q_state, k_weight, k_state, v_weight, v_state, rope,
                  head_dim, batch_size, attention_head_num, kv_head_num, kv_strides,
                  sequence_capacity, rope_position_stride=128, rope_head_stride=0, eps=1e-6,
-                 max_position_interval=None):
+                 max_position_interval=None, seq_table=None):
+        """seq_table: a KVCache.layer_ragged(...) view when k_state / v_state are a cache layer
+        whose sequences have different capacities."""
         self._lib = load_library()
-        self._keep = (hidden, q_weight, q_state, k_weight, k_state, v_weight, v_state, rope)
+        self._keep = (hidden, q_weight, q_state, k_weight, k_state, v_weight, v_state, rope, seq_table)
         dt = hidden.dtype
         hidden_size = hidden.shape[-1]
         interval = int(max_position_interval if max_position_interval is not None else hidden.shape[0])
         rows = interval * batch_size
-        kv_span = ((batch_size - 1) * int(kv_strides[0]) + (kv_head_num - 1) * int(kv_strides[1])
-                   + (int(sequence_capacity) - 1) * int(kv_strides[2]) + head_dim)
+        if seq_table is not None:
+            kv_span = seq_table.span_elems(batch_size, kv_head_num, int(kv_strides[1]))
+        else:
+            kv_span = ((batch_size - 1) * int(kv_strides[0]) + (kv_head_num - 1) * int(kv_strides[1])
+                       + (int(sequence_capacity) - 1) * int(kv_strides[2]) + head_dim)
         d = MatMul3Desc()
         d.hidden = _device_buffer("hidden", hidden, rows * hidden_size)
         d.q_weight = _device_buffer("q_weight", q_weight, attention_head_num * head_dim * hidden_size, dt)
@@ -53,7 +58,11 @@ class MatMul3:
         d.dtype = _dtype_code(hidden)
         self.desc = d
         self._handle = ctypes.c_void_p()
-        check(self._lib.ellm_matmul3_create(ctypes.byref(d), ctypes.byref(self._handle)))
+        if seq_table is not None:
+            check(self._lib.ellm_matmul3_create_ragged(ctypes.byref(d), ctypes.byref(seq_table.table),
+                                                       ctypes.byref(self._handle)))
+        else:
+            check(self._lib.ellm_matmul3_create(ctypes.byref(d), ctypes.byref(self._handle)))
 
     @classmethod
     def new(cls, *args, **kwargs):

@@ -183,6 +183,56 @@ int ellm_kv_layer(const ellm_kv_cache* cache, size_t layer, void** k, void** v,
                   size_t kv_strides[4]);
 
 /*
+ * A cache whose sequences (slots) have different capacities: still static, non-paged and
+ * contiguous per (layer, kv head, sequence) plane, offsets computed once at creation.
+ * Layout [layer][kv_head][sequence: its own positions][128]: the plane of (sequence s,
+ * head h) starts at  layer base + 128 * (positions of the sequences before s) +
+ * h * kv_strides[1].  A mixed step over 33 sequences of 16384 ... 131072 positions x 48
+ * layers then takes what the sequences need (~220 GB) instead of 33 x 131072 positions a
+ * layer (425 GB).  Same concept as the uniform cache (static max-shape K/V addressed by
+ * coordinates, README.md:51-54; per-layer persistent buffers, src/memory/cache.rs:23,
+ * 69-75); the reference itself has one capacity for every sequence.
+ * ellm_kv_append / ellm_kv_append_norm_rope work on both kinds of cache (a call with one
+ * shared position range must fit the shortest of the sequences it writes).
+ */
+typedef struct ellm_kv_ragged_desc {
+  size_t layers;
+  size_t sequences;
+  size_t kv_head_num;
+  size_t head_size;         /* 128 */
+  const size_t* capacities; /* host, [sequences]: positions per plane of each sequence, > 0 */
+  int dtype;                /* ellm_dtype */
+} ellm_kv_ragged_desc;
+int ellm_kv_create_ragged(const ellm_kv_ragged_desc* desc, ellm_kv_cache** out_cache);
+
+/* Where the sequences [first_sequence, ...) of such a cache start and how many positions
+ * each holds: what the operators need beside the strides.  The arrays belong to the cache
+ * and live as long as it does. */
+typedef struct ellm_kv_seq_table {
+  const size_t* seq_offsets;        /* device: element offset of each sequence's first plane */
+  const uint32_t* seq_capacity;     /* device: positions per plane of each sequence */
+  const size_t* seq_capacity_host;  /* host copy of the capacities */
+  size_t sequences;                 /* entries in each array */
+} ellm_kv_seq_table;
+
+/* ellm_kv_layer for a cache with per-sequence capacities.  kv_strides[1..3] are the head,
+ * position and element strides; kv_strides[0] has no meaning (every sequence has its own
+ * offset in the table) and is only there to keep the four-stride shape.  Hand k, v,
+ * kv_strides and the table to ellm_attn_create_ragged / ellm_matmul3_create_ragged:
+ * their sequence i is the cache's sequence first_sequence + i. */
+int ellm_kv_layer_ragged(const ellm_kv_cache* cache, size_t layer, size_t first_sequence, void** k,
+                         void** v, size_t kv_strides[4], ellm_kv_seq_table* table);
+
+/* ellm_attn_create on such a layer: sequence i's planes start at k + seq_offsets[i] +
+ * head * kv_strides[1]; desc->kv_strides[0] and desc->sequence_capacity are ignored (the
+ * capacity is per sequence: a run with one shared position range must fit every sequence it
+ * covers, per-sequence positions are clamped to each sequence's own capacity on the
+ * device).  desc->batch_size may not exceed table->sequences.  run / run_ragged / destroy
+ * as for any handle. */
+int ellm_attn_create_ragged(const ellm_attn_desc* desc, const ellm_kv_seq_table* table,
+                            ellm_attn** out_handle);
+
+/*
  * Writes n_tokens new positions [position_index, position_index + n_tokens) of
  * sequences [0, batch_size) of one layer.  k_src / v_src: device,
  * [n_tokens][src_batch_pitch][kv_head_num][128] — the layout in which the
@@ -326,6 +376,11 @@ typedef struct ellm_matmul3_desc {
 } ellm_matmul3_desc;
 typedef struct ellm_matmul3 ellm_matmul3;
 int ellm_matmul3_create(const ellm_matmul3_desc* desc, ellm_matmul3** out_handle);
+/* The same on a cache layer with per-sequence capacities (ellm_kv_layer_ragged): key and value
+ * rows of sequence i go to state + seq_offsets[i] + head * kv_strides[1] + position *
+ * kv_strides[2]; desc->kv_strides[0] and desc->sequence_capacity are ignored. */
+int ellm_matmul3_create_ragged(const ellm_matmul3_desc* desc, const ellm_kv_seq_table* table,
+                               ellm_matmul3** out_handle);
 /* MatMul3::run(position_index, position_interval, batch_size, cpu_num, thread_id) */
 int ellm_matmul3_run(ellm_matmul3* handle, size_t position_index, size_t position_interval,
                      size_t batch_size, void* stream);

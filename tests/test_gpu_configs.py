@@ -273,3 +273,128 @@ def test_config4_mixed_step_over_layers_reduced():
         op_pf.close()
         op_dec.close()
     cache.close()
+
+
+def test_config4_one_layer_at_its_real_shape_ragged_cache():
+    """One layer of the mixed step at full size, projection -> cache -> attention: sequence 0
+    prefills 16384 tokens while 32 sequences decode one token each against caches of lengths
+    U{1024..131072} (seed 7, as bench.py draws them), all 33 in ONE cache object whose sequences
+    have their own capacities (2.27 M positions: 2.3 GB each for K and V).  Q/K/V come from the
+    fused projection with random-init binary16 weights; sampled prefill rows and every
+    single-token row are checked against the oracle run on what the device holds, the
+    projection's own rows against the oracle's projection within one unit in the last place."""
+    import torch
+
+    import ellm_amd
+
+    dtype, hq, hkv, hidden_size, s_pf, n_dec = orc.F16, 32, 4, 2048, 16384, 32
+    td = torch.float16
+    sc = 1.0 / np.sqrt(D)
+    lengths = np.random.default_rng(7).integers(1024, 131072 + 1, size=n_dec)
+    caps = [s_pf] + [int((n + 63) // 64 * 64) for n in lengths]
+    total = sum(caps)
+    cache = ellm_amd.KVCache.ragged(1, caps, hkv, ellm_amd.DTYPE_F16)
+    kt, vt = cache.layer_flat_tensors(0, td)              # [hkv, total, 128]
+    for h in range(hkv):                                   # the caches already hold their tokens
+        kt[h].copy_(_device_normal((total, D), 200 + h, dtype))
+        vt[h].copy_(_device_normal((total, D), 210 + h, dtype))
+    w = [_device_normal((heads * D, hidden_size), 220 + i, dtype) * hidden_size ** -0.5
+         for i, heads in enumerate((hq, hkv, hkv))]
+    w = [x.to(td) for x in w]
+    jj = np.arange(D // 2, dtype=np.float64)
+    ang = np.arange(max(caps), dtype=np.float64)[:, None] * (1.0e6 ** (-2.0 * jj / D))[None, :]
+    rope_h = np.empty((max(caps), D), dtype=np.float32)
+    rope_h[:, 0::2], rope_h[:, 1::2] = np.cos(ang), np.sin(ang)
+    rope_h = orc.to_storage(rope_h, dtype)
+    rope = to_dev(rope_h, dtype)
+    x_pf = _device_normal((s_pf, 1, hidden_size), 230, dtype)
+    x_dec = _device_normal((1, n_dec, hidden_size), 231, dtype)
+    q_pf = torch.zeros((s_pf, 1, hq, D), dtype=td, device="cuda")
+    q_dec = torch.zeros((1, n_dec, hq, D), dtype=td, device="cuda")
+    out_pf, out_dec = torch.full_like(q_pf, float("nan")), torch.full_like(q_dec, float("nan"))
+    lse_pf = torch.zeros((s_pf, 1, hq), dtype=torch.float32, device="cuda")
+    lse_dec = torch.zeros((1, n_dec, hq), dtype=torch.float32, device="cuda")
+    v0, v1 = cache.layer_ragged(0, 0), cache.layer_ragged(0, 1)
+    assert v1.capacities == caps[1:]
+    proj_pf = ellm_amd.MatMul3(x_pf, w[0], q_pf, w[1], kt, w[2], vt, rope, D, 1, hq, hkv, v0.strides, 0,
+                               seq_table=v0)
+    proj_dec = ellm_amd.MatMul3(x_dec, w[0], q_dec, w[1], kt, w[2], vt, rope, D, n_dec, hq, hkv, v1.strides, 0,
+                                seq_table=v1)
+    att_pf = ellm_amd.Attention(q_pf, kt, vt, out_pf, 1, hq, hkv, D, v0.strides, sc, lse=lse_pf,
+                                max_position_interval=s_pf, seq_table=v0)
+    att_dec = ellm_amd.Attention(q_dec, kt, vt, out_dec, n_dec, hq, hkv, D, v1.strides, sc, lse=lse_dec,
+                                 max_position_interval=1, seq_table=v1)
+    pos = (lengths - 1).astype(np.int32)
+    dpos = torch.from_numpy(pos).cuda()
+    max_pos = int(pos.max())
+    proj_pf.run(0, s_pf, 1)
+    att_pf.run(0, s_pf, 1)
+    proj_dec.run_ragged(dpos, max_pos, n_dec)
+    att_dec.run_ragged(dpos, max_pos, n_dec)
+    torch.cuda.synchronize()
+
+    k_h, v_h = _host(kt, dtype), _host(vt, dtype)          # [hkv, total, 128]
+    strides = [0, total * D, D, 1]
+    offs = np.concatenate([[0], np.cumsum(caps)[:-1]])
+    rng = np.random.default_rng(240)
+
+    # projection rows: four windows of 16 prefill tokens and all 32 single tokens, 1 ulp
+    wh = [_host(x, dtype) for x in w]
+    xh_pf, xh_dec = _host(x_pf, dtype), _host(x_dec, dtype)
+    qh_pf, qh_dec = _host(q_pf, dtype), _host(q_dec, dtype)
+
+    def ulps(got, want):
+        got, want = orc.from_storage(got, dtype), orc.from_storage(want, dtype)
+        return float((np.abs(got - want) / storage_ulp_at(want)).max())
+
+    def storage_ulp_at(want):
+        return 2.0 ** (np.floor(np.log2(np.maximum(np.abs(want), 0.125))) - 10)
+
+    for t0 in (0, 5000, 12345, s_pf - 16):
+        oq = np.zeros((16, 1, hq, D), dtype=np.float16)
+        ok = np.zeros((1, hkv, s_pf, D), dtype=np.float16)
+        ov = np.zeros_like(ok)
+        assert orc.matmul3(np.ascontiguousarray(xh_pf[t0:t0 + 16]), wh[0], wh[1], wh[2], oq, ok, ov, rope_h,
+                           [hkv * s_pf * D, s_pf * D, D, 1], s_pf, t0, 16, dtype) == 0
+        worst = max(ulps(qh_pf[t0:t0 + 16], oq), ulps(k_h[:, t0:t0 + 16], ok[0, :, t0:t0 + 16]),
+                    ulps(v_h[:, t0:t0 + 16], ov[0, :, t0:t0 + 16]))
+        print(f"projection, prefill tokens {t0}..{t0 + 15}: worst {worst:.2f} ulp", flush=True)
+        assert worst <= 1.0
+    capmax = max(caps[1:])
+    oq = np.zeros((1, n_dec, hq, D), dtype=np.float16)
+    ok = np.zeros((n_dec, hkv, capmax, D), dtype=np.float16)
+    ov = np.zeros_like(ok)
+    assert orc.matmul3(xh_dec, wh[0], wh[1], wh[2], oq, ok, ov, rope_h, [hkv * capmax * D, capmax * D, D, 1],
+                       capmax, 0, 1, dtype, positions=pos.astype(np.uint32)) == 0
+    worst = ulps(qh_dec, oq)
+    for i in range(n_dec):
+        row = offs[1 + i] + pos[i]
+        worst = max(worst, ulps(k_h[:, row], ok[i, :, pos[i]]), ulps(v_h[:, row], ov[i, :, pos[i]]))
+    print(f"projection, single tokens: worst {worst:.2f} ulp", flush=True)
+    assert worst <= 1.0
+    del ok, ov
+
+    # attention, prefill side: sampled (token, head) rows on the device's own Q/K/V
+    ref_pf = orc.Operator(qh_pf, k_h, v_h, np.zeros((1,), np.float16), None, 1, hq, hkv, D, strides, sc, dtype)
+    toks = np.concatenate([[0, 31, 63, 64, s_pf - 1], rng.integers(0, s_pf, 27)])
+    rows = np.stack([toks, np.zeros_like(toks), rng.integers(0, hq, toks.size)], 1).astype(np.uint32)
+    _check_rows(ref_pf, rows, 0, out_pf, lse_pf, dtype)
+    # attention, single-token side: every (sequence, head) row
+    got_dec, got_lse = to_host(out_dec, dtype), lse_dec.cpu().numpy()
+    all_heads = np.array([[0, 0, h] for h in range(hq)], dtype=np.uint32)
+    worst_abs = worst_lse = 0.0
+    for i in range(n_dec):
+        o = offs[1 + i]
+        ref = orc.Operator(np.ascontiguousarray(qh_dec[:, i:i + 1]), k_h[:, o:], v_h[:, o:],
+                           np.zeros((1,), np.float16), None, 1, hq, hkv, D, strides, sc, dtype)
+        want, want_lse, _ = ref.run_rows(int(pos[i]), all_heads, 8)
+        res = compare(got_dec[0, i], orc.from_storage(want, dtype), dtype)
+        assert res["ok"], (i, int(lengths[i]), res)
+        worst_abs = max(worst_abs, res["max_abs"])
+        worst_lse = max(worst_lse, float(np.abs(got_lse[0, i] - want_lse).max()))
+    print(f"single-token rows of 32 sequences ({int(lengths.sum())} cached tokens): max_abs {worst_abs:.2e} "
+          f"lse_err {worst_lse:.2e}", flush=True)
+    assert worst_lse <= LSE_TOL
+    for op in (proj_pf, proj_dec, att_pf, att_dec):
+        op.close()
+    cache.close()
