@@ -60,13 +60,7 @@ struct DecodeKernelArgs {
   float scale_log2;   // scale * log2(e)
 };
 
-// Agent-scope (device-wide coherent) relaxed store / load of one float.
-__device__ __forceinline__ void store_coherent(float* p, float v) {
-  __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-}
-__device__ __forceinline__ float load_coherent(const float* p) {
-  return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-}
+// Agent-scope (device-wide coherent) relaxed 8-byte load / store of a pair of floats.
 __device__ __forceinline__ uint64_t load_coherent64(const float* p) {
   return __hip_atomic_load((const uint64_t*)p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
@@ -75,38 +69,19 @@ __device__ __forceinline__ void store_coherent64(float* p, float lo, float hi) {
                         ((uint64_t)__builtin_bit_cast(uint32_t, hi) << 32);
   __hip_atomic_store((uint64_t*)p, bits, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
-// Agent-scope load of four floats.  The compiler has no 16-byte atomic load, so the
-// instruction is written out (sc1 = agent scope, as its own 8-byte atomic loads carry)
-// and the caller waits for it with wait_loaded() before touching the result.
-__device__ __forceinline__ f32x4 load_coherent128_nowait(const float* p) {
-  f32x4 v;
-  asm volatile("global_load_dwordx4 %0, %1, off sc1" : "=v"(v) : "v"(p) : "memory");
-  return v;
+// Agent-scope load of four floats at byte offset `off` of a table: a buffer load with the
+// sc1 cache-policy bit (what the compiler's own agent-scope atomic loads carry).  There is no
+// 16-byte atomic load; as a builtin the compiler tracks the load's completion itself.
+constexpr int kCachePolicySc1 = 16;
+__device__ __forceinline__ f32x4 load_coherent128(__amdgpu_buffer_rsrc_t table, uint32_t off) {
+  return __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(table, off, 0, kCachePolicySc1));
 }
-// Wait for every outstanding vector-memory operation; the registers go through the
-// statement so that no use of them can be scheduled ahead of the wait.
-__device__ __forceinline__ void wait_loaded(f32x4 (&v)[16]) {
-  asm volatile("s_waitcnt vmcnt(0)"
-               : "+v"(v[0]), "+v"(v[1]), "+v"(v[2]), "+v"(v[3]), "+v"(v[4]), "+v"(v[5]), "+v"(v[6]),
-                 "+v"(v[7]));
-  asm volatile(""
-               : "+v"(v[8]), "+v"(v[9]), "+v"(v[10]), "+v"(v[11]), "+v"(v[12]), "+v"(v[13]),
-                 "+v"(v[14]), "+v"(v[15]));
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t table_rsrc(const float* table) {
+  return __builtin_amdgcn_make_buffer_rsrc((void*)table, 0, 0xffffffffu, 0x00020000);
 }
 // Block until every vector-memory operation this wave has issued is complete
 // (s_waitcnt vmcnt(0); expcnt and lgkmcnt left at their maxima).
 __device__ __forceinline__ void wait_vm_done() { __builtin_amdgcn_s_waitcnt(0x0F70); }
-
-// Final value of one output element: normalise, round to the storage type, and
-// (thread d == 0) write the row's log-sum-exp in natural-log units.
-template <typename T>
-__device__ __forceinline__ void store_row_elem(const DecodeKernelArgs& p, uint32_t seq,
-                                               uint32_t head, uint32_t d, float a, float lsum,
-                                               float mmax) {
-  const size_t row = (size_t)seq * p.n_q_heads + head;
-  p.out[row * kHeadDim + d] = (uint16_t)(Mfma<T>::pack2(a / lsum, 0.0f) & 0xffffu);
-  if (p.lse && d == 0) p.lse[row] = (mmax + fast_log2(lsum)) * kLn2;
-}
 
 // K/V rows are read once and never reused: non-temporal loads (measured 8 % faster)
 __device__ __forceinline__ u32x4 stream_load16(const uint16_t* p) {
@@ -118,7 +93,12 @@ __global__ __launch_bounds__(kDecWaves* kWave, 4) void decode_split_kernel(
     DecodeKernelArgs p) {
   __shared__ __attribute__((aligned(16))) uint16_t smem[kDecWaves * kWaveLdsHalves];
 
-  const uint32_t split = blockIdx.x;
+  // The split a workgroup takes is rotated by its plane's number.  Workgroups are dealt to the
+  // eight XCDs by their linear id; with the unrotated mapping (and a split count that is a
+  // multiple of 8) one XCD would read the same stretch of every plane, and XCDs differ in how
+  // fast they reach a given stretch of memory: 4 sequences x 32768 keys took 51.4 us
+  // unrotated, 48.0 us rotated (16 x 8192: no difference).
+  const uint32_t split = (blockIdx.x + blockIdx.y + gridDim.y * blockIdx.z) % gridDim.x;
   const uint32_t kvh = blockIdx.y / p.head_groups;
   const uint32_t hgrp = blockIdx.y % p.head_groups;
   const uint32_t seq = blockIdx.z;
@@ -251,49 +231,68 @@ __global__ __launch_bounds__(kDecWaves* kWave, 4) void decode_split_kernel(
   // Merge the four waves through LDS: red[wave][head][128 acc + max + sum].
   __syncthreads();
   float* red = (float*)smem;
-  constexpr int kRedPitch = kHeadDim + 2;
+  constexpr int kRedPitch = kHeadDim + 4;  // rows 16-byte aligned
   static_assert(kDecWaves * kMaxHeadsPerGroup * kRedPitch * 4 <= kDecWaves * kWaveLdsHalves * 2,
                 "reduction buffer must fit in the staging buffers");
   if ((uint32_t)c < heads_here) {
     float* row = red + (wave * kMaxHeadsPerGroup + c) * kRedPitch;
 #pragma unroll
-    for (int b = 0; b < 8; ++b)
-#pragma unroll
-      for (int r = 0; r < 4; ++r) row[16 * b + 4 * g + r] = acc[b][r];
-    if (g == 0) {
-      row[kHeadDim] = m_run;
-      row[kHeadDim + 1] = l_run;
-    }
+    for (int b = 0; b < 8; ++b) *(f32x4*)(row + 16 * b + 4 * g) = acc[b];
+    if (g == 0) *(f32x2*)(row + kHeadDim) = f32x2{m_run, l_run};
   }
   __syncthreads();
 
-  for (uint32_t idx = tid; idx < heads_here * kHeadDim; idx += kDecWaves * kWave) {
-    const uint32_t h = idx / kHeadDim, d = idx % kHeadDim;
-    float mw[kDecWaves];
+  // From here to the end a thread owns four consecutive columns of one head (an item;
+  // eight heads make 256 items, one per thread, sixteen heads two per thread).
+  constexpr int kQuads = kHeadDim / 4;
+  constexpr int kThreads = kDecWaves * kWave;
+  constexpr int kItems = kMaxHeadsPerGroup * kQuads / kThreads;
+  const uint32_t n_items = heads_here * kQuads;
+  auto emit_final = [&](uint32_t h, uint32_t dq, const f32x4& a, float l, float m) {
+    const size_t row = (size_t)seq * p.n_q_heads + head0 + h;
+    const float inv = 1.0f / l;
+    u32x2 w;
+    w[0] = Mfma<T>::pack2(a[0] * inv, a[1] * inv);
+    w[1] = Mfma<T>::pack2(a[2] * inv, a[3] * inv);
+    *(u32x2*)(p.out + row * kHeadDim + 4 * dq) = w;
+    if (p.lse && dq == 0) p.lse[row] = (m + fast_log2(l)) * kLn2;
+  };
+  // entry `index` of a table of partials with `pitch` entries per (sequence, head) row
+  auto store_partial = [&](float* acc_tab, float* ml_tab, uint32_t pitch, uint32_t index, uint32_t h,
+                           uint32_t dq, const f32x4& a, float l, float m) {
+    const size_t prow = ((size_t)seq * p.n_q_heads + head0 + h) * pitch + index;
+    store_coherent64(acc_tab + prow * kHeadDim + 4 * dq, a[0], a[1]);
+    store_coherent64(acc_tab + prow * kHeadDim + 4 * dq + 2, a[2], a[3]);
+    if (dq == 0) store_coherent64(ml_tab + prow * 2, m, l);
+  };
+#pragma unroll
+  for (int n = 0; n < kItems; ++n) {
+    const uint32_t item = tid + n * kThreads;
+    if (item >= n_items) continue;
+    const uint32_t h = item / kQuads, dq = item % kQuads;
+    f32x2 ml[kDecWaves];
+    f32x4 part[kDecWaves];
+#pragma unroll
+    for (int w = 0; w < kDecWaves; ++w) {
+      const float* row = red + (w * kMaxHeadsPerGroup + h) * kRedPitch;
+      ml[w] = *(const f32x2*)(row + kHeadDim);
+      part[w] = *(const f32x4*)(row + 4 * dq);
+    }
     float mmax = -INFINITY;
 #pragma unroll
-    for (int w = 0; w < kDecWaves; ++w) {
-      mw[w] = red[(w * kMaxHeadsPerGroup + h) * kRedPitch + kHeadDim];
-      mmax = fmaxf(mmax, mw[w]);
-    }
-    float lsum = 0.0f, a = 0.0f;
+    for (int w = 0; w < kDecWaves; ++w) mmax = fmaxf(mmax, ml[w][0]);
+    float lsum = 0.0f;
+    f32x4 a = {0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
     for (int w = 0; w < kDecWaves; ++w) {
-      const float wgt = (mw[w] == -INFINITY) ? 0.0f : fast_exp2(mw[w] - mmax);
-      lsum += wgt * red[(w * kMaxHeadsPerGroup + h) * kRedPitch + kHeadDim + 1];
-      a += wgt * red[(w * kMaxHeadsPerGroup + h) * kRedPitch + d];
+      const float wgt = (ml[w][0] == -INFINITY) ? 0.0f : fast_exp2(ml[w][0] - mmax);
+      lsum += wgt * ml[w][1];
+      a += wgt * part[w];
     }
-    const uint32_t head = head0 + h;
-    if (p.n_split == 1) {
-      store_row_elem<T>(p, seq, head, d, a, lsum, mmax);
-    } else {
-      const size_t prow = ((size_t)seq * p.n_q_heads + head) * p.n_split + split;
-      store_coherent(p.ws_acc + prow * kHeadDim + d, a);
-      if (d == 0) {
-        store_coherent(p.ws_ml + prow * 2, mmax);
-        store_coherent(p.ws_ml + prow * 2 + 1, lsum);
-      }
-    }
+    if (p.n_split == 1)
+      emit_final(h, dq, a, lsum, mmax);
+    else
+      store_partial(p.ws_acc, p.ws_ml, p.n_split, split, h, dq, a, lsum, mmax);
   }
   if (p.n_split == 1) return;
 
@@ -307,6 +306,11 @@ __global__ __launch_bounds__(kDecWaves* kWave, 4) void decode_split_kernel(
   // barrier collects all of them, and only then is the arrival counted; the
   // merging workgroup issues its loads only after the counter's return value
   // has been seen by all of its threads.
+  // (Measured and dropped: tickets taken at the end of the key loop, the holder of the
+  // last one keeping its partial in registers and waiting for a count of stored partials.
+  // The ticket order is not the order of finishing, so the folder mostly waits for a
+  // slower workgroup's store, count and its own poll: 0.3 us slower with one fold level,
+  // 2.7 us with two.)
   // Splits are grouped in clusters of 16.  The last arrival of a cluster folds
   // its partials into one cluster partial; the last cluster to finish folds the
   // cluster partials into the output.  A merge is one workgroup reading from
@@ -331,68 +335,60 @@ __global__ __launch_bounds__(kDecWaves* kWave, 4) void decode_split_kernel(
     __syncthreads();
     return s_last != 0;
   };
-  // Fold `count` (<= 16) partials of every head of this group, starting at
-  // partial `first` of a table with `pitch` partials per row.  A thread owns four
-  // consecutive columns of one head (one item; eight heads make 256 items, one per
-  // thread) and issues every load it needs before it waits for any: a fold costs
-  // one trip to memory, an 8-byte (max, sum) pair per thread, shared through LDS,
-  // and one 16-byte accumulator quad per partial.
+  // Fold `count` (<= 16) partials of every head of this group, starting at partial `first`
+  // of a table with `pitch` partials per row.  A thread issues every load its item needs
+  // before it uses any: a fold costs one trip to memory, an 8-byte (max, sum) pair per
+  // thread, shared through LDS, and one 16-byte accumulator quad per partial; the pairs come
+  // back from LDS into registers in one go as well (read one by one inside the loops below,
+  // every LDS round trip showed: 1.1 us for eight partials).
   // emit(h, dq, a[4], sum, max) receives columns 4 dq .. 4 dq + 3.
   auto fold = [&](const float* acc_tab, const float* ml_tab, uint32_t pitch, uint32_t first,
                   uint32_t count, auto emit) {
-    float* sm = (float*)smem;  // [head][kMergeFan][2]; the staging buffers are idle by now
+    float* sm = (float*)smem;  // [head][kMergeFan][2]; the reduction buffer is idle by now
+    const __amdgpu_buffer_rsrc_t acc_rsrc = table_rsrc(acc_tab);
     const uint32_t n_ml = heads_here * count;
     const uint32_t h_e = tid / count, s_e = tid % count;
     uint64_t ml_bits = 0;
     if ((uint32_t)tid < n_ml)
       ml_bits = load_coherent64(
           ml_tab + (((size_t)seq * p.n_q_heads + head0 + h_e) * pitch + first + s_e) * 2);
-    const uint32_t items = heads_here * (kHeadDim / 4);
-    bool published = false;
-    for (uint32_t item = tid; item < (items + kDecWaves * kWave - 1) / (kDecWaves * kWave) *
-                                         (kDecWaves * kWave);
-         item += kDecWaves * kWave) {  // same trip count for every thread: the loop holds a barrier
-      const bool mine = item < items;
-      const uint32_t h = mine ? item / (kHeadDim / 4) : 0, dq = item % (kHeadDim / 4);
-      const float* ac =
-          acc_tab + (((size_t)seq * p.n_q_heads + head0 + h) * pitch + first) * kHeadDim + 4 * dq;
+#pragma unroll
+    for (int n = 0; n < kItems; ++n) {
+      const uint32_t item = tid + n * kThreads;
+      const bool mine = item < n_items;
+      const uint32_t h = mine ? item / kQuads : 0, dq = item % kQuads;
+      // byte offset of entry `first`, columns 4 dq.. of this head's row (tables stay far below 4 GB)
+      const uint32_t at =
+          (uint32_t)(((((size_t)seq * p.n_q_heads + head0 + h) * pitch + first) * kHeadDim + 4 * dq) * 4);
       f32x4 av[kMergeFan];
 #pragma unroll
       for (int i = 0; i < kMergeFan; ++i) {
         av[i] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
-        if ((uint32_t)i < count) av[i] = load_coherent128_nowait(ac + (size_t)i * kHeadDim);
+        if (mine && (uint32_t)i < count) av[i] = load_coherent128(acc_rsrc, at + (uint32_t)i * (kHeadDim * 4));
       }
-      wait_loaded(av);  // (also covers ml_bits: the compiler's own wait for it comes no later)
-      if (!published) {
+      if (n == 0) {  // (every thread passes here once: the branch holds a barrier)
         if ((uint32_t)tid < n_ml) *(uint64_t*)(sm + (h_e * kMergeFan + s_e) * 2) = ml_bits;
         __syncthreads();
-        published = true;
       }
       if (!mine) continue;
       const float* hm = sm + h * kMergeFan * 2;
-      float m_new = hm[0];
-      for (uint32_t i = 1; i < count; ++i) m_new = fmaxf(m_new, hm[2 * i]);
+      f32x2 ml[kMergeFan];
+#pragma unroll
+      for (int i = 0; i < kMergeFan; ++i)
+        ml[i] = (uint32_t)i < count ? *(const f32x2*)(hm + 2 * i) : f32x2{-INFINITY, 0.0f};
+      float m_new = ml[0][0];
+#pragma unroll
+      for (int i = 1; i < kMergeFan; ++i) m_new = fmaxf(m_new, ml[i][0]);
       float l_acc = 0.0f;
       f32x4 a = {0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
       for (int i = 0; i < kMergeFan; ++i) {
-        if ((uint32_t)i < count) {
-          const float wgt = fast_exp2(hm[2 * i] - m_new);
-          l_acc += wgt * hm[2 * i + 1];
-          a += wgt * av[i];
-        }
+        const float wgt = fast_exp2(ml[i][0] - m_new);  // (an absent entry weighs exp2(-inf) = 0)
+        l_acc += wgt * ml[i][1];
+        a += wgt * av[i];
       }
       emit(h, dq, a, l_acc, m_new);
     }
-  };
-  auto emit_final = [&](uint32_t h, uint32_t dq, const f32x4& a, float l, float m) {
-    const size_t row = (size_t)seq * p.n_q_heads + head0 + h;
-    const float inv = 1.0f / l;
-    u32x2 w;
-    w[0] = Mfma<T>::pack2(a[0] * inv, a[1] * inv);
-    w[1] = Mfma<T>::pack2(a[2] * inv, a[3] * inv);
-    *(u32x2*)(p.out + row * kHeadDim + 4 * dq) = w;
-    if (p.lse && dq == 0) p.lse[row] = (m + fast_log2(l)) * kLn2;
   };
 
   if (!arrive(ctr + 1 + cluster, in_cluster)) return;
@@ -402,10 +398,7 @@ __global__ __launch_bounds__(kDecWaves* kWave, 4) void decode_split_kernel(
   }
   fold(p.ws_acc, p.ws_ml, p.n_split, cluster * kMergeFan, in_cluster,
        [&](uint32_t h, uint32_t dq, const f32x4& a, float l, float m) {
-         const size_t crow = ((size_t)seq * p.n_q_heads + head0 + h) * p.n_cluster_max + cluster;
-         store_coherent64(p.ws2_acc + crow * kHeadDim + 4 * dq, a[0], a[1]);
-         store_coherent64(p.ws2_acc + crow * kHeadDim + 4 * dq + 2, a[2], a[3]);
-         if (dq == 0) store_coherent64(p.ws2_ml + crow * 2, m, l);
+         store_partial(p.ws2_acc, p.ws2_ml, p.n_cluster_max, cluster, h, dq, a, l, m);
        });
   if (!arrive(ctr, n_clusters)) return;
   fold(p.ws2_acc, p.ws2_ml, p.n_cluster_max, 0, n_clusters, emit_final);
