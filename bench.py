@@ -137,7 +137,7 @@ def bench_decode(batch, length, steps, warmup, hq=32, hkv=4, copies=4):
     }
 
 
-def bench_prefill(seq, steps, warmup, hq=32, hkv=4, dtype_name="f16", p0=0, zero_kv=False):
+def bench_prefill(seq, steps, warmup, hq=32, hkv=4, dtype_name="f16", p0=0, zero_kv=False, batch=1, copies=1):
     import torch
 
     import ellm_amd
@@ -150,20 +150,23 @@ def bench_prefill(seq, steps, warmup, hq=32, hkv=4, dtype_name="f16", p0=0, zero
     qs = torch.rand((1, 1, hq, 1), generator=g, device="cuda") * 1.5 + 0.5   # per-head scale U[0.5, 2]
     ks = torch.rand((1, hkv, 1, 1), generator=g, device="cuda") * 1.5 + 0.5
     vs = torch.rand((1, hkv, 1, 1), generator=g, device="cuda") * 1.5 + 0.5
-    q = (_dev_normal((seq, 1, hq, D), torch.float32, 11) * qs).to(dt)
-    k = (_dev_normal((1, hkv, cap, D), torch.float32, 12) * ks).to(dt)
-    v = (_dev_normal((1, hkv, cap, D), torch.float32, 13) * vs).to(dt)
-    if zero_kv:  # diagnostic: same instruction stream, operands that toggle nothing
-        k.zero_()
-        v.zero_()
-    out = torch.zeros_like(q)
-    lse = torch.zeros((seq, 1, hq), dtype=torch.float32, device="cuda")
-    op = ellm_amd.Attention(q, k, v, out, 1, hq, hkv, D, [hkv * cap * D, cap * D, D, 1], scale,
-                            lse=lse, sequence_capacity=cap, max_position_interval=seq)
-    per, step_ms = _time_steps(lambda i: op.run(p0, seq, 1), steps, warmup)
-    flops = 4 * D * hq * (seq * p0 + seq * (seq + 1) // 2)
+    ops = []
+    for c in range(copies):     # several cache sets in rotation where a step should find nothing cached
+        q = (_dev_normal((seq, batch, hq, D), torch.float32, 11 + 10 * c) * qs).to(dt)
+        k = (_dev_normal((batch, hkv, cap, D), torch.float32, 12 + 10 * c) * ks).to(dt)
+        v = (_dev_normal((batch, hkv, cap, D), torch.float32, 13 + 10 * c) * vs).to(dt)
+        if zero_kv:  # diagnostic: same instruction stream, operands that toggle nothing
+            k.zero_()
+            v.zero_()
+        out = torch.zeros_like(q)
+        lse = torch.zeros((seq, batch, hq), dtype=torch.float32, device="cuda")
+        ops.append((ellm_amd.Attention(q, k, v, out, batch, hq, hkv, D, [hkv * cap * D, cap * D, D, 1], scale,
+                                       lse=lse, sequence_capacity=cap, max_position_interval=seq), q, k, v, out, lse))
+    per, step_ms = _time_steps(lambda i: ops[i % copies][0].run(p0, seq, batch), steps, warmup)
+    flops = batch * 4 * D * hq * (seq * p0 + seq * (seq + 1) // 2)
     kern_ms = sum(per) / len(per)
-    op.close()
+    for op in ops:
+        op[0].close()
     return {
         "flops": flops,
         "ms_per_step": step_ms,
@@ -779,7 +782,7 @@ def main():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--skip-cpu", action="store_true")
-    ap.add_argument("--only", default="", help="decode | prefill | decode128k | chunk | smallchunk | mixed | mixed48 | kvwrite | tokenstep | layerstep | qkv | oproj | chunkproj | chunkblock | stepproj")
+    ap.add_argument("--only", default="", help="decode | prefill | decode128k | chunk | smallchunk | lastchunk | mixed | mixed48 | kvwrite | tokenstep | layerstep | qkv | oproj | chunkproj | chunkblock | stepproj")
     ap.add_argument("--prefill-zero-kv", action="store_true",
                     help="diagnostic for --only prefill: K and V all zero (the kernel issues the same "
                          "instructions; separates its cycle count from the clock the part sustains "
@@ -907,6 +910,28 @@ def main():
             "metric": "prefill attn TFLOP/s", "value": round(sc["tflops"], 2), "unit": "TFLOP/s",
             "ms_per_step": round(sc["ms_per_step"], 5), "steps": args.steps,
             "kv_gbs": round(2 * 4 * (8192 + 64) * D * 2 / (sc["ms_per_step"] * 1e-3) / 1e9, 1),
+        })
+
+    if args.only in ("", "lastchunk"):
+        # the reference's serving loop ends a prompt with a chunk of (prompt % 64) positions x 24 sequences
+        # (src/serving/start copy.rs:71-101): few query rows per K/V plane over thousands of cached tokens
+        lc_dec = bench_decode(24, 8192, args.steps, min(args.warmup, 5), copies=3)
+        lc = {t: bench_prefill(t, args.steps, min(args.warmup, 5), p0=8192, batch=24, copies=3) for t in (2, 8, 16, 33)}
+        kv_bytes = 2 * 24 * 4 * 8192 * D * 2
+        also.append({
+            "workload": "short last chunk of a prompt: 2 / 8 / 16 / 33 new tokens x 24 sequences on 8192-token caches, "
+                        "32q/4kv heads, fp16 (up to 16 tokens: the streaming chunk kernel, one workgroup per GQA "
+                        "group's rows, keys split over workgroups + merge launch; 33 tokens: the tile kernel); "
+                        "beside it the single-token kernel on the same caches",
+            "metric": "chunk attention us per call", "unit": "us",
+            "value": round(lc[16]["ms_per_step"] * 1e3, 1),
+            "us_by_tokens": {str(t): round(r["ms_per_step"] * 1e3, 1) for t, r in lc.items()},
+            "single_token_us": round(lc_dec["ms_per_step"] * 1e3, 1),
+            "kv_gbs_by_tokens": {str(t): round(kv_bytes / (r["ms_per_step"] * 1e-3) / 1e9, 1) for t, r in lc.items()},
+            "steps": args.steps,
+            "roofline": {"bound": "hbm", "achieved": round(kv_bytes / (lc[16]["kernel_ms"] * 1e-3) / 1e9, 1),
+                         "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                         "frac": round(kv_bytes / (lc[16]["kernel_ms"] * 1e-3) / 1e9 / HBM_PEAK_GBS, 4), "traffic": None},
         })
 
     if args.only in ("", "mixed"):

@@ -75,6 +75,11 @@ struct PrefillKernelArgs {
 // Rows: wave w owns row block w (32 rows) of 8; all 256 rows read the same K/V
 // tiles.  Waves 0-3 stage the K tiles, waves 4-7 the V tiles.
 // ---------------------------------------------------------------------------
+__device__ __forceinline__ uint64_t uniform64(const void* p) {  // the compiler cannot see that p is wave-uniform
+  const uint32_t lo = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(uint64_t)p);
+  const uint32_t hi = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)((uint64_t)p >> 32));
+  return ((uint64_t)hi << 32) | (uint64_t)lo;
+}
 typedef __attribute__((address_space(3))) uint16_t LdsHalf;
 typedef __attribute__((address_space(3))) u32x4 LdsU32x4;
 typedef __attribute__((address_space(3))) u32x2 LdsU32x2;
@@ -429,6 +434,216 @@ __global__ __launch_bounds__(kPpThreads, 2) void prefill_pingpong_kernel(Prefill
   }
 }
 
+// ---------------------------------------------------------------------------
+// Few query rows per K/V plane: the short last chunk of a prompt (2 - 33 tokens x 24
+// sequences on caches of thousands of tokens in the reference's serving loop,
+// src/serving/start copy.rs:71-101).  The ping-pong kernel above is built for tiles that
+// are re-used by thousands of rows and sit in L2; here every K/V byte is used once by at
+// most 128 rows and the call is a stream from HBM, like the single-token kernel: what
+// matters is bytes in flight, not MFMA issue.  One workgroup = 4 waves x 32 query rows =
+// all (token, head) pairs of one GQA group (row r of the plane = token r / group, head
+// r % group), so a plane is read once; the key range is split over gridDim.y workgroups
+// (about three per compute unit, 36 KB of LDS each), which leave partial rows for
+// prefill_merge_kernel as the split form of the kernel above does.  Chunks of 32 keys go
+// memory -> registers -> LDS (double-buffered, one barrier a chunk, the next chunk's loads in
+// flight during the MFMAs of this one); operands and soft-max as above.
+// ---------------------------------------------------------------------------
+constexpr int kSK = 32;                        // keys per chunk
+constexpr int kStThreads = 4 * kWave;
+constexpr int kStKsHalves = kSK * kKsPitch;
+constexpr int kStVsHalves = kSK * kVsPitch;
+
+// (Tried and dropped: two chunks of loads in flight per workgroup through a second set of
+// staging registers, 192 registers a wave: 16 tokens x 24 sequences on 8192 keys 94 -> 112 us.)
+template <typename T>
+__global__ __launch_bounds__(kStThreads, 3) void chunk_stream_kernel(PrefillKernelArgs p) {
+  __shared__ __attribute__((aligned(16))) uint16_t smem[2 * kStKsHalves + 2 * kStVsHalves];
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int j = lane & 31, g = lane >> 5;
+  const uint32_t seq = blockIdx.x / p.n_kv_heads, kvh = blockIdx.x % p.n_kv_heads;
+  const uint32_t S = p.interval, P0 = p.position_index;
+  const uint32_t kmax = P0 + S - 1;
+  const uint32_t all_tiles = kmax / kBK + 1;
+  const uint32_t kt0 = blockIdx.y * p.split_tiles;
+  if (kt0 >= all_tiles) return;  // (prefill_merge_kernel derives the live splits the same way)
+  const uint32_t n_tiles = min(all_tiles - kt0, p.split_tiles);
+  const uint32_t k0 = kt0 * kBK;                                   // first key of this split
+  const uint32_t n_chunks = (min(kmax + 1, k0 + n_tiles * kBK) - k0 + kSK - 1) / kSK;
+
+  const uint32_t rows = S * p.group;                                // query rows of the plane, <= 128
+  const uint32_t r = 32 * wave + j;
+  const bool row_valid = r < rows;
+  const uint32_t rc = row_valid ? r : rows - 1;
+  const uint32_t tok = rc / p.group, head = kvh * p.group + rc % p.group;
+  const uint32_t rowpos = P0 + tok;
+  // positions of the wave's first and last row: chunks past the last are skipped, chunks up to
+  // the first need no mask
+  const uint32_t wave_first_pos = P0 + min(32u * wave, rows - 1) / p.group;
+  const uint32_t wave_last_pos = P0 + min(32u * wave + 31u, rows - 1) / p.group;
+  const bool wave_has_rows = 32u * wave < rows;
+
+  u32x4 qreg[8];
+  {
+    const uint16_t* qrow =
+        p.q + (size_t)tok * p.q_token_stride + ((size_t)seq * p.n_q_heads + head) * kHeadDim;
+#pragma unroll
+    for (int s = 0; s < 8; ++s) {
+      qreg[s] = load16(qrow + 16 * s + 8 * g);
+      if (p.negate_q) qreg[s] ^= 0x80008000u;
+    }
+  }
+  const float c = p.c;
+
+  const size_t plane_at = seq_plane_offset(p.seq_offsets, p.kv_stride_seq, seq) + kvh * p.kv_stride_head;
+  const uint16_t* kplane = p.k + plane_at;
+  const uint16_t* vplane = p.v + plane_at;
+  const uint32_t stride_pos = (uint32_t)p.kv_stride_pos;
+  // staging: 256 threads move one 32 x 128 chunk of K and one of V, two 16-byte pieces of each
+  // (rows ld_r and ld_r + 16, columns 8 ld_c ..), through buffer loads whose descriptor ends
+  // at the last visible key: rows beyond it read as zeros.
+  const int ld_c = tid & 15, ld_r = tid >> 4;
+  const uint64_t kplane_u = uniform64(kplane), vplane_u = uniform64(vplane);
+  const uint32_t chunk_bytes = kSK * stride_pos * 2;
+  const uint32_t valid_bytes = (kmax * stride_pos + kHeadDim) * 2;
+  const uint32_t piece_off0 = (ld_r * stride_pos + 8 * ld_c) * 2;
+  const uint32_t piece_off1 = ((ld_r + 16) * stride_pos + 8 * ld_c) * 2;
+  u32x4 stg_a[4];
+  auto load_chunk = [&](uint32_t ck, u32x4 (&stg)[4]) {  // ck relative to this split's first chunk; wave-uniform
+    const uint32_t off = k0 * stride_pos * 2 + ck * chunk_bytes;
+    const uint32_t left = valid_bytes - __builtin_amdgcn_readfirstlane(min(valid_bytes, off));
+    const __amdgpu_buffer_rsrc_t kr = __builtin_amdgcn_make_buffer_rsrc((void*)(kplane_u + off), 0, left, kBufferFlags);
+    const __amdgpu_buffer_rsrc_t vr = __builtin_amdgcn_make_buffer_rsrc((void*)(vplane_u + off), 0, left, kBufferFlags);
+    stg[0] = __builtin_amdgcn_raw_buffer_load_b128(kr, piece_off0, 0, 2);   // 2: non-temporal, read once
+    stg[1] = __builtin_amdgcn_raw_buffer_load_b128(kr, piece_off1, 0, 2);
+    stg[2] = __builtin_amdgcn_raw_buffer_load_b128(vr, piece_off0, 0, 2);
+    stg[3] = __builtin_amdgcn_raw_buffer_load_b128(vr, piece_off1, 0, 2);
+  };
+  const uint32_t lds0 = (uint32_t)(uintptr_t)(LdsHalf*)smem;
+  const uint32_t ks_store = lds0 + 2 * (ld_r * kKsPitch + 8 * ld_c);
+  const uint32_t vs_store = lds0 + 2 * (2 * kStKsHalves + ld_r * kVsPitch + 8 * ld_c);
+  auto store_chunk = [&](uint32_t buf, const u32x4 (&stg)[4]) {
+    *(LdsU32x4*)(ks_store + 2 * buf * kStKsHalves) = stg[0];
+    *(LdsU32x4*)(ks_store + 2 * (buf * kStKsHalves + 16 * kKsPitch)) = stg[1];
+    *(LdsU32x4*)(vs_store + 2 * buf * kStVsHalves) = stg[2];
+    *(LdsU32x4*)(vs_store + 2 * (buf * kStVsHalves + 16 * kVsPitch)) = stg[3];
+  };
+  // operand addresses: as in the kernel above (K rows as the A operand of S^T = K.Q^T, V through
+  // the transposing read as the A operand of O^T += V^T.P^T, keys in the order P is left in)
+  const uint32_t k_read = lds0 + 2 * (j * kKsPitch + 8 * g);
+  const uint32_t v_read = lds0 + 2 * (2 * kStKsHalves + (4 * g + ((lane & 15) >> 2)) * kVsPitch +
+                                      16 * ((lane >> 4) & 1) + 4 * (lane & 3));
+
+  float m_run = -INFINITY, l_run = 0.0f;
+  f32x16 oacc[4];
+#pragma unroll
+  for (int db = 0; db < 4; ++db)
+#pragma unroll
+    for (int e = 0; e < 16; ++e) oacc[db][e] = 0.0f;
+
+  auto compute = [&](uint32_t ck) __attribute__((always_inline)) {
+    const uint32_t kb = k0 + ck * kSK;
+    const uint32_t buf = ck & 1;
+    if (wave_has_rows && kb <= wave_last_pos) {
+      const uint32_t ks = k_read + 2 * buf * kStKsHalves;
+      const uint32_t vs = v_read + 2 * buf * kStVsHalves;
+      f32x16 st;
+#pragma unroll
+      for (int e = 0; e < 16; ++e) st[e] = 0.0f;
+#pragma unroll
+      for (int s = 0; s < 8; ++s) {
+        const u32x4 a = *(const LdsU32x4*)(ks + 2 * 16 * s);
+        st = Mfma<T>::m32x32x16(a, qreg[s], st);
+      }
+      if (kb + kSK - 1 > wave_first_pos) {  // chunk crosses the diagonal of some row of this wave
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+          const uint32_t key = kb + 8 * (e >> 2) + 4 * g + (e & 3);
+          st[e] = (key <= rowpos) ? st[e] : -INFINITY;
+        }
+      }
+      float rmax = st[0];
+#pragma unroll
+      for (int e = 1; e < 16; ++e) rmax = fmaxf(rmax, st[e]);
+      rmax = max_with_partner_half(rmax);
+      const float tmax = rmax * c;
+      const bool grow = tmax > m_run + kRescaleStep;
+      if (__any(grow)) {
+        const float m_new = grow ? tmax : m_run;
+        const float alpha = grow ? fast_exp2(m_run - m_new) : 1.0f;
+        m_run = m_new;
+        l_run *= alpha;
+#pragma unroll
+        for (int db = 0; db < 4; ++db) oacc[db] *= alpha;
+      }
+      const float neg_m = (m_run == -INFINITY) ? 0.0f : -m_run;
+      float psum = 0.0f;
+      u32x4 pk[2];
+#pragma unroll
+      for (int cc = 0; cc < 2; ++cc)
+#pragma unroll
+        for (int w = 0; w < 4; ++w) {
+          const float p0 = fast_exp2(__builtin_fmaf(st[8 * cc + 2 * w], c, neg_m));
+          const float p1 = fast_exp2(__builtin_fmaf(st[8 * cc + 2 * w + 1], c, neg_m));
+          pk[cc][w] = Mfma<T>::pack2(p0, p1);
+          psum += p0 + p1;
+        }
+      l_run += psum;
+#pragma unroll
+      for (int cc = 0; cc < 2; ++cc)
+#pragma unroll
+        for (int db = 0; db < 4; ++db) {
+          const uint32_t at = vs + 2 * (16 * cc * kVsPitch + 32 * db);
+          const i16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((LdsI16x4*)at);
+          const i16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((LdsI16x4*)(at + 2 * 8 * kVsPitch));
+          const u32x2 l2 = __builtin_bit_cast(u32x2, lo), h2 = __builtin_bit_cast(u32x2, hi);
+          oacc[db] = Mfma<T>::m32x32x16(u32x4{l2[0], l2[1], h2[0], h2[1]}, pk[cc], oacc[db]);
+        }
+    }
+  };
+  load_chunk(0, stg_a);
+  store_chunk(0, stg_a);
+  if (n_chunks > 1) load_chunk(1, stg_a);
+  __syncthreads();
+  for (uint32_t ck = 0; ck < n_chunks; ++ck) {
+    compute(ck);
+    if (ck + 1 < n_chunks) {
+      store_chunk((ck & 1) ^ 1, stg_a);
+      if (ck + 2 < n_chunks) load_chunk(ck + 2, stg_a);
+    }
+    __syncthreads();
+  }
+
+  const float l = sum_with_partner_half(l_run);
+  if (!row_valid) return;
+  if (p.n_split > 1) {
+    const size_t part = (((size_t)tok * p.batch_pitch + seq) * p.n_q_heads + head) * p.n_split + blockIdx.y;
+    float* orow = p.part_o + part * kHeadDim;
+#pragma unroll
+    for (int db = 0; db < 4; ++db)
+#pragma unroll
+      for (int q4 = 0; q4 < 4; ++q4)
+        *(f32x4*)(orow + 32 * db + 8 * q4 + 4 * g) =
+            f32x4{oacc[db][4 * q4], oacc[db][4 * q4 + 1], oacc[db][4 * q4 + 2], oacc[db][4 * q4 + 3]};
+    if (g == 0) *(float2*)(p.part_ml + part * 2) = float2{m_run, l};
+  } else {
+    const float inv = 1.0f / l;
+    uint16_t* orow =
+        p.out + (size_t)tok * p.q_token_stride + ((size_t)seq * p.n_q_heads + head) * kHeadDim;
+#pragma unroll
+    for (int db = 0; db < 4; ++db)
+#pragma unroll
+      for (int q4 = 0; q4 < 4; ++q4) {
+        u32x2 w;
+        w[0] = Mfma<T>::pack2(oacc[db][4 * q4] * inv, oacc[db][4 * q4 + 1] * inv);
+        w[1] = Mfma<T>::pack2(oacc[db][4 * q4 + 2] * inv, oacc[db][4 * q4 + 3] * inv);
+        *(u32x2*)(orow + 32 * db + 8 * q4 + 4 * g) = w;
+      }
+    if (p.lse && g == 0)
+      p.lse[((size_t)tok * p.batch_pitch + seq) * p.n_q_heads + head] = (m_run + fast_log2(l)) * kLn2;
+  }
+}
+
 // Folds the partial results of a split launch: G lanes per (query row, four columns) take
 // the row's splits in turn and combine through lane exchanges (with hundreds of splits and
 // few rows a thread walking them alone would be one long chain of memory round trips).
@@ -526,6 +741,50 @@ hipError_t launch_pingpong(const AttnArgs& a, hipStream_t stream) {
   // scale == 0 (uniform attention): a tiny positive c keeps -inf * c == -inf for masked keys
   p.c = c > 0.0f ? c : 1e-37f;
 
+  p.part_o = a.prefill_part_o;
+  p.part_ml = a.prefill_part_ml;
+  auto merge_launch = [&]() {
+    const size_t items = (size_t)a.position_interval * a.batch * a.n_q_heads * (kHeadDim / 4);
+    auto merge = [&](auto kernel, size_t lanes) {
+      hipLaunchKernelGGL(kernel, dim3((uint32_t)((items * lanes + 255) / 256)), dim3(256), 0, stream, p, a.batch);
+      return hipGetLastError();
+    };
+    // lanes per item: more when there are many splits to walk, as long as the grid stays small
+    constexpr size_t kLanesMax = (size_t)1 << 21;
+    if (p.n_split > 32 && items * 64 <= kLanesMax) return merge(prefill_merge_kernel<T, 64>, 64);
+    if (p.n_split > 8 && items * 8 <= kLanesMax) return merge(prefill_merge_kernel<T, 8>, 8);
+    return merge(prefill_merge_kernel<T, 1>, 1);
+  };
+
+  // Few query rows per plane on a cache long enough to be worth streaming: one workgroup
+  // covers all rows of a GQA group, the key range is split until there are about three
+  // workgroups per compute unit (splits of at least 256 keys), as far as the workspace holds
+  // the partial rows.
+  const uint32_t all_tiles = (a.position_index + a.position_interval - 1) / kBK + 1;
+  const size_t all_rows = (size_t)a.position_interval * a.batch_pitch * a.n_q_heads;
+  if ((size_t)a.position_interval * a.group <= 128 && all_tiles >= 8) {
+    const uint32_t planes = a.batch * a.n_kv_heads;
+    // rows in one wave only: three workgroups per unit; more rows: two per unit, i.e. fewer and
+    // longer splits, less traffic of partial rows (measured, 24 sequences on 8192 keys: 2 tokens
+    // 70.7 / 75.3 us with three / two per unit, 16 tokens 108 / 94.5 us)
+    const uint32_t per_cu = (size_t)a.position_interval * a.group > 32 ? 2 : 3;
+    uint32_t want = (per_cu * a.n_cu + planes - 1) / planes;
+    const size_t room = a.prefill_part_o ? a.prefill_part_rows / all_rows : 1;
+    if (want > room) want = (uint32_t)room;
+    if (want > all_tiles / 4) want = all_tiles / 4;
+    if (want < 1) want = 1;
+    p.split_tiles = (all_tiles + want - 1) / want;
+    p.n_split = (all_tiles + p.split_tiles - 1) / p.split_tiles;
+    // enough workgroups to be worth it (a lone sequence with one split would leave the part idle)
+    if ((size_t)planes * p.n_split * 2 >= a.n_cu || planes * p.n_split >= p.combos * p.n_wg_tokens) {
+      p.tblocks_per_wg = (a.position_interval + 31) / 32;  // (the merge derives every row's live splits from the chunk's last token)
+      hipLaunchKernelGGL((chunk_stream_kernel<T>), dim3(planes, p.n_split), dim3(kStThreads), 0, stream, p);
+      const hipError_t e = hipGetLastError();
+      if (e != hipSuccess || p.n_split == 1) return e;
+      return merge_launch();
+    }
+  }
+
   uint32_t n_wg;
   if (p.xcd_mode) {
     const uint32_t per = 8 / p.combos;
@@ -539,14 +798,15 @@ hipError_t launch_pingpong(const AttnArgs& a, hipStream_t stream) {
   // partial rows.
   p.n_split = 1;
   p.split_tiles = 0;
-  p.part_o = a.prefill_part_o;
-  p.part_ml = a.prefill_part_ml;
   const uint32_t base = p.combos * p.n_wg_tokens;
   const uint32_t max_tiles = (a.position_index + a.position_interval - 1) / kBK + 1;
   const size_t rows = (size_t)a.position_interval * a.batch_pitch * a.n_q_heads;
   if (a.prefill_part_o && base < a.n_cu && max_tiles >= 16) {
     uint32_t want = (2 * a.n_cu + base - 1) / base;
-    const size_t room = a.prefill_part_rows / rows;   // splits the workspace holds for every row
+    // splits the workspace holds for every row (of the 256 x units rows this path was tuned with:
+    // the streaming path's larger workspace would buy a third split here, measured slower)
+    const size_t tuned = (size_t)256 * a.n_cu;
+    const size_t room = (a.prefill_part_rows < tuned ? a.prefill_part_rows : tuned) / rows;
     if (want > room) want = (uint32_t)room;
     if (want > 1) {
       uint32_t split_tiles = (max_tiles + want - 1) / want;
@@ -561,18 +821,9 @@ hipError_t launch_pingpong(const AttnArgs& a, hipStream_t stream) {
     return hipGetLastError();
   }
   hipLaunchKernelGGL((prefill_pingpong_kernel<T, true>), dim3(n_wg, p.n_split), dim3(kPpThreads), 0, stream, p);
-  hipError_t e = hipGetLastError();
+  const hipError_t e = hipGetLastError();
   if (e != hipSuccess) return e;
-  const size_t items = (size_t)a.position_interval * a.batch * a.n_q_heads * (kHeadDim / 4);
-  auto merge = [&](auto kernel, size_t lanes) {
-    hipLaunchKernelGGL(kernel, dim3((uint32_t)((items * lanes + 255) / 256)), dim3(256), 0, stream, p, a.batch);
-    return hipGetLastError();
-  };
-  // lanes per item: more when there are many splits to walk, as long as the grid stays small
-  constexpr size_t kLanesMax = (size_t)1 << 21;
-  if (p.n_split > 32 && items * 64 <= kLanesMax) return merge(prefill_merge_kernel<T, 64>, 64);
-  if (p.n_split > 8 && items * 8 <= kLanesMax) return merge(prefill_merge_kernel<T, 8>, 8);
-  return merge(prefill_merge_kernel<T, 1>, 1);
+  return merge_launch();
 }
 
 }  // namespace
@@ -583,7 +834,7 @@ size_t prefill_workspace_rows(uint32_t max_interval, uint32_t batch_capacity, ui
                               uint32_t n_cu) {
   if (max_interval < 2) return 0;  // single-token calls take the other kernel
   const size_t rows = (size_t)max_interval * batch_capacity * n_q_heads;
-  const size_t cap = (size_t)256 * n_cu;
+  const size_t cap = (size_t)512 * n_cu;
   return rows * 256 < cap ? rows * 256 : cap;
 }
 

@@ -98,7 +98,7 @@ typedef struct ellm_attn ellm_attn;
 
 /* Validates the description and allocates the operator's own workspace (split
  * partial results for the single-token path and, when max_position_interval > 1,
- * for short chunks on long caches: at most 34 MB).  Borrowed pointers are not owned. */
+ * for short chunks on long caches: at most 68 MB).  Borrowed pointers are not owned. */
 int ellm_attn_create(const ellm_attn_desc* desc, ellm_attn** out_handle);
 
 /* Frees the handle and its workspace only.  NULL is accepted. */

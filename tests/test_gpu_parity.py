@@ -47,6 +47,18 @@ PREFILL = [
     ("split_from_zero_later_splits_empty_for_early_rows", 1, 1, 8, 1, 1152, 0, 1100),
     ("split_qwen3_chunk_64_on_8k", 1, 1, 32, 4, 8320, 8192, 64),
     ("split_three_tokens_on_20k_forty_splits", 1, 1, 8, 1, 20480, 20000, 3),
+    # at most 128 query rows per K/V plane on a cache of 512 keys or more: the streaming chunk
+    # kernel (one workgroup holds all (token, head) rows of a GQA group, keys split over workgroups);
+    # the short last chunk of a prompt in the reference's serving loop, 24 sequences
+    ("stream_2tok_b24_on_tile_edge", 24, 24, 32, 4, 1200, 1024, 2),
+    ("stream_3tok_b24_off_edge", 24, 24, 32, 4, 1200, 1000, 3),
+    ("stream_16tok_b24_across_chunk_edge", 24, 24, 32, 4, 1200, 1087, 16),
+    ("stream_16tok_b24_on_chunk_edge", 24, 24, 32, 4, 1216, 1088, 16),
+    ("pingpong_33tok_b24", 24, 24, 32, 4, 1200, 1001, 33),           # 264 rows a plane: the tile kernel
+    ("stream_batch_below_capacity_9tok", 5, 3, 8, 2, 900, 700, 9),    # 36 rows: a part-filled second wave
+    ("stream_g16_8tok_full_workgroup", 1, 1, 16, 1, 3000, 2900, 8),   # 128 rows exactly
+    ("stream_first_split_only_for_early_rows", 2, 2, 8, 2, 700, 500, 5),
+    ("stream_unsplit_many_sequences", 160, 160, 32, 4, 600, 560, 16),  # no room for partial rows: one split
 ]
 
 
