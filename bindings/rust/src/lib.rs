@@ -175,6 +175,9 @@ extern "C" {
         out_handle: *mut *mut ellm_attn,
     ) -> c_int;
     pub fn ellm_attn_destroy(handle: *mut ellm_attn) -> c_int;
+    pub fn ellm_attn_reset(handle: *mut ellm_attn, stream: Stream) -> c_int;
+    pub fn ellm_matmul3_reset(handle: *mut ellm_matmul3, stream: Stream) -> c_int;
+    pub fn ellm_matmul_add_reset(handle: *mut ellm_matmul_add, stream: Stream) -> c_int;
     pub fn ellm_attn_run(
         handle: *mut ellm_attn,
         position_index: usize,

@@ -124,6 +124,9 @@ ABI_SYMBOLS = {
     "ellm_device_count": (ctypes.c_int, []),
     "ellm_attn_create": (ctypes.c_int, [ctypes.POINTER(AttnDesc), _pvp]),
     "ellm_attn_destroy": (ctypes.c_int, [_vp]),
+    "ellm_attn_reset": (ctypes.c_int, [_vp, _vp]),
+    "ellm_matmul3_reset": (ctypes.c_int, [_vp, _vp]),
+    "ellm_matmul_add_reset": (ctypes.c_int, [_vp, _vp]),
     "ellm_attn_run": (ctypes.c_int, [_vp, _sz, _sz, _sz, _vp]),
     "ellm_attn_run_ragged": (ctypes.c_int, [_vp, _vp, _sz, _sz, _vp]),
     "ellm_attn_run_noalloc": (ctypes.c_int, [ctypes.POINTER(AttnDesc), _vp, _sz, _sz, _vp]),

@@ -130,6 +130,10 @@ class Attention:
         check(self._lib.ellm_attn_run_noalloc(ctypes.byref(self.desc), pos_ptr, int(position),
                                               batch_size, _stream_ptr(stream)))
 
+    def reset(self, stream=None):
+        """Arrival counters back to zero (after a launch of this handle that did not finish)."""
+        check(self._lib.ellm_attn_reset(self._handle, _stream_ptr(stream)))
+
     def close(self):
         if self._handle:
             check(self._lib.ellm_attn_destroy(self._handle))

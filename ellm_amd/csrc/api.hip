@@ -305,6 +305,14 @@ int ellm_attn_create_ragged(const ellm_attn_desc* d, const ellm_kv_seq_table* ta
   return attn_create(d, table, out_handle);
 }
 
+int ellm_attn_reset(ellm_attn* h, void* stream) {
+  if (!h) return fail(ELLM_ERR_INVALID_ARGUMENT, "null handle");
+  if (int st = ellm::check_current_device(h->device)) return st;
+  const hipError_t e = ellm::launch_fill_u32(h->counters, h->ws.counters, 0u, (hipStream_t)stream);
+  if (e != hipSuccess) return fail_hip(e, "counter reset launch");
+  return ELLM_OK;
+}
+
 int ellm_attn_destroy(ellm_attn* h) {
   if (!h) return ELLM_OK;
   hipError_t e = free_workspace(h);

@@ -103,6 +103,8 @@ hipError_t launch_kv_append_norm_rope(void* k_dst, void* v_dst, const void* k_sr
 
 hipError_t launch_positions_advance(uint32_t* positions, uint32_t n, uint32_t by,
                                     hipStream_t stream);
+// p[i] = value for i < n: a kernel, not a memset node, so that it can be recorded into a graph.
+hipError_t launch_fill_u32(uint32_t* p, size_t n, uint32_t value, hipStream_t stream);
 
 // Projection C = X . W^T on MFMA with the per-head epilogue (see project.hip).
 // Column segment 0 (heads0 heads, weights w0) goes row-major to out0 [rows][heads0 * 128],

@@ -112,12 +112,23 @@ __global__ __launch_bounds__(256) void kv_append_norm_rope_kernel(
   }
 }
 
+__global__ void fill_u32_kernel(uint32_t* p, size_t n, uint32_t value) {
+  const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) p[i] = value;
+}
+
 __global__ void positions_advance_kernel(uint32_t* positions, uint32_t n, uint32_t by) {
   const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
   if (i < n) positions[i] += by;
 }
 
 }  // namespace
+
+hipError_t launch_fill_u32(uint32_t* p, size_t n, uint32_t value, hipStream_t stream) {
+  if (n == 0) return hipSuccess;
+  hipLaunchKernelGGL(fill_u32_kernel, dim3((uint32_t)((n + 255) / 256)), dim3(256), 0, stream, p, n, value);
+  return hipGetLastError();
+}
 
 hipError_t launch_positions_advance(uint32_t* positions, uint32_t n, uint32_t by,
                                     hipStream_t stream) {

@@ -144,6 +144,16 @@ int ellm_matmul3_create_ragged(const ellm_matmul3_desc* d, const ellm_kv_seq_tab
   return matmul3_create(d, table, out_handle);
 }
 
+int ellm_matmul3_reset(ellm_matmul3* h, void* stream) {
+  if (!h) return ellm::set_error(ELLM_ERR_INVALID_ARGUMENT, "null handle");
+  if (int st = ellm::check_current_device(h->device)) return st;
+  if (!h->counters) return ELLM_OK;
+  const hipError_t e = ellm::launch_fill_u32(h->counters, h->d.attention_head_num + 2 * h->d.kv_head_num, 0u,
+                                             (hipStream_t)stream);
+  if (e != hipSuccess) return ellm::set_error(ELLM_ERR_HIP, "counter reset launch: %s", hipGetErrorString(e));
+  return ELLM_OK;
+}
+
 int ellm_matmul3_destroy(ellm_matmul3* h) {
   if (!h) return ELLM_OK;
   const int rc = free_small_workspace(h->ws, h->counters);
@@ -253,6 +263,15 @@ int ellm_matmul_add_create(const ellm_matmul_add_desc* d, ellm_matmul_add** out_
     return rc;
   }
   *out_handle = h;
+  return ELLM_OK;
+}
+
+int ellm_matmul_add_reset(ellm_matmul_add* h, void* stream) {
+  if (!h) return ellm::set_error(ELLM_ERR_INVALID_ARGUMENT, "null handle");
+  if (int st = ellm::check_current_device(h->device)) return st;
+  if (!h->counters) return ELLM_OK;
+  const hipError_t e = ellm::launch_fill_u32(h->counters, h->d.n / 128, 0u, (hipStream_t)stream);
+  if (e != hipSuccess) return ellm::set_error(ELLM_ERR_HIP, "counter reset launch: %s", hipGetErrorString(e));
   return ELLM_OK;
 }
 

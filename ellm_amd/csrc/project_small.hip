@@ -28,12 +28,12 @@ constexpr int kRoundK = 32 * kStepsPerRound;
 __device__ __forceinline__ void store_coherent(float* p, float v) {
   __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
-// Device-coherent 16-byte load (the compiler has no 16-byte atomic load); the caller waits
-// for it (s_waitcnt vmcnt(0)) before touching the result.
-__device__ __forceinline__ f32x4 load_coherent128_nowait(const float* p) {
-  f32x4 v;
-  asm volatile("global_load_dwordx4 %0, %1, off sc1" : "=v"(v) : "v"(p) : "memory");
-  return v;
+// Device-coherent 16-byte load at byte offset `off` of a table: a buffer load with the sc1
+// cache-policy bit (what the compiler's own agent-scope atomic loads carry; it has no 16-byte
+// atomic load).  As a builtin the compiler tracks the load's completion itself.
+constexpr int kCachePolicySc1 = 16;
+__device__ __forceinline__ f32x4 load_coherent128(__amdgpu_buffer_rsrc_t table, uint32_t off) {
+  return __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(table, off, 0, kCachePolicySc1));
 }
 __device__ __forceinline__ void wait_vm_done() { __builtin_amdgcn_s_waitcnt(0x0F70); }
 
@@ -225,18 +225,18 @@ __global__ __launch_bounds__((NTB == 2 || NB == 2) ? 512 : 1024) void project_sm
   const int c8 = tid & 15;
   constexpr int kOctets = kGroupCols / 8;
   const uint32_t one_zero = M::pack2(1.0f, 0.0f);
+  // (the workspace of a handle stays far below 4 GB: byte offsets fit 32 bits)
+  const __amdgpu_buffer_rsrc_t ws_rsrc =
+      __builtin_amdgcn_make_buffer_rsrc((void*)uniform64(ws), 0, 0xffffffffu, kBufFlags);
   for (uint32_t R = tid >> 4; R < rows_cap; R += blockDim.x >> 4) {
-    const float* src =
-        ws + (((size_t)hh * kGroupsPerHead + c8 / kOctets) * rows_cap + R) * kGroupCols + 8 * (c8 % kOctets);
-    // (the two results are not to be copied or read before the wait below: the compiler takes the
-    // asm statements for ordinary instructions whose results exist at once)
-    f32x4 lo = load_coherent128_nowait(src), hi = load_coherent128_nowait(src + 4);
+    const uint32_t src = (uint32_t)(
+        ((((size_t)hh * kGroupsPerHead + c8 / kOctets) * rows_cap + R) * kGroupCols + 8 * (c8 % kOctets)) * 4);
+    const f32x4 lo = load_coherent128(ws_rsrc, src), hi = load_coherent128(ws_rsrc, src + 16);
     const uint32_t t = R / p.batch_pitch, b = R % p.batch_pitch;
     const bool live = R < p.rows && b < p.batch;
     const uint32_t pos = t + (p.positions ? (live ? min(p.positions[b], p.max_start) : 0u) : p.position_index);
     u32x4 rr = {one_zero, one_zero, one_zero, one_zero};
     if (live) rr = load16(p.rope + (size_t)pos * p.rope_pos_stride + (size_t)hs * p.rope_head_stride + 8 * c8);
-    asm volatile("s_waitcnt vmcnt(0)" : "+v"(lo), "+v"(hi), "+v"(rr));
     float o[8] = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
     float ss = 0.0f;
 #pragma unroll

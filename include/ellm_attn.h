@@ -10,7 +10,13 @@
  * All pointers named "device" are HIP device pointers.  Every function returns
  * ELLM_OK (0) or an ellm_status; nothing aborts the process.  Functions taking a
  * stream enqueue work on it and return without waiting (stream = NULL is the
- * HIP null stream).  A handle may be used from one host thread at a time.  A
+ * HIP null stream).  A handle may be used from one host thread at a time, and
+ * ONE LAUNCH OF A HANDLE MAY BE IN FLIGHT AT A TIME: a handle's workspace (split
+ * partials, arrival counters) is shared by all its runs, so runs of one handle
+ * on two streams, or two graphs recorded from one handle replayed at once, race
+ * and give wrong results; runs in stream order do not.  The arrival counters are
+ * zero between launches (the kernels put them back); a launch that was killed
+ * half-way leaves them counting, and ellm_*_reset puts them right.  A
  * handle (operator, cache, projection) belongs to the device that was current
  * when it was created: its workspace lives there, and a run or append called
  * while another device is current returns ELLM_ERR_INVALID_ARGUMENT.
@@ -104,6 +110,12 @@ int ellm_attn_create(const ellm_attn_desc* desc, ellm_attn** out_handle);
 /* Frees the handle and its workspace only.  NULL is accepted. */
 int ellm_attn_destroy(ellm_attn* handle);
 
+/* Puts the handle's arrival counters back to zero, in stream order (a small fill kernel: it
+ * may be recorded into a graph).  Only needed after a launch of this handle did not run to
+ * its end (a killed process sharing the memory, a device reset survived by the allocation);
+ * no counterpart in the reference. */
+int ellm_attn_reset(ellm_attn* handle, void* stream);
+
 /*
  * Attention::run (src/compiler/mul/attention.rs:69-76) without the cpu_num /
  * thread_id pair: queries at positions [position_index, position_index +
@@ -112,7 +124,14 @@ int ellm_attn_destroy(ellm_attn* handle);
  * position_interval == 1 takes the split-KV single-token kernel, larger
  * intervals the tiled MFMA kernel (with the key range split over workgroups and
  * a merge launch behind it when the call has too few query rows to fill the
- * device).  Zero batch_size or position_interval is a no-op returning ELLM_OK.
+ * device; calls with at most 128 query rows per K/V plane on 512 keys or more
+ * take a kernel that streams every plane once).  Zero batch_size or
+ * position_interval is a no-op returning ELLM_OK.  One run of a handle in flight
+ * at a time (see the top of this file).
+ * K/V rows at positions up to position_index + position_interval - 1 must hold finite
+ * values: a query row multiplies the value rows of the chunk's later tokens by a
+ * probability of exactly 0, and 0 x infinity is not 0 (the reference never reads them;
+ * rows beyond the call's last position are never read here either).
  */
 int ellm_attn_run(ellm_attn* handle, size_t position_index, size_t position_interval,
                   size_t batch_size, void* stream);
@@ -308,7 +327,8 @@ int ellm_schedule_calls(size_t prompt_begin, size_t prompt_end, size_t chunk, si
  * ellm_positions_advance on `stream` are recorded instead of executed; the
  * per-sequence positions live in device memory, so one recording serves every
  * step.  `stream` must be a created stream, not the null stream.  A handle
- * recorded into a graph must outlive it.
+ * recorded into a graph must outlive it, and a graph holding a handle's launches
+ * must not run at the same time as another launch of that handle (one in flight).
  */
 typedef struct ellm_graph ellm_graph;
 int ellm_graph_begin(void* stream);
@@ -388,6 +408,8 @@ int ellm_matmul3_run(ellm_matmul3* handle, size_t position_index, size_t positio
 int ellm_matmul3_run_ragged(ellm_matmul3* handle, const uint32_t* positions, size_t max_position,
                             size_t batch_size, void* stream);
 int ellm_matmul3_destroy(ellm_matmul3* handle);
+/* As ellm_attn_reset, for the counters of the few-rows kernel. */
+int ellm_matmul3_reset(ellm_matmul3* handle, void* stream);
 
 /*
  * Output projection with residual: replaces MatMulAdd::new / run
@@ -415,6 +437,7 @@ int ellm_matmul_add_create(const ellm_matmul_add_desc* desc, ellm_matmul_add** o
 int ellm_matmul_add_run(ellm_matmul_add* handle, size_t position_index, size_t position_interval,
                         size_t batch_size, void* stream);
 int ellm_matmul_add_destroy(ellm_matmul_add* handle);
+int ellm_matmul_add_reset(ellm_matmul_add* handle, void* stream);
 
 /*
  * Which projection kernel and tile shape a call with `rows` activation rows

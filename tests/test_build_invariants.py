@@ -40,3 +40,36 @@ def test_hot_kernels_do_not_spill(name, tmp_path):
     text = _listing(name, tmp_path)
     sizes = [int(x) for x in re.findall(r"\.private_segment_fixed_size:\s*(\d+)", text)]
     assert sizes and all(v == 0 for v in sizes), sizes
+
+
+def _loops(lines):
+    """(first, last) line ranges of backward branches: label ... s_cbranch to that label."""
+    labels = {}
+    for n, l in enumerate(lines):
+        m = re.match(r"^(\.LBB\d+_\d+):", l)
+        if m:
+            labels[m.group(1)] = n
+    out = []
+    for n, l in enumerate(lines):
+        m = re.match(r"\s+s_cbranch_\w+\s+(\.LBB\d+_\d+)", l)
+        if m and m.group(1) in labels and labels[m.group(1)] < n:
+            out.append((labels[m.group(1)], n))
+    return out
+
+
+@pytest.mark.parametrize("name,limit,in_loop", [("project.hip", 64, 0), ("project_small.hip", 32, 4)])
+def test_projection_kernels_keep_scratch_out_of_their_matrix_loops(name, limit, in_loop, tmp_path):
+    """The 256 x 256 tile kernel runs at 512 registers a lane and parks a few epilogue values
+    (destination rows, computed once per tile after the K loop) in scratch; the few-rows
+    kernel does the same with a handful of its finishing step's.  That is harmless only while
+    it stays a few dozen bytes and the K loop of the tile kernel never touches scratch (the
+    few-rows kernel's only loop with MFMAs is its loop over passes of 16 or 32 token rows, one
+    trip for a single-token step: at most four scratch accesses a trip)."""
+    text = _listing(name, tmp_path)
+    sizes = [int(x) for x in re.findall(r"\.private_segment_fixed_size:\s*(\d+)", text)]
+    assert sizes and max(sizes) <= limit, sizes
+    lines = [l.split(";")[0] for l in text.splitlines()]
+    for first, last in _loops(lines):
+        body = lines[first:last + 1]
+        if any("v_mfma" in l for l in body):
+            assert sum("scratch_" in l for l in body) <= in_loop, (name, first, last)
