@@ -32,8 +32,9 @@ HBM_PEAK_GBS = 8000.0       # MI355X HBM3E, published
 # copy of known size; summaries and commands under profiles/).  Not measurable from inside
 # this script; null for workloads without a counter run.
 TRAFFIC_BYTES = {
-    "decode": (264959 + 2523) * 1024,          # 16 x 8192 and 1 x 131072 dispatches averaged
-    "decode128k": (264959 + 2523) * 1024,
+    "decode": (2 * 132699 + 4372) * 1024,      # 16 x 8192
+    "decode128k": (2 * 132286 + 4489) * 1024,  # 1 x 131072
+    "lastchunk": (2 * (198584 + 18744) + 37683 + 3120) * 1024,   # 16 tokens x 24: stream kernel + merge launch
     "prefill": (1363516 + 319881) * 1024,
     "kvwrite": (73808 + 65536) * 1024,
     "qkv": (1130126 + 327680) * 1024,          # fetched past the L2s (mostly from the last-level cache) + written
@@ -931,7 +932,8 @@ def main():
             "steps": args.steps,
             "roofline": {"bound": "hbm", "achieved": round(kv_bytes / (lc[16]["kernel_ms"] * 1e-3) / 1e9, 1),
                          "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                         "frac": round(kv_bytes / (lc[16]["kernel_ms"] * 1e-3) / 1e9 / HBM_PEAK_GBS, 4), "traffic": None},
+                         "frac": round(kv_bytes / (lc[16]["kernel_ms"] * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
+                         "traffic": TRAFFIC_BYTES["lastchunk"]},
         })
 
     if args.only in ("", "mixed"):
