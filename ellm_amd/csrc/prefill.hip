@@ -443,20 +443,28 @@ __global__ __launch_bounds__(kPpThreads, 2) void prefill_pingpong_kernel(Prefill
 // matters is bytes in flight, not MFMA issue.  One workgroup = 4 waves x 32 query rows =
 // all (token, head) pairs of one GQA group (row r of the plane = token r / group, head
 // r % group), so a plane is read once; the key range is split over gridDim.y workgroups
-// (about three per compute unit, 36 KB of LDS each), which leave partial rows for
+// (two per compute unit, 36 KB of LDS each), which leave partial rows for
 // prefill_merge_kernel as the split form of the kernel above does.  Chunks of 32 keys go
 // memory -> registers -> LDS (double-buffered, one barrier a chunk, the next chunk's loads in
 // flight during the MFMAs of this one); operands and soft-max as above.
 // ---------------------------------------------------------------------------
-constexpr int kSK = 32;                        // keys per chunk
+constexpr int kSK = 32;                        // keys per compute step
 constexpr int kStThreads = 4 * kWave;
-constexpr int kStKsHalves = kSK * kKsPitch;
-constexpr int kStVsHalves = kSK * kVsPitch;
 
-// (Tried and dropped: two chunks of loads in flight per workgroup through a second set of
-// staging registers, 192 registers a wave: 16 tokens x 24 sequences on 8192 keys 94 -> 112 us.)
+// kStDepth = chunks of loads a workgroup keeps in flight, each in its own set of staging
+// registers (16 KB a chunk).  The call is bound by bytes in flight: with one chunk a workgroup
+// moves 16 KB per memory round trip, whatever else it does.  Two chunks and two workgroups
+// per compute unit measured 4-12 % faster than one chunk and three workgroups (24 sequences
+// on 8192 keys: 2 tokens 70.1 -> 67.1 us, 8 tokens 80.2 -> 73.0, 16 tokens 94.9 -> 91.2; 16
+// tokens x 16 sequences 78.4 -> 68.6); three chunks no better than two.
+constexpr int kStDepth = 2;
 template <typename T>
-__global__ __launch_bounds__(kStThreads, 3) void chunk_stream_kernel(PrefillKernelArgs p) {
+__global__ __launch_bounds__(kStThreads, 2) void chunk_stream_kernel(PrefillKernelArgs p) {
+  constexpr int DEPTH = kStDepth;
+  constexpr int kCK = kSK;                       // keys per staged chunk
+  constexpr int kStKsHalves = kCK * kKsPitch;
+  constexpr int kStVsHalves = kCK * kVsPitch;
+  constexpr int kPieces = 2;                     // 16-byte pieces of K (and of V) a thread moves per chunk
   __shared__ __attribute__((aligned(16))) uint16_t smem[2 * kStKsHalves + 2 * kStVsHalves];
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -469,7 +477,7 @@ __global__ __launch_bounds__(kStThreads, 3) void chunk_stream_kernel(PrefillKern
   if (kt0 >= all_tiles) return;  // (prefill_merge_kernel derives the live splits the same way)
   const uint32_t n_tiles = min(all_tiles - kt0, p.split_tiles);
   const uint32_t k0 = kt0 * kBK;                                   // first key of this split
-  const uint32_t n_chunks = (min(kmax + 1, k0 + n_tiles * kBK) - k0 + kSK - 1) / kSK;
+  const uint32_t n_chunks = (min(kmax + 1, k0 + n_tiles * kBK) - k0 + kCK - 1) / kCK;
 
   const uint32_t rows = S * p.group;                                // query rows of the plane, <= 128
   const uint32_t r = 32 * wave + j;
@@ -504,29 +512,31 @@ __global__ __launch_bounds__(kStThreads, 3) void chunk_stream_kernel(PrefillKern
   // at the last visible key: rows beyond it read as zeros.
   const int ld_c = tid & 15, ld_r = tid >> 4;
   const uint64_t kplane_u = uniform64(kplane), vplane_u = uniform64(vplane);
-  const uint32_t chunk_bytes = kSK * stride_pos * 2;
+  const uint32_t chunk_bytes = kCK * stride_pos * 2;
   const uint32_t valid_bytes = (kmax * stride_pos + kHeadDim) * 2;
   const uint32_t piece_off0 = (ld_r * stride_pos + 8 * ld_c) * 2;
-  const uint32_t piece_off1 = ((ld_r + 16) * stride_pos + 8 * ld_c) * 2;
-  u32x4 stg_a[4];
-  auto load_chunk = [&](uint32_t ck, u32x4 (&stg)[4]) {  // ck relative to this split's first chunk; wave-uniform
+  const uint32_t piece_step = 16 * stride_pos * 2;
+  u32x4 stg[DEPTH][2 * kPieces];
+  auto load_chunk = [&](uint32_t ck, u32x4 (&st)[2 * kPieces]) {  // ck relative to this split's first chunk; wave-uniform
     const uint32_t off = k0 * stride_pos * 2 + ck * chunk_bytes;
     const uint32_t left = valid_bytes - __builtin_amdgcn_readfirstlane(min(valid_bytes, off));
     const __amdgpu_buffer_rsrc_t kr = __builtin_amdgcn_make_buffer_rsrc((void*)(kplane_u + off), 0, left, kBufferFlags);
     const __amdgpu_buffer_rsrc_t vr = __builtin_amdgcn_make_buffer_rsrc((void*)(vplane_u + off), 0, left, kBufferFlags);
-    stg[0] = __builtin_amdgcn_raw_buffer_load_b128(kr, piece_off0, 0, 2);   // 2: non-temporal, read once
-    stg[1] = __builtin_amdgcn_raw_buffer_load_b128(kr, piece_off1, 0, 2);
-    stg[2] = __builtin_amdgcn_raw_buffer_load_b128(vr, piece_off0, 0, 2);
-    stg[3] = __builtin_amdgcn_raw_buffer_load_b128(vr, piece_off1, 0, 2);
+#pragma unroll
+    for (int i = 0; i < kPieces; ++i) {
+      st[i] = __builtin_amdgcn_raw_buffer_load_b128(kr, piece_off0 + i * piece_step, 0, 2);   // 2: non-temporal, read once
+      st[kPieces + i] = __builtin_amdgcn_raw_buffer_load_b128(vr, piece_off0 + i * piece_step, 0, 2);
+    }
   };
   const uint32_t lds0 = (uint32_t)(uintptr_t)(LdsHalf*)smem;
   const uint32_t ks_store = lds0 + 2 * (ld_r * kKsPitch + 8 * ld_c);
   const uint32_t vs_store = lds0 + 2 * (2 * kStKsHalves + ld_r * kVsPitch + 8 * ld_c);
-  auto store_chunk = [&](uint32_t buf, const u32x4 (&stg)[4]) {
-    *(LdsU32x4*)(ks_store + 2 * buf * kStKsHalves) = stg[0];
-    *(LdsU32x4*)(ks_store + 2 * (buf * kStKsHalves + 16 * kKsPitch)) = stg[1];
-    *(LdsU32x4*)(vs_store + 2 * buf * kStVsHalves) = stg[2];
-    *(LdsU32x4*)(vs_store + 2 * (buf * kStVsHalves + 16 * kVsPitch)) = stg[3];
+  auto store_chunk = [&](uint32_t buf, const u32x4 (&st)[2 * kPieces]) {
+#pragma unroll
+    for (int i = 0; i < kPieces; ++i) {
+      *(LdsU32x4*)(ks_store + 2 * (buf * kStKsHalves + 16 * i * kKsPitch)) = st[i];
+      *(LdsU32x4*)(vs_store + 2 * (buf * kStVsHalves + 16 * i * kVsPitch)) = st[kPieces + i];
+    }
   };
   // operand addresses: as in the kernel above (K rows as the A operand of S^T = K.Q^T, V through
   // the transposing read as the A operand of O^T += V^T.P^T, keys in the order P is left in)
@@ -542,7 +552,7 @@ __global__ __launch_bounds__(kStThreads, 3) void chunk_stream_kernel(PrefillKern
     for (int e = 0; e < 16; ++e) oacc[db][e] = 0.0f;
 
   auto compute = [&](uint32_t ck) __attribute__((always_inline)) {
-    const uint32_t kb = k0 + ck * kSK;
+    const uint32_t kb = k0 + ck * kCK;
     const uint32_t buf = ck & 1;
     if (wave_has_rows && kb <= wave_last_pos) {
       const uint32_t ks = k_read + 2 * buf * kStKsHalves;
@@ -601,17 +611,27 @@ __global__ __launch_bounds__(kStThreads, 3) void chunk_stream_kernel(PrefillKern
         }
     }
   };
-  load_chunk(0, stg_a);
-  store_chunk(0, stg_a);
-  if (n_chunks > 1) load_chunk(1, stg_a);
+  // chunk n travels through register set n % DEPTH; LDS is double-buffered by chunk parity
+#pragma unroll
+  for (int d = 0; d < DEPTH; ++d)
+    if ((uint32_t)d < n_chunks) load_chunk(d, stg[d]);
+  store_chunk(0, stg[0]);
+  if ((uint32_t)DEPTH < n_chunks) load_chunk(DEPTH, stg[0]);
   __syncthreads();
-  for (uint32_t ck = 0; ck < n_chunks; ++ck) {
-    compute(ck);
-    if (ck + 1 < n_chunks) {
-      store_chunk((ck & 1) ^ 1, stg_a);
-      if (ck + 2 < n_chunks) load_chunk(ck + 2, stg_a);
+  for (uint32_t ck0 = 0; ck0 < n_chunks; ck0 += DEPTH) {
+#pragma unroll
+    for (int u = 0; u < DEPTH; ++u) {
+      const uint32_t ck = ck0 + u;
+      if (ck < n_chunks) {  // (uniform over the workgroup: the barrier below is reached by all or none)
+        compute(ck);
+        if (ck + 1 < n_chunks) {
+          const int set = (u + 1) % DEPTH;
+          store_chunk((ck & 1) ^ 1, stg[set]);
+          if (ck + 1 + DEPTH < n_chunks) load_chunk(ck + 1 + DEPTH, stg[set]);
+        }
+        __syncthreads();
+      }
     }
-    __syncthreads();
   }
 
   const float l = sum_with_partner_half(l_run);
@@ -757,18 +777,15 @@ hipError_t launch_pingpong(const AttnArgs& a, hipStream_t stream) {
   };
 
   // Few query rows per plane on a cache long enough to be worth streaming: one workgroup
-  // covers all rows of a GQA group, the key range is split until there are about three
+  // covers all rows of a GQA group, the key range is split until there are two
   // workgroups per compute unit (splits of at least 256 keys), as far as the workspace holds
   // the partial rows.
   const uint32_t all_tiles = (a.position_index + a.position_interval - 1) / kBK + 1;
   const size_t all_rows = (size_t)a.position_interval * a.batch_pitch * a.n_q_heads;
   if ((size_t)a.position_interval * a.group <= 128 && all_tiles >= 8) {
     const uint32_t planes = a.batch * a.n_kv_heads;
-    // rows in one wave only: three workgroups per unit; more rows: two per unit, i.e. fewer and
-    // longer splits, less traffic of partial rows (measured, 24 sequences on 8192 keys: 2 tokens
-    // 70.7 / 75.3 us with three / two per unit, 16 tokens 108 / 94.5 us)
-    const uint32_t per_cu = (size_t)a.position_interval * a.group > 32 ? 2 : 3;
-    uint32_t want = (per_cu * a.n_cu + planes - 1) / planes;
+    // two workgroups per compute unit (with one chunk in flight three were better: see kStDepth)
+    uint32_t want = 2 * a.n_cu / planes;
     const size_t room = a.prefill_part_o ? a.prefill_part_rows / all_rows : 1;
     if (want > room) want = (uint32_t)room;
     if (want > all_tiles / 4) want = all_tiles / 4;
