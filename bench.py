@@ -917,12 +917,12 @@ def main():
         # the reference's serving loop ends a prompt with a chunk of (prompt % 64) positions x 24 sequences
         # (src/serving/start copy.rs:71-101): few query rows per K/V plane over thousands of cached tokens
         lc_dec = bench_decode(24, 8192, args.steps, min(args.warmup, 5), copies=3)
-        lc = {t: bench_prefill(t, args.steps, min(args.warmup, 5), p0=8192, batch=24, copies=3) for t in (2, 8, 16, 33)}
+        lc = {t: bench_prefill(t, args.steps, min(args.warmup, 5), p0=8192, batch=24, copies=3) for t in (2, 8, 16, 24, 33, 48)}
         kv_bytes = 2 * 24 * 4 * 8192 * D * 2
         also.append({
-            "workload": "short last chunk of a prompt: 2 / 8 / 16 / 33 new tokens x 24 sequences on 8192-token caches, "
-                        "32q/4kv heads, fp16 (up to 16 tokens: the streaming chunk kernel, one workgroup per GQA "
-                        "group's rows, keys split over workgroups + merge launch; 33 tokens: the tile kernel); "
+            "workload": "short last chunk of a prompt: 2 / 8 / 16 / 24 / 33 / 48 new tokens x 24 sequences on 8192-token "
+                        "caches, 32q/4kv heads, fp16 (the streaming chunk kernel: one workgroup of 4, 8 or 12 waves "
+                        "per GQA group's rows, up to 16, 32 or 48 tokens, keys split over workgroups + merge launch); "
                         "beside it the single-token kernel on the same caches",
             "metric": "chunk attention us per call", "unit": "us",
             "value": round(lc[16]["ms_per_step"] * 1e3, 1),

@@ -22,6 +22,7 @@
 // and keeps the token span (and so the masked part of the diagonal tile) short.
 #include <type_traits>
 
+#include "chunk_plan.hpp"
 #include "common.hpp"
 #include "kernels.hpp"
 
@@ -449,7 +450,7 @@ __global__ __launch_bounds__(kPpThreads, 2) void prefill_pingpong_kernel(Prefill
 // flight during the MFMAs of this one); operands and soft-max as above.
 // ---------------------------------------------------------------------------
 constexpr int kSK = 32;                        // keys per compute step
-constexpr int kStThreads = 4 * kWave;
+constexpr int kStStagersMax = 8 * kWave;       // one 16-byte piece of K and of V each moves a whole chunk
 
 // kStDepth = chunks of loads a workgroup keeps in flight, each in its own set of staging
 // registers (16 KB a chunk).  The call is bound by bytes in flight: with one chunk a workgroup
@@ -458,13 +459,20 @@ constexpr int kStThreads = 4 * kWave;
 // on 8192 keys: 2 tokens 70.1 -> 67.1 us, 8 tokens 80.2 -> 73.0, 16 tokens 94.9 -> 91.2; 16
 // tokens x 16 sequences 78.4 -> 68.6); three chunks no better than two.
 constexpr int kStDepth = 2;
-template <typename T>
-__global__ __launch_bounds__(kStThreads, 2) void chunk_stream_kernel(PrefillKernelArgs p) {
+// WAVES = 4, 8 or 12 waves of 32 query rows each: up to 128, 256 or 384 rows of a plane (16, 32
+// or 48 tokens of a sequence with eight heads a group).  Four waves leave room for two
+// workgroups a compute unit; eight and twelve fill a unit with one.
+template <typename T, int WAVES>
+__global__ __launch_bounds__(WAVES * kWave, WAVES == 4 ? 2 : 1) void chunk_stream_kernel(PrefillKernelArgs p) {
   constexpr int DEPTH = kStDepth;
+  constexpr int kThreads = WAVES * kWave;
+  constexpr int kStagers = kThreads < kStStagersMax ? kThreads : kStStagersMax;  // threads that move K/V
   constexpr int kCK = kSK;                       // keys per staged chunk
   constexpr int kStKsHalves = kCK * kKsPitch;
   constexpr int kStVsHalves = kCK * kVsPitch;
-  constexpr int kPieces = 2;                     // 16-byte pieces of K (and of V) a thread moves per chunk
+  constexpr int kPieces = kCK * 16 / kStagers;   // 16-byte pieces of K (and of V) a staging thread moves per chunk
+  constexpr int kPieceRows = kStagers / 16;      // rows between a thread's pieces
+  static_assert(kPieces * kStagers == kCK * 16, "the staging threads must tile a chunk");
   __shared__ __attribute__((aligned(16))) uint16_t smem[2 * kStKsHalves + 2 * kStVsHalves];
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -479,7 +487,7 @@ __global__ __launch_bounds__(kStThreads, 2) void chunk_stream_kernel(PrefillKern
   const uint32_t k0 = kt0 * kBK;                                   // first key of this split
   const uint32_t n_chunks = (min(kmax + 1, k0 + n_tiles * kBK) - k0 + kCK - 1) / kCK;
 
-  const uint32_t rows = S * p.group;                                // query rows of the plane, <= 128
+  const uint32_t rows = S * p.group;                                // query rows of the plane, <= 32 WAVES
   const uint32_t r = 32 * wave + j;
   const bool row_valid = r < rows;
   const uint32_t rc = row_valid ? r : rows - 1;
@@ -507,17 +515,19 @@ __global__ __launch_bounds__(kStThreads, 2) void chunk_stream_kernel(PrefillKern
   const uint16_t* kplane = p.k + plane_at;
   const uint16_t* vplane = p.v + plane_at;
   const uint32_t stride_pos = (uint32_t)p.kv_stride_pos;
-  // staging: 256 threads move one 32 x 128 chunk of K and one of V, two 16-byte pieces of each
-  // (rows ld_r and ld_r + 16, columns 8 ld_c ..), through buffer loads whose descriptor ends
-  // at the last visible key: rows beyond it read as zeros.
-  const int ld_c = tid & 15, ld_r = tid >> 4;
+  // staging: the first 256 or 512 threads move one 32 x 128 chunk of K and one of V, two or one
+  // 16-byte pieces of each (rows ld_r + 16 i or row ld_r, columns 8 ld_c ..), through buffer loads
+  // whose descriptor ends at the last visible key: rows beyond it read as zeros.
+  const bool stager = kThreads == kStagers || __builtin_amdgcn_readfirstlane(wave) < kStagers / kWave;
+  const int ld_c = tid & 15, ld_r = (tid >> 4) & (kPieceRows - 1);
   const uint64_t kplane_u = uniform64(kplane), vplane_u = uniform64(vplane);
   const uint32_t chunk_bytes = kCK * stride_pos * 2;
   const uint32_t valid_bytes = (kmax * stride_pos + kHeadDim) * 2;
   const uint32_t piece_off0 = (ld_r * stride_pos + 8 * ld_c) * 2;
-  const uint32_t piece_step = 16 * stride_pos * 2;
+  const uint32_t piece_step = kPieceRows * stride_pos * 2;
   u32x4 stg[DEPTH][2 * kPieces];
   auto load_chunk = [&](uint32_t ck, u32x4 (&st)[2 * kPieces]) {  // ck relative to this split's first chunk; wave-uniform
+    if (!stager) return;
     const uint32_t off = k0 * stride_pos * 2 + ck * chunk_bytes;
     const uint32_t left = valid_bytes - __builtin_amdgcn_readfirstlane(min(valid_bytes, off));
     const __amdgpu_buffer_rsrc_t kr = __builtin_amdgcn_make_buffer_rsrc((void*)(kplane_u + off), 0, left, kBufferFlags);
@@ -532,10 +542,11 @@ __global__ __launch_bounds__(kStThreads, 2) void chunk_stream_kernel(PrefillKern
   const uint32_t ks_store = lds0 + 2 * (ld_r * kKsPitch + 8 * ld_c);
   const uint32_t vs_store = lds0 + 2 * (2 * kStKsHalves + ld_r * kVsPitch + 8 * ld_c);
   auto store_chunk = [&](uint32_t buf, const u32x4 (&st)[2 * kPieces]) {
+    if (!stager) return;
 #pragma unroll
     for (int i = 0; i < kPieces; ++i) {
-      *(LdsU32x4*)(ks_store + 2 * (buf * kStKsHalves + 16 * i * kKsPitch)) = st[i];
-      *(LdsU32x4*)(vs_store + 2 * (buf * kStVsHalves + 16 * i * kVsPitch)) = st[kPieces + i];
+      *(LdsU32x4*)(ks_store + 2 * (buf * kStKsHalves + kPieceRows * i * kKsPitch)) = st[i];
+      *(LdsU32x4*)(vs_store + 2 * (buf * kStVsHalves + kPieceRows * i * kVsPitch)) = st[kPieces + i];
     }
   };
   // operand addresses: as in the kernel above (K rows as the A operand of S^T = K.Q^T, V through
@@ -782,20 +793,44 @@ hipError_t launch_pingpong(const AttnArgs& a, hipStream_t stream) {
   // the partial rows.
   const uint32_t all_tiles = (a.position_index + a.position_interval - 1) / kBK + 1;
   const size_t all_rows = (size_t)a.position_interval * a.batch_pitch * a.n_q_heads;
-  if ((size_t)a.position_interval * a.group <= 128 && all_tiles >= 8) {
+  const size_t plane_rows = (size_t)a.position_interval * a.group;
+  if (plane_rows <= 384 && all_tiles >= 8) {
     const uint32_t planes = a.batch * a.n_kv_heads;
-    // two workgroups per compute unit (with one chunk in flight three were better: see kStDepth)
-    uint32_t want = 2 * a.n_cu / planes;
+    // workgroups of four waves: two per compute unit (with one chunk in flight three were
+    // better: see kStDepth); of eight or twelve waves: one.  Pieces of at least four tiles.
+    const uint32_t waves = plane_rows <= 128 ? 4 : plane_rows <= 256 ? 8 : 12;
+    const uint32_t slots = (waves == 4 ? 2 : 1) * a.n_cu;
     const size_t room = a.prefill_part_o ? a.prefill_part_rows / all_rows : 1;
-    if (want > room) want = (uint32_t)room;
-    if (want > all_tiles / 4) want = all_tiles / 4;
-    if (want < 1) want = 1;
-    p.split_tiles = (all_tiles + want - 1) / want;
-    p.n_split = (all_tiles + p.split_tiles - 1) / p.split_tiles;
+    // a workgroup's time per tile (us, measured on 24 sequences x 8192 keys), and what one more
+    // partial row per query row costs: written and read once, at about 4 TB/s
+    const double tile_us = waves == 8 ? 2.0 : 2.5;
+    const double split_us = (double)a.position_interval * a.batch * a.n_q_heads * (kHeadDim + 2) * 8 / 4e6;
+    const uint32_t max_split = (uint32_t)(room < 4096 ? room : 4096);
+    if (waves == 4) {
+      // Two workgroups share a compute unit's throughput, so a slot that opens early is not
+      // spare capacity: equal pieces, never more workgroups than slots (24 sequences on 8192
+      // keys, 2 / 8 tokens: 67.6 / 73.1 us; as 5 pieces of 25 tiles and one of 4: 70.1 / 78.9)
+      uint32_t want = slots / planes;
+      if (want > max_split) want = max_split;
+      if (want > all_tiles / 4) want = all_tiles / 4;
+      if (want < 1) want = 1;
+      p.split_tiles = (all_tiles + want - 1) / want;
+      p.n_split = (all_tiles + p.split_tiles - 1) / p.split_tiles;
+    } else {
+      const KeySplit ks = plan_key_split(all_tiles, planes, slots, 4, max_split, split_us / tile_us);
+      p.split_tiles = ks.split_tiles;
+      p.n_split = ks.n_split;
+    }
     // enough workgroups to be worth it (a lone sequence with one split would leave the part idle)
     if ((size_t)planes * p.n_split * 2 >= a.n_cu || planes * p.n_split >= p.combos * p.n_wg_tokens) {
       p.tblocks_per_wg = (a.position_interval + 31) / 32;  // (the merge derives every row's live splits from the chunk's last token)
-      hipLaunchKernelGGL((chunk_stream_kernel<T>), dim3(planes, p.n_split), dim3(kStThreads), 0, stream, p);
+      const dim3 grid(planes, p.n_split);
+      if (waves == 4)
+        hipLaunchKernelGGL((chunk_stream_kernel<T, 4>), grid, dim3(4 * kWave), 0, stream, p);
+      else if (waves == 8)
+        hipLaunchKernelGGL((chunk_stream_kernel<T, 8>), grid, dim3(8 * kWave), 0, stream, p);
+      else
+        hipLaunchKernelGGL((chunk_stream_kernel<T, 12>), grid, dim3(12 * kWave), 0, stream, p);
       const hipError_t e = hipGetLastError();
       if (e != hipSuccess || p.n_split == 1) return e;
       return merge_launch();
@@ -809,27 +844,28 @@ hipError_t launch_pingpong(const AttnArgs& a, hipStream_t stream) {
   } else {
     n_wg = p.combos * p.n_wg_tokens;
   }
-  // Few row blocks on a long cache: split the key range until there are about two
-  // workgroups per compute unit (four measured no faster), a split no shorter than eight
-  // tiles (each pays the pipeline's first and last step), as far as the workspace holds the
-  // partial rows.
+  // Few row blocks on a long cache: split the key range over more workgroups, as far as the
+  // workspace holds the partial rows (plan_key_split weighs the longest chain of pieces a
+  // compute unit runs against the partial rows every piece adds).
   p.n_split = 1;
   p.split_tiles = 0;
   const uint32_t base = p.combos * p.n_wg_tokens;
   const uint32_t max_tiles = (a.position_index + a.position_interval - 1) / kBK + 1;
   const size_t rows = (size_t)a.position_interval * a.batch_pitch * a.n_q_heads;
-  if (a.prefill_part_o && base < a.n_cu && max_tiles >= 16) {
-    uint32_t want = (2 * a.n_cu + base - 1) / base;
-    // splits the workspace holds for every row (of the 256 x units rows this path was tuned with:
-    // the streaming path's larger workspace would buy a third split here, measured slower)
-    const size_t tuned = (size_t)256 * a.n_cu;
-    const size_t room = (a.prefill_part_rows < tuned ? a.prefill_part_rows : tuned) / rows;
-    if (want > room) want = (uint32_t)room;
-    if (want > 1) {
-      uint32_t split_tiles = (max_tiles + want - 1) / want;
-      if (split_tiles < 8) split_tiles = 8;
-      p.split_tiles = split_tiles;
-      p.n_split = (max_tiles + split_tiles - 1) / split_tiles;
+  // Only while the unsplit launch leaves at least half of the compute units idle: with more
+  // of them busy the part runs this kernel at its power limit, idle units or not, and a split
+  // only adds the partial rows (64 tokens x 24 sequences on 8192 keys, 192 workgroups: 229 us
+  // unsplit, 235 us as pieces of 97 + 32 tiles on all 256 units).
+  if (a.prefill_part_o && 2 * base <= a.n_cu && max_tiles >= 16) {
+    // pieces of at least eight tiles (each pays the pipeline's first and last step); 1.9 us a
+    // tile and workgroup (measured, 64 tokens x 24 sequences on 8192 keys)
+    const size_t room = a.prefill_part_rows / rows;
+    const double split_us = (double)a.position_interval * a.batch * a.n_q_heads * (kHeadDim + 2) * 8 / 4e6;
+    const KeySplit ks = plan_key_split(max_tiles, base, a.n_cu, 8, (uint32_t)(room < 4096 ? room : 4096),
+                                       split_us / 1.9);
+    if (ks.n_split > 1) {
+      p.split_tiles = ks.split_tiles;
+      p.n_split = ks.n_split;
     }
   }
   if (p.n_split <= 1) {
@@ -845,8 +881,8 @@ hipError_t launch_pingpong(const AttnArgs& a, hipStream_t stream) {
 
 }  // namespace
 
-// The key range is split only while the unsplit launch has fewer workgroups than compute
-// units, i.e. at most 256 n_cu query rows, and then into at most ~n_cu workgroups in all.
+// Partial rows (128 + 2 floats each) a handle keeps for calls whose key range is split: 256
+// splits of every row it can be asked for, at most 512 per compute unit (68 MB on 256 units).
 size_t prefill_workspace_rows(uint32_t max_interval, uint32_t batch_capacity, uint32_t n_q_heads,
                               uint32_t n_cu) {
   if (max_interval < 2) return 0;  // single-token calls take the other kernel

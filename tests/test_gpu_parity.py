@@ -54,7 +54,14 @@ PREFILL = [
     ("stream_3tok_b24_off_edge", 24, 24, 32, 4, 1200, 1000, 3),
     ("stream_16tok_b24_across_chunk_edge", 24, 24, 32, 4, 1200, 1087, 16),
     ("stream_16tok_b24_on_chunk_edge", 24, 24, 32, 4, 1216, 1088, 16),
-    ("pingpong_33tok_b24", 24, 24, 32, 4, 1200, 1001, 33),           # 264 rows a plane: the tile kernel
+    # 129-256 and 257-384 rows a plane: the same kernel with eight and twelve waves
+    ("stream_17tok_b24_eight_waves", 24, 24, 32, 4, 1200, 1001, 17),
+    ("stream_32tok_b24_eight_waves_full", 24, 24, 32, 4, 1200, 1056, 32),
+    ("stream_33tok_b24_twelve_waves", 24, 24, 32, 4, 1200, 1001, 33),
+    ("stream_48tok_b6_twelve_waves_full", 6, 6, 32, 4, 1200, 1087, 48),
+    ("stream_g16_20tok_twelve_waves_below_capacity", 3, 2, 16, 1, 900, 700, 20),
+    ("stream_g3_50tok_eight_waves_odd_group", 2, 2, 6, 2, 800, 600, 50),
+    ("pingpong_49tok_b24", 24, 24, 32, 4, 1200, 1001, 49),           # 392 rows a plane: the tile kernel
     ("stream_batch_below_capacity_9tok", 5, 3, 8, 2, 900, 700, 9),    # 36 rows: a part-filled second wave
     ("stream_g16_8tok_full_workgroup", 1, 1, 16, 1, 3000, 2900, 8),   # 128 rows exactly
     ("stream_first_split_only_for_early_rows", 2, 2, 8, 2, 700, 500, 5),
