@@ -159,11 +159,16 @@ __global__ __launch_bounds__((NTB == 2 || NB == 2) ? 512 : 1024) void project_sm
       __syncthreads();  // the sums reuse the rows' LDS
     }
     // the weight operands stay in registers; the token rows of the next pass are requested
-    // before those of this one are used
+    // before those of this one are used, where the registers are there for them (a second set
+    // of token rows in the widest forms would not fit, and a kernel that spills, by however
+    // little, pays several microseconds a launch for its scratch memory to be set up)
+    constexpr bool kAhead = NTB == 1 && !(MODE == kModeQkv && NB == 1);
     for (uint32_t pass = 0; pass < passes; ++pass) {
-      u32x4 xnext[NTB][kStepsPerRound];
+      u32x4 xnext[kAhead ? NTB : 1][kAhead ? kStepsPerRound : 1];
       const bool more = pass + 1 < passes;  // (uniform)
-      if (more) fetch_x(xnext, pass + 1, k_first);
+      if constexpr (kAhead) {
+        if (more) fetch_x(xnext, pass + 1, k_first);
+      }
       f32x4 acc[kColBlocks][NTB];
 #pragma unroll
       for (int nb = 0; nb < kColBlocks; ++nb)
@@ -175,13 +180,18 @@ __global__ __launch_bounds__((NTB == 2 || NB == 2) ? 512 : 1024) void project_sm
         for (int nb = 0; nb < kColBlocks; ++nb)
 #pragma unroll
           for (int tb = 0; tb < NTB; ++tb) acc[nb][tb] = M::m16x16x32(wreg[nb][s], xcur[tb][s], acc[nb][tb]);
+      if constexpr (!kAhead) {
+        if (more) fetch_x(xcur, pass + 1, k_first);
+      }
       finish_pass(pass, acc);
       if (more) {
         __syncthreads();  // the sums are rewritten by the next pass
+        if constexpr (kAhead) {
 #pragma unroll
-        for (int tb = 0; tb < NTB; ++tb)
+          for (int tb = 0; tb < NTB; ++tb)
 #pragma unroll
-          for (int s = 0; s < kStepsPerRound; ++s) xcur[tb][s] = xnext[tb][s];
+            for (int s = 0; s < kStepsPerRound; ++s) xcur[tb][s] = xnext[tb][s];
+        }
       }
     }
   } else {
