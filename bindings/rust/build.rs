@@ -27,9 +27,10 @@ fn main() {
     // so that binaries find the library without LD_LIBRARY_PATH
     println!("cargo:rustc-link-arg=-Wl,-rpath,{}", lib_dir.display());
     for f in [
-        "api.hip", "noalloc.hip", "decode.hip", "prefill.hip", "kv_cache.hip", "project.hip",
-        "project_mid.hip", "project_small.hip", "project_api.hip", "common.hpp", "kernels.hpp",
-        "project_common.hpp", "project_epilogue.hpp", "Makefile",
+        "api.hip", "noalloc.hip", "decode.hip", "decode_balanced.hip", "prefill.hip", "kv_cache.hip",
+        "project.hip", "project_mid.hip", "project_small.hip", "project_api.hip", "common.hpp",
+        "kernels.hpp", "decode_common.hpp", "chunk_plan.hpp", "project_common.hpp",
+        "project_epilogue.hpp", "Makefile",
     ] {
         println!("cargo:rerun-if-changed={}", csrc.join(f).display());
     }

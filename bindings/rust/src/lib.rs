@@ -192,6 +192,7 @@ extern "C" {
         batch_size: usize,
         stream: Stream,
     ) -> c_int;
+    pub fn ellm_attn_ragged_path(handle: *const ellm_attn, max_position: usize, batch_size: usize) -> c_int;
     pub fn ellm_attn_run_noalloc(
         desc: *const ellm_attn_desc,
         positions: *const u32,

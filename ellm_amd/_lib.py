@@ -129,6 +129,7 @@ ABI_SYMBOLS = {
     "ellm_matmul_add_reset": (ctypes.c_int, [_vp, _vp]),
     "ellm_attn_run": (ctypes.c_int, [_vp, _sz, _sz, _sz, _vp]),
     "ellm_attn_run_ragged": (ctypes.c_int, [_vp, _vp, _sz, _sz, _vp]),
+    "ellm_attn_ragged_path": (ctypes.c_int, [_vp, _sz, _sz]),
     "ellm_attn_run_noalloc": (ctypes.c_int, [ctypes.POINTER(AttnDesc), _vp, _sz, _sz, _vp]),
     "ellm_kv_create": (ctypes.c_int, [ctypes.POINTER(KvDesc), _pvp]),
     "ellm_kv_create_ragged": (ctypes.c_int, [ctypes.POINTER(KvRaggedDesc), _pvp]),

@@ -123,6 +123,14 @@ class Attention:
         check(self._lib.ellm_attn_run_ragged(self._handle, _positions_ptr(positions, batch_size),
                                              int(max_position), batch_size, _stream_ptr(stream)))
 
+    def ragged_path(self, max_position, batch_size):
+        """Which kernel run_ragged takes for this call: 0 = every plane split alike, 1 = the keys
+        of all planes dealt evenly to the workgroups (ellm_attn_ragged_path)."""
+        path = self._lib.ellm_attn_ragged_path(self._handle, int(max_position), batch_size)
+        if path < 0:
+            check(-path)
+        return path
+
     def run_noalloc(self, position, batch_size, positions=None, stream=None):
         """The single-token step through ellm_attn_run_noalloc: this operator's description,
         the library's static device scratch instead of the handle's workspace."""

@@ -336,7 +336,22 @@ static void fill_args(const ellm_attn* h, ellm::AttnArgs* a) {
   a->seq_caps = h->seq_caps;
 }
 
+// sequences of different lengths: equal shares of all keys, two workgroups per compute unit
+static bool takes_balanced(const ellm_attn* h, size_t batch, size_t max_position, uint32_t* wgs) {
+  *wgs = 2 * (uint32_t)h->n_cu;
+  const ellm_attn_desc& d = h->desc;
+  return ellm::decode_balanced_takes(h->ws, (uint32_t)batch, (uint32_t)d.kv_head_num,
+                                     (uint32_t)(d.attention_head_num / d.kv_head_num),
+                                     (uint32_t)max_position + 1, *wgs);
+}
+
 static int run_decode(ellm_attn* h, ellm::AttnArgs* a, uint32_t max_position, hipStream_t stream) {
+  uint32_t wgs = 0;
+  if (a->positions && takes_balanced(h, a->batch, max_position, &wgs)) {
+    const hipError_t e = ellm::launch_decode_balanced(*a, wgs, stream);
+    if (e != hipSuccess) return fail_hip(e, "single-token attention launch");
+    return ELLM_OK;
+  }
   const ellm::DecodePlan plan =
       ellm::decode_plan(max_position + 1, a->batch, a->n_kv_heads, (uint32_t)h->n_cu);
   a->split_len = plan.split_len;
@@ -400,6 +415,15 @@ int ellm_attn_run_ragged(ellm_attn* h, const uint32_t* positions, size_t max_pos
   a.batch = (uint32_t)batch_size;
   a.positions = positions;
   return run_decode(h, &a, (uint32_t)max_position, (hipStream_t)stream);
+}
+
+int ellm_attn_ragged_path(const ellm_attn* h, size_t max_position, size_t batch_size) {
+  if (!h) return -fail(ELLM_ERR_INVALID_ARGUMENT, "null handle");
+  if (batch_size == 0 || batch_size > h->desc.batch_size || max_position >= h->desc.sequence_capacity)
+    return -fail(ELLM_ERR_OUT_OF_RANGE, "batch_size %zu / max_position %zu outside the handle's %zu / %zu",
+                 batch_size, max_position, h->desc.batch_size, h->desc.sequence_capacity);
+  uint32_t wgs = 0;
+  return takes_balanced(h, batch_size, max_position, &wgs) ? 1 : 0;
 }
 
 /* ---- K/V cache ---------------------------------------------------------- */

@@ -75,6 +75,11 @@ bool decode_plan_fits(const DecodeWorkspace& w, uint32_t batch, uint32_t n_q_hea
                       uint32_t n_kv_heads, uint32_t group, uint32_t n_split);
 
 hipError_t launch_decode(const AttnArgs& a, hipStream_t stream);
+// Per-sequence positions, the planes' keys dealt evenly to `wgs` workgroups (decode_balanced.hip):
+// whether a call of this shape goes there, and the launch (a.positions must be set).
+bool decode_balanced_takes(const DecodeWorkspace& w, uint32_t batch, uint32_t n_kv_heads, uint32_t group,
+                           uint32_t max_len, uint32_t wgs);
+hipError_t launch_decode_balanced(const AttnArgs& a, uint32_t wgs, hipStream_t stream);
 hipError_t launch_prefill(const AttnArgs& a, hipStream_t stream);
 
 // Where the rows of a cache layer live: plane of (sequence, head) at

@@ -148,6 +148,17 @@ int ellm_attn_run_ragged(ellm_attn* handle, const uint32_t* positions, size_t ma
                          size_t batch_size, void* stream);
 
 /*
+ * Which kernel ellm_attn_run_ragged runs for a call with this max_position and batch_size
+ * on this handle: 0 = the single-token kernel of ellm_attn_run (every K/V plane split alike,
+ * sized for max_position), 1 = the kernel that deals the keys of all planes to the workgroups
+ * in equal shares, whatever the sequences' lengths (taken when the call is large enough for
+ * the split to matter); negative: a status code (null handle, arguments out of range).  No
+ * counterpart in the reference (its Attention::run has one code path); it lets a test or a
+ * harness see which kernel its shapes reach.
+ */
+int ellm_attn_ragged_path(const ellm_attn* handle, size_t max_position, size_t batch_size);
+
+/*
  * The single-token step of ellm_attn_run / ellm_attn_run_ragged (position_interval == 1)
  * without a handle and without any allocation.  No counterpart in the reference: it is
  * for callers that cannot call hipMalloc — code under HIP graph capture, tight serving

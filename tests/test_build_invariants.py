@@ -35,7 +35,7 @@ def test_one_head_tile_kernels_leave_m0_to_the_inline_asm(tmp_path):
     assert not any("movrel" in l or "s_set_gpr_idx" in l for l in code)
 
 
-@pytest.mark.parametrize("name", ["project_mid.hip", "project_small.hip", "prefill.hip", "decode.hip"])
+@pytest.mark.parametrize("name", ["project_mid.hip", "project_small.hip", "prefill.hip", "decode.hip", "decode_balanced.hip"])
 def test_hot_kernels_do_not_spill(name, tmp_path):
     text = _listing(name, tmp_path)
     sizes = [int(x) for x in re.findall(r"\.private_segment_fixed_size:\s*(\d+)", text)]

@@ -1,7 +1,9 @@
 """ellm_attn_run_noalloc (the single-token step on the library's static device scratch, for
 callers that cannot allocate) against ellm_attn_run / ellm_attn_run_ragged (the same step on
 a handle's own workspace): same kernel, same split plan, so the outputs and the log-sum-exp
-must be equal bit for bit.  Two calls in a row share the static scratch; the second is
+must be equal bit for bit (the calls with per-sequence positions here are small, so the handle
+keeps the kernel the no-alloc entry point always uses; large ones go to the handle's kernel for
+sequences of different lengths, which splits the keys differently).  Two calls in a row share the static scratch; the second is
 smaller, so whatever the first one left behind (partials, counters) must not show.
 Also checked against the CPU oracle within the operator's tolerance."""
 import numpy as np
