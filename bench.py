@@ -34,7 +34,8 @@ HBM_PEAK_GBS = 8000.0       # MI355X HBM3E, published
 TRAFFIC_BYTES = {
     "decode": (2 * 132699 + 4372) * 1024,      # 16 x 8192
     "decode128k": (2 * 132286 + 4489) * 1024,  # 1 x 131072
-    "lastchunk": (2 * (198584 + 18744) + 37683 + 3120) * 1024,   # 16 tokens x 24: stream kernel + merge launch
+    "lastchunk": (2 * (198592 + 15674) + 31309 + 3120) * 1024,   # 16 tokens x 24: stream kernel + merge launch
+    "mixed_decode": (2 * 2258263 + 5415) * 1024,                 # 32 sequences U{1024..131072}, seed 7
     "prefill": (1363516 + 319881) * 1024,
     "kvwrite": (73808 + 65536) * 1024,
     "qkv": (1130126 + 327680) * 1024,          # fetched past the L2s (mostly from the last-level cache) + written
@@ -971,7 +972,8 @@ def main():
                 msp["qkv_bytes"] / (msp["qkv_kernel_ms"] * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
             "roofline": {"bound": "hbm", "achieved": round(md["kernel_gbs"], 1),
                          "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                         "frac": round(md["kernel_gbs"] / HBM_PEAK_GBS, 4), "traffic": None},
+                         "frac": round(md["kernel_gbs"] / HBM_PEAK_GBS, 4),
+                         "traffic": TRAFFIC_BYTES["mixed_decode"]},
             "cpu_baseline": mx_cpu,
         })
 

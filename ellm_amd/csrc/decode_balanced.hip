@@ -48,42 +48,64 @@ __global__ __launch_bounds__(kDecThreads, 2) void decode_balanced_kernel(DecodeK
     if (p.seq_caps) pos = min(pos, p.seq_caps[b] - 1);
     return pos;
   };
-  if (t.wave == 0) {
-    uint32_t carry = 0, umax = 0;
-    for (uint32_t base = 0; base < B; base += kWave) {
-      const bool live = base + t.lane < B;
-      const uint32_t pos_b = live ? position_of(base + t.lane) : 0u;
-      if (live) s_pos[base + t.lane] = pos_b;
-      const uint32_t u = live ? pos_b / kUnitKeys + 1 : 0u;
-      uint32_t incl = u;
+  // Units per sequence and their running sum.  Up to 64 sequences: every wave keeps them in
+  // registers, sequence b in lane b (no LDS, no barrier, and the look-up below is a ballot);
+  // more: wave 0 scans them into LDS, 64 at a time.
+  auto wave_scan = [&](uint32_t v) {   // inclusive sum over the lanes below and this one
 #pragma unroll
-      for (int d = 1; d < kWave; d <<= 1) {
-        const uint32_t below = __shfl_up(incl, d, kWave);
-        if (t.lane >= d) incl += below;
+    for (int d = 1; d < kWave; d <<= 1) {
+      const uint32_t below = __shfl_up(v, d, kWave);
+      if (t.lane >= d) v += below;
+    }
+    return v;
+  };
+  auto wave_max = [&](uint32_t v) {
+#pragma unroll
+    for (int d = 1; d < kWave; d <<= 1) v = max(v, (uint32_t)__shfl_xor(v, d, kWave));
+    return v;
+  };
+  auto lane_value = [&](uint32_t v, uint32_t l) { return (uint32_t)__builtin_amdgcn_readlane((int)v, (int)l); };
+  const bool in_registers = B <= (uint32_t)kWave;   // (uniform)
+  uint32_t r_pos = 0, r_units = 0, r_incl = 0, total_units, umax_all;
+  if (in_registers) {
+    const bool live = (uint32_t)t.lane < B;
+    r_pos = live ? position_of(t.lane) : 0u;
+    r_units = live ? r_pos / kUnitKeys + 1 : 0u;
+    r_incl = wave_scan(r_units);
+    total_units = lane_value(r_incl, kWave - 1);
+    umax_all = uni(wave_max(r_units));
+  } else {
+    if (t.wave == 0) {
+      uint32_t carry = 0, umax = 0;
+      for (uint32_t base = 0; base < B; base += kWave) {
+        const bool live = base + t.lane < B;
+        const uint32_t pos_b = live ? position_of(base + t.lane) : 0u;
+        if (live) s_pos[base + t.lane] = pos_b;
+        const uint32_t u = live ? pos_b / kUnitKeys + 1 : 0u;
+        const uint32_t incl = wave_scan(u);
+        if (live) prefix[base + t.lane + 1] = carry + incl;
+        carry += __shfl(incl, kWave - 1, kWave);
+        umax = max(umax, wave_max(u));
       }
-      if (live) prefix[base + t.lane + 1] = carry + incl;
-      carry += __shfl(incl, kWave - 1, kWave);
-      uint32_t m = u;
-#pragma unroll
-      for (int d = 1; d < kWave; d <<= 1) m = max(m, (uint32_t)__shfl_xor(m, d, kWave));
-      umax = max(umax, m);
+      if (t.lane == 0) {
+        prefix[0] = 0;
+        s_umax = umax;
+      }
     }
-    if (t.lane == 0) {
-      prefix[0] = 0;
-      s_umax = umax;
-    }
+    __syncthreads();
+    total_units = uni(prefix[B]);
+    umax_all = uni(s_umax);
   }
-  __syncthreads();
 
   // All of the index arithmetic is 32-bit (the launcher keeps calls with 2^31 units or more
   // away): a 64-bit division is a subroutine of a few hundred instructions, and a handful of
   // them per piece showed as 2 us on a 47 us launch.
   const uint32_t PL = p.n_kv_heads * p.head_groups;   // planes per sequence
-  const uint32_t U = uni(PL * prefix[B]);
+  const uint32_t U = PL * total_units;
   // workgroups that take part: at most one per unit, and few enough that no plane is cut
   // into more pieces than two fold levels take (a plane of u units has at most u / q + 2
   // pieces, q = U / W units being the smaller share)
-  const uint32_t q_min = (uni(s_umax) + kMaxPieces - 3) / (kMaxPieces - 2);
+  const uint32_t q_min = (umax_all + kMaxPieces - 3) / (kMaxPieces - 2);
   uint32_t W = min(min((uint32_t)gridDim.x, U), U / q_min);
   // Workgroups are dealt to the eight XCDs by their id modulo 8.  Each XCD takes one contiguous
   // eighth of the shares, so that no two of them walk the same stretch of memory side by side
@@ -109,18 +131,28 @@ __global__ __launch_bounds__(kDecThreads, 2) void decode_balanced_kernel(DecodeK
   const uint32_t x_end = share_begin(w + 1);
   while (x < x_end) {
     // the sequence that holds unit x: the last b with PL prefix[b] <= x
-    uint32_t lo = 0, hi = B;
-    while (hi - lo > 1) {
-      const uint32_t mid = (lo + hi) >> 1;
-      if (PL * prefix[mid] <= x)
-        lo = mid;
-      else
-        hi = mid;
-    }
     // (every thread computes the same values; readfirstlane tells the compiler so)
-    const uint32_t seq = uni(lo);
-    const uint32_t u_seq = uni(prefix[seq + 1] - prefix[seq]);
-    const uint32_t seq_start = uni(PL * prefix[seq]);
+    uint32_t seq, u_seq, seq_start, pos;
+    if (in_registers) {
+      const uint64_t ended = __ballot((uint32_t)t.lane < B && PL * r_incl <= x);   // sequences that end at or before x
+      seq = (uint32_t)__builtin_popcountll(ended);
+      u_seq = lane_value(r_units, seq);
+      seq_start = PL * (lane_value(r_incl, seq) - u_seq);
+      pos = lane_value(r_pos, seq);
+    } else {
+      uint32_t lo = 0, hi = B;
+      while (hi - lo > 1) {
+        const uint32_t mid = (lo + hi) >> 1;
+        if (PL * prefix[mid] <= x)
+          lo = mid;
+        else
+          hi = mid;
+      }
+      seq = uni(lo);
+      u_seq = uni(prefix[seq + 1] - prefix[seq]);
+      seq_start = uni(PL * prefix[seq]);
+      pos = uni(s_pos[seq]);
+    }
     const uint32_t r = x - seq_start;
     const uint32_t pl = r / u_seq, a = r - pl * u_seq;        // plane of the sequence, first unit in it
     const uint32_t S = seq_start + pl * u_seq, E = S + u_seq;
@@ -131,7 +163,6 @@ __global__ __launch_bounds__(kDecThreads, 2) void decode_balanced_kernel(DecodeK
     const uint32_t plane_id = seq * PL + pl;
     const uint32_t slot0 = first_w + plane_id;
 
-    const uint32_t pos = uni(s_pos[seq]);
     const uint32_t k_begin = a * kUnitKeys;
     const uint32_t k_end = min(pos + 1, a_end * kUnitKeys);
     const uint32_t kvh = pl / p.head_groups, hgrp = pl % p.head_groups;
