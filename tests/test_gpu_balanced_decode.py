@@ -123,3 +123,69 @@ def test_small_calls_keep_the_plain_kernel():
             op.ragged_path(100, 5)       # beyond the batch capacity
     finally:
         op.close()
+
+
+def test_recorded_step_replays_like_eager_while_the_lengths_move():
+    """The step (attention over per-sequence positions + advance of the positions) recorded once
+    through ellm_graph_* and replayed: the lengths change between replays, and with them the split of
+    the keys over the workgroups, which the kernel derives from the device array at every launch.
+    Every replay must equal the eager launch on the same lengths, bit for bit."""
+    import torch
+
+    import ellm_amd
+
+    dtype = orc.F16
+    bcap, hq, hkv, cap = 12, 32, 4, 6000
+    q = rand_storage((1, bcap, hq, D), 71, dtype)
+    k = rand_storage((bcap, hkv, cap, D), 72, dtype)
+    v = rand_storage((bcap, hkv, cap, D), 73, dtype)
+    scale = 1.0 / np.sqrt(D)
+    op, (dq, dk, dv, dout, dlse) = _operator(q, k, v, dtype, scale)
+    start = np.array([5000, 3, 62, 63, 64, 1000, 2500, 127, 4090, 700, 1, 3333], dtype=np.uint32)
+    steps, by = 4, 37
+    try:
+        assert op.ragged_path(cap - 1, bcap) == 1
+        stream = torch.cuda.Stream()
+
+        def walk(use_graph):
+            pos = torch.from_numpy(start.view(np.int32).copy()).cuda()
+            outs = []
+            graph = None
+            with torch.cuda.stream(stream):
+                for n in range(steps):
+                    dout.fill_(float("nan"))
+
+                    def step():
+                        op.run_ragged(pos, cap - 1, bcap, stream=stream)
+                        ellm_amd.positions_advance(pos, by, stream=stream)
+
+                    if not use_graph:
+                        step()
+                    else:
+                        if graph is None:
+                            stream.synchronize()
+                            with ellm_amd.StepGraph(stream) as graph:
+                                step()
+                        graph.launch()
+                    stream.synchronize()
+                    outs.append((dout.view(torch.int16).cpu().numpy().copy(), dlse.cpu().numpy().copy()))
+                    _ = float(dout.float().sum())     # eager work between replays
+            if graph is not None:
+                graph.close()
+            return outs, pos.cpu().numpy().view(np.uint32)
+
+        eager, pos_e = walk(False)
+        replay, pos_g = walk(True)
+        assert np.array_equal(pos_e, start + steps * by) and np.array_equal(pos_g, pos_e)
+        for n in range(steps):
+            assert np.array_equal(eager[n][0], replay[n][0]), n
+            assert np.array_equal(eager[n][1].view(np.uint32), replay[n][1].view(np.uint32)), n
+        # and the last step against the oracle
+        last = start + (steps - 1) * by
+        want, want_lse = orc.attention(q, k, v, scale, dtype, positions=last, batch=bcap)
+        got = orc.from_storage(replay[-1][0].view(np.uint16), dtype)
+        res = compare(got, orc.from_storage(want, dtype), dtype)
+        assert res["ok"], res
+        assert np.abs(replay[-1][1] - want_lse).max() <= LSE_TOL
+    finally:
+        op.close()
