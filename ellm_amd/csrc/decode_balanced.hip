@@ -18,6 +18,7 @@
 // Reference semantics unchanged: per (sequence, query head) the result of flash_attention
 // (src/kernel/x86_64/f16_512/flash_attention.rs:30-92) over keys 0..=position of the sequence.
 #include "decode_common.hpp"
+#include "decode_shares.hpp"
 
 namespace ellm {
 using namespace dec;
@@ -39,7 +40,7 @@ __global__ __launch_bounds__(kDecThreads, 2) void decode_balanced_kernel(DecodeK
   __shared__ __attribute__((aligned(16))) uint16_t smem[kDecWaves * kWaveLdsHalves];
   __shared__ uint32_t prefix[kMaxBatch + 1];   // units of the sequences before sequence b (per plane)
   __shared__ uint32_t s_pos[kMaxBatch];        // last position of every sequence
-  __shared__ uint32_t s_last, s_umax;
+  __shared__ uint32_t s_last, s_umax, s_umin;
   const Lane t;
   const uint32_t B = p.batch;
 
@@ -64,9 +65,14 @@ __global__ __launch_bounds__(kDecThreads, 2) void decode_balanced_kernel(DecodeK
     for (int d = 1; d < kWave; d <<= 1) v = max(v, (uint32_t)__shfl_xor(v, d, kWave));
     return v;
   };
+  auto wave_min = [&](uint32_t v) {
+#pragma unroll
+    for (int d = 1; d < kWave; d <<= 1) v = min(v, (uint32_t)__shfl_xor(v, d, kWave));
+    return v;
+  };
   auto lane_value = [&](uint32_t v, uint32_t l) { return (uint32_t)__builtin_amdgcn_readlane((int)v, (int)l); };
   const bool in_registers = B <= (uint32_t)kWave;   // (uniform)
-  uint32_t r_pos = 0, r_units = 0, r_incl = 0, total_units, umax_all;
+  uint32_t r_pos = 0, r_units = 0, r_incl = 0, total_units, umax_all, umin_all;
   if (in_registers) {
     const bool live = (uint32_t)t.lane < B;
     r_pos = live ? position_of(t.lane) : 0u;
@@ -74,9 +80,10 @@ __global__ __launch_bounds__(kDecThreads, 2) void decode_balanced_kernel(DecodeK
     r_incl = wave_scan(r_units);
     total_units = lane_value(r_incl, kWave - 1);
     umax_all = uni(wave_max(r_units));
+    umin_all = uni(wave_min(live ? r_units : 0xffffffffu));
   } else {
     if (t.wave == 0) {
-      uint32_t carry = 0, umax = 0;
+      uint32_t carry = 0, umax = 0, umin = 0xffffffffu;
       for (uint32_t base = 0; base < B; base += kWave) {
         const bool live = base + t.lane < B;
         const uint32_t pos_b = live ? position_of(base + t.lane) : 0u;
@@ -86,15 +93,18 @@ __global__ __launch_bounds__(kDecThreads, 2) void decode_balanced_kernel(DecodeK
         if (live) prefix[base + t.lane + 1] = carry + incl;
         carry += __shfl(incl, kWave - 1, kWave);
         umax = max(umax, wave_max(u));
+        umin = min(umin, wave_min(live ? u : 0xffffffffu));
       }
       if (t.lane == 0) {
         prefix[0] = 0;
         s_umax = umax;
+        s_umin = umin;
       }
     }
     __syncthreads();
     total_units = uni(prefix[B]);
     umax_all = uni(s_umax);
+    umin_all = uni(s_umin);
   }
 
   // All of the index arithmetic is 32-bit (the launcher keeps calls with 2^31 units or more
@@ -107,21 +117,25 @@ __global__ __launch_bounds__(kDecThreads, 2) void decode_balanced_kernel(DecodeK
   // pieces, q = U / W units being the smaller share)
   const uint32_t q_min = (umax_all + kMaxPieces - 3) / (kMaxPieces - 2);
   uint32_t W = min(min((uint32_t)gridDim.x, U), U / q_min);
+  // Planes of equal length (to the unit): a whole number of workgroups per plane, so that the
+  // shares below end where the planes end and no workgroup starts a second piece (24 sequences
+  // x 8192 keys: 96 planes, 480 workgroups of 5 pieces a plane instead of 512 shares of 5.33).
+  const uint32_t planes_all = PL * B;
+  const bool equal_planes = umax_all == umin_all && planes_all <= W;
+  if (equal_planes) W -= W % planes_all;
   // Workgroups are dealt to the eight XCDs by their id modulo 8.  Each XCD takes one contiguous
   // eighth of the shares, so that no two of them walk the same stretch of memory side by side
   // (with shares numbered like the workgroups and as many pieces per plane as XCDs, every XCD
   // would read the same stretch of every plane).
   uint32_t w = blockIdx.x;
-  if (W >= 8) {
-    W &= ~7u;
-    if (w >= W) return;
-    w = (w & 7u) * (W >> 3) + (w >> 3);
-  }
+  if (W >= 8 && !equal_planes) W &= ~7u;
   if (w >= W) return;
-  // shares: the first `rem` workgroups take q + 1 units, the others q
-  const uint32_t q = U / W, rem = U - q * W, big = rem * (q + 1);
-  auto share_begin = [&](uint32_t g) { return g * q + min(g, rem); };
-  auto holder = [&](uint32_t unit) { return unit < big ? unit / (q + 1) : rem + (unit - big) / q; };
+  if ((W & 7u) == 0) w = (w & 7u) * (W >> 3) + (w >> 3);
+  // share g begins at floor(g U / W) (decode_shares.hpp): equal to the unit, and for equal planes
+  // with W a multiple of their number a plane's end is a share's end
+  const Shares shares(W, U);
+  auto share_begin = [&](uint32_t g) { return shares.begin(g); };
+  auto holder = [&](uint32_t unit) { return shares.holder(unit); };
   const uint32_t G = min((uint32_t)kMaxHeadsPerGroup, p.group);   // partial rows per slot
   // cluster partials and their counters are indexed by cluster slot; the planes' own counters
   // follow the cluster counters
@@ -158,7 +172,10 @@ __global__ __launch_bounds__(kDecThreads, 2) void decode_balanced_kernel(DecodeK
     const uint32_t S = seq_start + pl * u_seq, E = S + u_seq;
     const uint32_t stop = min(x_end, E);
     const uint32_t a_end = a + (stop - x);
-    const uint32_t first_w = holder(S), last_w = holder(E - 1);
+    // the workgroups that hold the plane's first and last unit (this one, when the piece starts
+    // or ends with the plane: no look-up then)
+    const uint32_t first_w = x == S ? w : holder(S);
+    const uint32_t last_w = stop == E ? w : holder(E - 1);
     const uint32_t n_pieces = last_w - first_w + 1, piece = w - first_w;
     const uint32_t plane_id = seq * PL + pl;
     const uint32_t slot0 = first_w + plane_id;
@@ -223,7 +240,7 @@ bool decode_balanced_takes(const DecodeWorkspace& w, uint32_t batch, uint32_t n_
   const uint64_t head_groups = (group + kMaxHeadsPerGroup - 1) / kMaxHeadsPerGroup;
   const uint64_t planes = (uint64_t)batch * n_kv_heads * head_groups;
   const uint64_t units = planes * ((max_len + kUnitKeys - 1) / kUnitKeys);
-  if (units < 8ull * wgs || units + wgs >= (1ull << 31)) return false;
+  if (units < 8ull * wgs || units + wgs >= (1ull << 31) || wgs >= (1u << 16)) return false;
   const uint64_t G = group < (uint32_t)kMaxHeadsPerGroup ? group : (uint32_t)kMaxHeadsPerGroup;
   const uint64_t slots = wgs + planes, cslots = planes + slots / kMergeFan + 2;
   return slots * G <= w.rows && cslots * G <= w.rows2 && cslots + planes <= w.counters;
