@@ -50,3 +50,55 @@ def test_random_chunk_shapes_match_oracle(block):
         lse_err = float(np.abs(got_lse[:, :c["b"]] - want_lse[:, :c["b"]]).max())
         assert res["ok"], (c, res)
         assert lse_err <= LSE_TOL, (c, lse_err)
+
+
+def _draw_ragged(rng):
+    hkv = int(rng.choice([1, 2, 4, 8]))
+    g = int(rng.choice([1, 2, 3, 4, 8, 16, 32]))
+    b = int(rng.choice([1, 5, 16, 33, 64, 65, 130, 300]))
+    cap = int(rng.choice([300, 2500, 8192, 20000, 50000]))
+    # cache size and the oracle's work bounded
+    while b * hkv * cap * D * 2 > 2.5e8 or b * hkv * g * cap > 5e7:
+        if b > 16:
+            b //= 2
+        elif cap > 1024:
+            cap //= 2
+        else:
+            g = max(1, g // 2)
+    kind = int(rng.integers(0, 4))
+    if kind == 0:
+        pos = rng.integers(0, cap, size=b)
+    elif kind == 1:                                  # one long, the rest short
+        pos = rng.integers(0, min(cap, 200), size=b)
+        pos[int(rng.integers(0, b))] = cap - 1
+    elif kind == 2:                                  # all equal
+        pos = np.full(b, int(rng.integers(0, cap)))
+    else:                                            # around the 64-key unit
+        pos = rng.choice([0, 62, 63, 64, 65, 127, 128, cap - 1, cap - 2], size=b)
+    return dict(hq=hkv * g, hkv=hkv, b=b, cap=cap, pos=np.minimum(pos, cap - 1).astype(np.uint32))
+
+
+@pytest.mark.parametrize("block", range(3))
+def test_random_ragged_single_token_steps_match_oracle(block):
+    """Per-sequence positions: small calls keep the kernel that splits every plane alike, large ones
+    take the kernel that deals the keys evenly; both paths are drawn."""
+    import torch
+
+    import ellm_amd
+
+    rng = np.random.default_rng(2000 + block)
+    paths = set()
+    for n in range(6):
+        c = _draw_ragged(rng)
+        dtype = orc.F16 if (n + block) % 2 else orc.BF16
+        print("case", block, n, {k: v for k, v in c.items() if k != "pos"}, c["pos"][:8], flush=True)
+        b, hq, hkv, cap = c["b"], c["hq"], c["hkv"], c["cap"]
+        q = rand_storage((1, b, hq, D), 7500 + 10 * block + n, dtype)
+        k = rand_storage((b, hkv, cap, D), 8500 + 10 * block + n, dtype)
+        v = rand_storage((b, hkv, cap, D), 9500 + 10 * block + n, dtype)
+        scale = 1.0 / np.sqrt(D)
+        want, want_lse = orc.attention(q, k, v, scale, dtype, positions=c["pos"], batch=b)
+        got, got_lse = gpu_attention(q, k, v, scale, dtype, positions=c["pos"], batch=b)
+        res = compare(got, orc.from_storage(want, dtype), dtype)
+        assert res["ok"], (c, res)
+        assert float(np.abs(got_lse - want_lse).max()) <= LSE_TOL, c
