@@ -143,6 +143,10 @@ int ellm_attn_run(ellm_attn* handle, size_t position_index, size_t position_inte
  * 0..=positions[i].  max_position: an upper bound (inclusive) on every entry,
  * known on the host; it sizes the launch.  Entries above max_position or at or
  * beyond sequence_capacity are clamped to that bound on the device.
+ * Large calls (see ellm_attn_ragged_path) deal the keys of all K/V planes to the
+ * workgroups in equal shares, so that the time follows the sum of the lengths and
+ * not the longest of them; the split of the work depends on the positions only,
+ * hence equal positions give equal bits.
  */
 int ellm_attn_run_ragged(ellm_attn* handle, const uint32_t* positions, size_t max_position,
                          size_t batch_size, void* stream);
@@ -168,7 +172,10 @@ int ellm_attn_ragged_path(const ellm_attn* handle, size_t max_position, size_t b
  *   positions == NULL : every sequence attends to keys 0..=position;
  *   positions != NULL : device uint32[batch_size], one position per sequence, each
  *                       clamped to `position` (their upper bound, which sizes the launch).
- * Same kernel and split plan as the handle's path, so the results are bit-identical.
+ * Same kernel and split plan as ellm_attn_run and as the ellm_attn_run_ragged calls for which
+ * ellm_attn_ragged_path returns 0, so those results are bit-identical (the kernel for large
+ * calls with per-sequence positions, path 1, splits the keys differently: same tolerance,
+ * other bits).
  * The split partials and arrival counters live in a static device array of 5,074,944
  * bytes that every device the library runs on holds until the process ends; the call
  * uses the current device's copy.  Limit: sequences x query heads x splits <= 8192
