@@ -139,7 +139,89 @@ def bench_decode(batch, length, steps, warmup, hq=32, hkv=4, copies=4):
     }
 
 
-def bench_prefill(seq, steps, warmup, hq=32, hkv=4, dtype_name="f16", p0=0, zero_kv=False, batch=1, copies=1):
+def _board_sensors():
+    """hwmon files of every card the kernel driver shows: power (uW), power cap (uW), engine clock (Hz)."""
+    import glob
+
+    cards = []
+    for dev in sorted(glob.glob("/sys/class/drm/card*/device")):
+        for hw in glob.glob(os.path.join(dev, "hwmon", "hwmon*")):
+            f = {}
+            for key, names in (("power", ("power1_input", "power1_average")), ("cap", ("power1_cap",)),
+                               ("sclk", ("freq1_input",))):
+                for n in names:
+                    if os.path.exists(os.path.join(hw, n)):
+                        f[key] = os.path.join(hw, n)
+                        break
+            if "sclk" not in f and os.path.exists(os.path.join(dev, "pp_dpm_sclk")):
+                f["dpm_sclk"] = os.path.join(dev, "pp_dpm_sclk")   # lines "n: <MHz>Mhz", the current one starred
+            if "power" in f:
+                cards.append(f)
+    return cards
+
+
+def board_power_during(run_pass, seconds=1.0, period=0.02):
+    """Board power and engine clock, read from the driver's hwmon files every `period` seconds on a
+    second thread while run_pass() (a batch of launches ending in a synchronisation) is repeated for
+    `seconds`.  Not part of any timed region.  With several cards visible the one that draws most is
+    taken.  None where the files are missing or unreadable."""
+    import statistics
+    import threading
+
+    cards = _board_sensors()
+    if not cards:
+        return None
+
+    def read(path):
+        try:
+            return float(open(path).read().strip())
+        except (OSError, ValueError):
+            return None
+
+    def read_clock(c):
+        if "sclk" in c:
+            return read(c["sclk"])
+        if "dpm_sclk" in c:
+            try:
+                for line in open(c["dpm_sclk"]).read().splitlines():
+                    if "*" in line:
+                        return float(line.split(":")[1].lower().replace("mhz", "").replace("*", "").strip()) * 1e6
+            except (OSError, ValueError, IndexError):
+                pass
+        return None
+
+    rows, stop = [], threading.Event()
+
+    def poll():
+        while not stop.is_set():
+            rows.append([(read(c["power"]), read_clock(c)) for c in cards])
+            stop.wait(period)
+
+    th = threading.Thread(target=poll, daemon=True)
+    th.start()
+    t0 = time.perf_counter()
+    while time.perf_counter() - t0 < seconds:
+        run_pass()
+    stop.set()
+    th.join()
+    rows = rows[len(rows) // 4:]      # the first quarter: clocks and the sensor's average still moving
+    best = None
+    for i, c in enumerate(cards):
+        watts = [r[i][0] / 1e6 for r in rows if r[i][0] is not None]
+        if not watts:
+            continue
+        mhz = [r[i][1] / 1e6 for r in rows if r[i][1] is not None]
+        cap = read(c["cap"]) if "cap" in c else None
+        entry = {"watts": round(statistics.mean(watts), 1), "watts_max": round(max(watts), 1),
+                 "cap_watts": round(cap / 1e6, 1) if cap else None,
+                 "engine_mhz": round(statistics.mean(mhz), 0) if mhz else None, "samples": len(watts)}
+        if best is None or entry["watts"] > best["watts"]:
+            best = entry
+    return best
+
+
+def bench_prefill(seq, steps, warmup, hq=32, hkv=4, dtype_name="f16", p0=0, zero_kv=False, batch=1, copies=1,
+                  power_seconds=0.0):
     import torch
 
     import ellm_amd
@@ -167,6 +249,14 @@ def bench_prefill(seq, steps, warmup, hq=32, hkv=4, dtype_name="f16", p0=0, zero
     per, step_ms = _time_steps(lambda i: ops[i % copies][0].run(p0, seq, batch), steps, warmup)
     flops = batch * 4 * D * hq * (seq * p0 + seq * (seq + 1) // 2)
     kern_ms = sum(per) / len(per)
+    passes = _last_passes
+    power = None
+    if power_seconds > 0:       # after the timed passes, not inside them
+        def run_pass():
+            for i in range(8):
+                ops[i % copies][0].run(p0, seq, batch)
+            torch.cuda.synchronize()
+        power = board_power_during(run_pass, power_seconds)
     for op in ops:
         op[0].close()
     return {
@@ -175,7 +265,8 @@ def bench_prefill(seq, steps, warmup, hq=32, hkv=4, dtype_name="f16", p0=0, zero
         "kernel_ms": kern_ms,
         "tflops": flops / (step_ms * 1e-3) / 1e12,
         "kernel_tflops": flops / (kern_ms * 1e-3) / 1e12,
-        "passes": _last_passes,
+        "passes": passes,
+        "power": power,
     }
 
 
@@ -822,7 +913,10 @@ def main():
         dec = bench_decode(16, 8192, args.steps, args.warmup)
     if args.only in ("", "prefill"):
         pf_steps = max(3, min(args.steps, 10))
-        pf = bench_prefill(32768, pf_steps, min(args.warmup, 2), zero_kv=args.prefill_zero_kv)
+        pf = bench_prefill(32768, pf_steps, min(args.warmup, 2), zero_kv=args.prefill_zero_kv, power_seconds=1.0)
+        # the same launch on zero K and V: same instruction stream, operands that toggle nothing
+        # (not a result: it shows what the operand values cost in clock under the board's power cap)
+        pf_zero = None if args.prefill_zero_kv else bench_prefill(32768, 3, 1, zero_kv=True, power_seconds=1.0)
         # the ceiling this box gives any MFMA kernel on dense random fp16 operands, timed right
         # after the kernel it is compared with
         n_cu = torch.cuda.get_device_properties(0).multi_processor_count
@@ -843,6 +937,14 @@ def main():
                          "frac": round(pf["kernel_tflops"] / MFMA_F16_PEAK_TFLOPS, 4),
                          "traffic": TRAFFIC_BYTES["prefill"]},
             "passes": pf["passes"],
+            "board_power": {
+                "what": "board power and engine clock from the driver's hwmon files, sampled every 20 ms while the "
+                        "launch is repeated for a second right after the timed passes; and the same launch on "
+                        "K = V = 0 (same instruction stream, operands that toggle nothing)",
+                "this_workload": pf["power"],
+                "zero_kv": None if pf_zero is None else dict(pf_zero["power"] or {}, ms_per_step=round(pf_zero["ms_per_step"], 4),
+                                                             tflops=round(pf_zero["tflops"], 1)),
+            },
             "mfma_stream_on_n01_fp16": {
                 "what": "pure v_mfma_f32_32x32x16_f16 stream on N(0,1) operands, one wave per SIMD on every "
                         "compute unit, no memory access in the loop, timed in this run (libellm_diag.so)",
