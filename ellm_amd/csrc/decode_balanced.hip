@@ -28,12 +28,14 @@ constexpr uint32_t kUnitKeys = kDecodeStepKeys;   // 64: one step of the four wa
 constexpr uint32_t kMaxBatch = 1024;              // lengths are scanned in LDS
 constexpr uint32_t kMaxPieces = kMergeFan * kMergeFan;  // two fold levels of 16
 
+// (the compiler cannot see that a value every lane computes alike is wave-uniform)
+__device__ __forceinline__ uint32_t uni(uint32_t v) { return (uint32_t)__builtin_amdgcn_readfirstlane((int)v); }
+
 // Pieces of plane p occupy consecutive partial slots first_w(p) + p .. (the pair (workgroup,
 // plane) moves on by one in exactly one of the two from piece to piece, so workgroup + plane
 // numbers the pieces of a launch without gaps that matter and without collisions); a plane's
 // clusters of 16 pieces take cluster slots p + slot0 / 16 + c, which are distinct for the same
 // reason (1 + floor(n / 16) >= ceil(n / 16)).
-__device__ __forceinline__ uint32_t uni(uint32_t v) { return (uint32_t)__builtin_amdgcn_readfirstlane((int)v); }
 
 template <typename T>
 __global__ __launch_bounds__(kDecThreads, 2) void decode_balanced_kernel(DecodeKernelArgs p) {
