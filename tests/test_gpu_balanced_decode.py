@@ -63,6 +63,8 @@ CASES = [
     ("mha_heads", 8, 4, 4, 9000, [4000, 3000, 2000, 1000, 8999, 10, 100, 640]),
     ("batch_below_capacity", 30, 16, 4, 3400, [3399, 5, 1500, 64] * 5),
     ("shares_smaller_than_planes_many_sequences", 200, 8, 2, 1400, list(range(200, 1400, 6))),
+    # more than 64 sequences (lengths scanned in LDS) and one plane cut into hundreds of pieces
+    ("one_long_among_many_short", 70, 8, 1, 20000, [19999] + [(7 * i) % 300 for i in range(69)]),
 ]
 
 
