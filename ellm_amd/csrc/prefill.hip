@@ -436,18 +436,18 @@ __global__ __launch_bounds__(kPpThreads, 2) void prefill_pingpong_kernel(Prefill
 }
 
 // ---------------------------------------------------------------------------
-// Few query rows per K/V plane: the short last chunk of a prompt (2 - 33 tokens x 24
+// Few query rows per K/V plane: the short last chunk of a prompt (1 - 63 tokens x 24
 // sequences on caches of thousands of tokens in the reference's serving loop,
 // src/serving/start copy.rs:71-101).  The ping-pong kernel above is built for tiles that
 // are re-used by thousands of rows and sit in L2; here every K/V byte is used once by at
-// most 128 rows and the call is a stream from HBM, like the single-token kernel: what
-// matters is bytes in flight, not MFMA issue.  One workgroup = 4 waves x 32 query rows =
-// all (token, head) pairs of one GQA group (row r of the plane = token r / group, head
-// r % group), so a plane is read once; the key range is split over gridDim.y workgroups
-// (two per compute unit, 36 KB of LDS each), which leave partial rows for
-// prefill_merge_kernel as the split form of the kernel above does.  Chunks of 32 keys go
-// memory -> registers -> LDS (double-buffered, one barrier a chunk, the next chunk's loads in
-// flight during the MFMAs of this one); operands and soft-max as above.
+// most 384 rows and the call is a stream from HBM, like the single-token kernel: with few
+// rows what matters is bytes in flight, not MFMA issue.  One workgroup = 4, 8 or 12 waves x
+// 32 query rows = all (token, head) pairs of one GQA group (row r of the plane = token
+// r / group, head r % group), so a plane is read once; the key range is split over gridDim.y
+// workgroups (36 KB of LDS each), which leave partial rows for prefill_merge_kernel as the
+// split form of the kernel above does.  Chunks of 32 keys go memory -> registers -> LDS
+// (double-buffered, one barrier a chunk, the next chunks' loads in flight during the MFMAs of
+// this one); operands and soft-max as above.
 // ---------------------------------------------------------------------------
 constexpr int kSK = 32;                        // keys per compute step
 constexpr int kStStagersMax = 8 * kWave;       // one 16-byte piece of K and of V each moves a whole chunk

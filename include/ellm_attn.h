@@ -124,7 +124,7 @@ int ellm_attn_reset(ellm_attn* handle, void* stream);
  * position_interval == 1 takes the split-KV single-token kernel, larger
  * intervals the tiled MFMA kernel (with the key range split over workgroups and
  * a merge launch behind it when the call has too few query rows to fill the
- * device; calls with at most 128 query rows per K/V plane on 512 keys or more
+ * device; calls with at most 384 query rows per K/V plane on 512 keys or more
  * take a kernel that streams every plane once).  Zero batch_size or
  * position_interval is a no-op returning ELLM_OK.  One run of a handle in flight
  * at a time (see the top of this file).
