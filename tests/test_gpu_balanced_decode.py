@@ -191,3 +191,25 @@ def test_recorded_step_replays_like_eager_while_the_lengths_move():
         assert np.abs(replay[-1][1] - want_lse).max() <= LSE_TOL
     finally:
         op.close()
+
+
+@pytest.mark.parametrize("scale", [-0.07, 0.0, 1.0])
+def test_unusual_scales_and_garbage_beyond_the_positions(scale):
+    """Negative, zero and large scales; cache rows after a sequence's position hold NaN / Inf / huge
+    values, which must not leak (the stream clamps its reads to the last valid row)."""
+    dtype = orc.F16
+    bcap, hq, hkv, cap = 16, 16, 4, 4200
+    positions = [4199, 0, 63, 64, 1000, 2047, 2048, 3000, 17, 4100, 128, 129, 500, 3999, 1, 2500]
+    q = rand_storage((1, bcap, hq, D), 81, dtype)
+    k = rand_storage((bcap, hkv, cap, D), 82, dtype, scale=0.3)
+    v = rand_storage((bcap, hkv, cap, D), 83, dtype)
+    kf, vf = k.view(np.float16), v.view(np.float16)
+    for b, pos in enumerate(positions):
+        kf[b, :, pos + 1:] = [np.nan, np.inf, -np.inf, 6.0e4][b % 4]
+        vf[b, :, pos + 1:] = [np.inf, np.nan, 6.0e4, -np.inf][b % 4]
+    op, bufs = _operator(q, k, v, dtype, scale)
+    try:
+        got, _ = _run_and_check(op, bufs, q, k, v, dtype, scale, positions, bound=cap - 1)
+        assert np.isfinite(got).all()
+    finally:
+        op.close()
