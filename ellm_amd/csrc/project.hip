@@ -163,24 +163,29 @@ __global__ __launch_bounds__(kProjThreads) void project_kernel(ProjectKernelArgs
   __syncthreads();
 
   // One iteration = one chunk: four 16-wide steps, 64 MFMAs.  Chunk c sits in stage c % 2;
-  // during it the staging registers (chunk c + 1) are stored to the other stage and
-  // refilled with chunk c + 2.  The operands of a step are read during the step before
-  // it, except those of a chunk's first step: the stage is complete only at the barrier.
-  // LDS traffic is spread evenly (a read every second MFMA, a store every fourth): the four
+  // during its first three steps the staging registers (chunk c + 1) are stored to the other
+  // stage and refilled with chunk c + 2; the iteration's one barrier stands before step 3, and
+  // the operands of the next chunk's first step are read, from the stage just completed, during
+  // step 3.  So the operands of every step are read during the step before it, across chunks
+  // too.  The barrier orders both hazards: the stage being refilled was last read for step 3 of
+  // chunk c - 1, and those reads had returned before the previous barrier.
+  // LDS traffic is spread evenly (a read every second MFMA, a store every third): the four
   // waves together keep the LDS pipe busy most of the time, and a burst of stores
   // would still be draining when the barrier is reached.
   u32x4 opa[8], opb[8];
+#pragma unroll
+  for (int o = 0; o < 8; ++o) opa[o] = read_operand(x_read[0], w_read[0], o);
   for (uint32_t c = 0; c < n_chunks; ++c) {
     const uint32_t cur = (c & 1) * kStageBytes, nxt = kStageBytes - cur;
-    uint32_t xb[4], wb[4];
+    uint32_t xb[5], wb[5];   // [4]: first step of the next chunk
 #pragma unroll
-    for (int st = 0; st < 4; ++st) {
+    for (int st = 1; st < 4; ++st) {
       xb[st] = pin(x_read[st] + cur);
       wb[st] = pin(w_read[st] + cur);
     }
+    xb[4] = pin(x_read[0] + nxt);
+    wb[4] = pin(w_read[0] + nxt);
     const uint32_t store_at = pin(st_store + nxt);
-#pragma unroll
-    for (int o = 0; o < 8; ++o) opa[o] = read_operand(xb[0], wb[0], o);
     __builtin_amdgcn_sched_barrier(0);
     static_for<64>([&](auto n_) {
       constexpr int n = decltype(n_)::value;
@@ -190,17 +195,20 @@ __global__ __launch_bounds__(kProjThreads) void project_kernel(ProjectKernelArgs
         if constexpr ((n & 1) == 0) opb[m >> 1] = read_operand(xb[st + 1], wb[st + 1], m >> 1);
       } else {
         acc[m >> 2][m & 3] = M::m32x32x16(opb[w_of(m)], opb[x_of(m)], acc[m >> 2][m & 3]);
-        if constexpr ((n & 1) == 0 && st < 3) opa[m >> 1] = read_operand(xb[st + 1], wb[st + 1], m >> 1);
+        if constexpr ((n & 1) == 0) opa[m >> 1] = read_operand(xb[st + 1], wb[st + 1], m >> 1);
       }
-      if constexpr ((n & 3) == 3) {
-        store_piece(store_at, n >> 2);
-        load_piece(c + 2, n >> 2);
+      if constexpr (n < 48 && n % 3 == 2) {
+        store_piece(store_at, n / 3);
+        load_piece(c + 2, n / 3);
+      }
+      if constexpr (n == 47) {
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+        __builtin_amdgcn_s_barrier();
       }
       __builtin_amdgcn_sched_barrier(0);
     });
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
-    __builtin_amdgcn_s_barrier();
   }
+  __syncthreads();   // every wave is past its last operand reads: the epilogue reuses the stages
 
   const HeadRows<4> head = prepare_head<S, MODE, 4>(p, 2 * tn + wn, row0 + wm * 128, lane);
   finish_head<S, MODE, 4>(p, acc, head, lds0 + wave * kEpWaveBytes, lane);
