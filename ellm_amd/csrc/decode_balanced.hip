@@ -118,19 +118,34 @@ __global__ __launch_bounds__(kDecThreads, 2) void decode_balanced_kernel(DecodeK
   // into more pieces than two fold levels take (a plane of u units has at most u / q + 2
   // pieces, q = U / W units being the smaller share)
   const uint32_t q_min = (umax_all + kMaxPieces - 3) / (kMaxPieces - 2);
-  uint32_t W = min(min((uint32_t)gridDim.x, U), U / q_min);
   // Planes of equal length (to the unit): a whole number of workgroups per plane, so that the
   // shares below end where the planes end and no workgroup starts a second piece (24 sequences
   // x 8192 keys: 96 planes, 480 workgroups of 5 pieces a plane instead of 512 shares of 5.33).
+  // Else a multiple of eight, for the XCD order below.
   const uint32_t planes_all = PL * B;
-  const bool equal_planes = umax_all == umin_all && planes_all <= W;
-  if (equal_planes) W -= W % planes_all;
+  auto takers = [&](uint32_t limit) {
+    uint32_t n = min(min(limit, U), U / q_min);
+    if (umax_all == umin_all && planes_all <= n)
+      n -= n % planes_all;
+    else if (n >= 8)
+      n &= ~7u;
+    return n;
+  };
+  // One workgroup per compute unit streams as fast as two that share one, leaves half the
+  // partial rows to fold and ends more evenly (32 sequences of 1k-128k keys: 658 against 679 us);
+  // two per unit are better where the rounding above would leave units idle (96 equal planes:
+  // 192 of 256) and where a workgroup walks several short planes one after the other, each with
+  // its own start-up that a second workgroup on the unit hides (400 planes of 100-4096 keys).
+  uint32_t W = takers(gridDim.x);
+  if (p.wgs_one < gridDim.x && planes_all <= p.wgs_one) {
+    const uint32_t one_each = takers(p.wgs_one);
+    if (100u * one_each >= 47u * W) W = one_each;
+  }
   // Workgroups are dealt to the eight XCDs by their id modulo 8.  Each XCD takes one contiguous
   // eighth of the shares, so that no two of them walk the same stretch of memory side by side
   // (with shares numbered like the workgroups and as many pieces per plane as XCDs, every XCD
   // would read the same stretch of every plane).
   uint32_t w = blockIdx.x;
-  if (W >= 8 && !equal_planes) W &= ~7u;
   if (w >= W) return;
   if ((W & 7u) == 0) w = (w & 7u) * (W >> 3) + (w >> 3);
   // share g begins at floor(g U / W) (decode_shares.hpp): equal to the unit, and for equal planes
@@ -274,6 +289,7 @@ hipError_t launch_decode_balanced(const AttnArgs& a, uint32_t wgs, hipStream_t s
   p.split_len = 0;
   p.n_split = 0;
   p.batch = a.batch;
+  p.wgs_one = a.n_cu ? a.n_cu : wgs;
   p.scale_log2 = a.scale * kLog2e;
   // cluster slots (the kernel's cslot0 + cluster stays below this): the planes' own counters follow
   const uint32_t planes = a.batch * a.n_kv_heads * p.head_groups;

@@ -44,6 +44,7 @@ struct DecodeKernelArgs {
   uint32_t position;  // shared position (positions == null) or upper bound
   uint32_t split_len, n_split;
   uint32_t batch;     // sequences (decode_balanced.hip)
+  uint32_t wgs_one;   // workgroups that find a compute unit each (decode_balanced.hip)
   float scale_log2;   // scale * log2(e)
 };
 
