@@ -152,6 +152,10 @@ pub struct ellm_graph {
     _private: [u8; 0],
 }
 #[repr(C)]
+pub struct ellm_side_stream {
+    _private: [u8; 0],
+}
+#[repr(C)]
 pub struct ellm_matmul3 {
     _private: [u8; 0],
 }
@@ -261,6 +265,11 @@ extern "C" {
     pub fn ellm_graph_end(stream: Stream, out_graph: *mut *mut ellm_graph) -> c_int;
     pub fn ellm_graph_launch(graph: *mut ellm_graph, stream: Stream) -> c_int;
     pub fn ellm_graph_destroy(graph: *mut ellm_graph) -> c_int;
+    pub fn ellm_side_stream_create(out_side: *mut *mut ellm_side_stream) -> c_int;
+    pub fn ellm_side_stream_get(side: *mut ellm_side_stream) -> Stream;
+    pub fn ellm_side_stream_fork(side: *mut ellm_side_stream, stream: Stream) -> c_int;
+    pub fn ellm_side_stream_join(side: *mut ellm_side_stream, stream: Stream) -> c_int;
+    pub fn ellm_side_stream_destroy(side: *mut ellm_side_stream) -> c_int;
     pub fn ellm_positions_advance(positions: *mut u32, batch_size: usize, by: u32, stream: Stream) -> c_int;
 
     pub fn ellm_matmul3_create(desc: *const ellm_matmul3_desc, out_handle: *mut *mut ellm_matmul3) -> c_int;

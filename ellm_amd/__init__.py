@@ -17,4 +17,4 @@ from ._lib import (  # noqa: F401
 )
 from .attention import Attention, KVCache  # noqa: F401
 from .projection import MatMul3, MatMulAdd  # noqa: F401
-from .schedule import StepGraph, positions_advance, schedule_calls  # noqa: F401
+from .schedule import SideStream, StepGraph, positions_advance, schedule_calls  # noqa: F401

@@ -148,6 +148,11 @@ ABI_SYMBOLS = {
     "ellm_graph_end": (ctypes.c_int, [_vp, _pvp]),
     "ellm_graph_launch": (ctypes.c_int, [_vp, _vp]),
     "ellm_graph_destroy": (ctypes.c_int, [_vp]),
+    "ellm_side_stream_create": (ctypes.c_int, [_pvp]),
+    "ellm_side_stream_get": (ctypes.c_void_p, [_vp]),
+    "ellm_side_stream_fork": (ctypes.c_int, [_vp, _vp]),
+    "ellm_side_stream_join": (ctypes.c_int, [_vp, _vp]),
+    "ellm_side_stream_destroy": (ctypes.c_int, [_vp]),
     "ellm_positions_advance": (ctypes.c_int, [_vp, _sz, ctypes.c_uint32, _vp]),
     "ellm_matmul3_create": (ctypes.c_int, [ctypes.POINTER(MatMul3Desc), _pvp]),
     "ellm_matmul3_run": (ctypes.c_int, [_vp, _sz, _sz, _sz, _vp]),

@@ -732,6 +732,67 @@ int ellm_graph_destroy(ellm_graph* graph) {
   return ELLM_OK;
 }
 
+struct ellm_side_stream {
+  int device;
+  hipStream_t stream;
+  hipEvent_t forked;   // recorded on the caller's stream, awaited by the side stream
+  hipEvent_t joined;   // recorded on the side stream, awaited by the caller's stream
+};
+
+int ellm_side_stream_create(ellm_side_stream** out) {
+  if (!out) return fail(ELLM_ERR_INVALID_ARGUMENT, "null output");
+  *out = nullptr;
+  int device = 0, n_cu = 0;
+  if (int st = ellm::current_gfx950_device(&device, &n_cu)) return st;
+  ellm_side_stream* s = new (std::nothrow) ellm_side_stream{device, nullptr, nullptr, nullptr};
+  if (!s) return fail(ELLM_ERR_HIP, "out of host memory");
+  // (default priority, as every stream that shares the device with the caller's)
+  hipError_t e = hipStreamCreateWithFlags(&s->stream, hipStreamNonBlocking);
+  if (e == hipSuccess) e = hipEventCreateWithFlags(&s->forked, hipEventDisableTiming);
+  if (e == hipSuccess) e = hipEventCreateWithFlags(&s->joined, hipEventDisableTiming);
+  if (e != hipSuccess) {
+    (void)ellm_side_stream_destroy(s);
+    return fail_hip(e, "side stream");
+  }
+  *out = s;
+  return ELLM_OK;
+}
+
+void* ellm_side_stream_get(ellm_side_stream* s) { return s ? (void*)s->stream : nullptr; }
+
+int ellm_side_stream_fork(ellm_side_stream* s, void* stream) {
+  if (!s) return fail(ELLM_ERR_INVALID_ARGUMENT, "null side stream");
+  if (int st = ellm::check_current_device(s->device)) return st;
+  hipError_t e = hipEventRecord(s->forked, (hipStream_t)stream);
+  if (e == hipSuccess) e = hipStreamWaitEvent(s->stream, s->forked, 0);
+  if (e != hipSuccess) return fail_hip(e, "side stream fork");
+  return ELLM_OK;
+}
+
+int ellm_side_stream_join(ellm_side_stream* s, void* stream) {
+  if (!s) return fail(ELLM_ERR_INVALID_ARGUMENT, "null side stream");
+  if (int st = ellm::check_current_device(s->device)) return st;
+  hipError_t e = hipEventRecord(s->joined, s->stream);
+  if (e == hipSuccess) e = hipStreamWaitEvent((hipStream_t)stream, s->joined, 0);
+  if (e != hipSuccess) return fail_hip(e, "side stream join");
+  return ELLM_OK;
+}
+
+int ellm_side_stream_destroy(ellm_side_stream* s) {
+  if (!s) return ELLM_OK;
+  hipError_t first = hipSuccess;
+  auto note = [&](hipError_t e) {
+    if (e != hipSuccess && first == hipSuccess) first = e;
+  };
+  if (s->stream) note(hipStreamSynchronize(s->stream));
+  if (s->forked) note(hipEventDestroy(s->forked));
+  if (s->joined) note(hipEventDestroy(s->joined));
+  if (s->stream) note(hipStreamDestroy(s->stream));
+  delete s;
+  if (first != hipSuccess) return fail_hip(first, "side stream destroy");
+  return ELLM_OK;
+}
+
 int ellm_positions_advance(uint32_t* positions, size_t batch_size, uint32_t by, void* stream) {
   if (batch_size == 0) return ELLM_OK;
   if (!positions) return fail(ELLM_ERR_INVALID_ARGUMENT, "null positions");

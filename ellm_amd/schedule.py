@@ -6,7 +6,9 @@ The reference's serving thread walks a request as: the prompt in chunks of
 (src/serving/start copy.rs:71-113); every operator of the graph is run once per such
 call.  `schedule_calls` returns those (position_index, position_interval) pairs;
 `StepGraph` records the launches of one single-token step into a HIP graph so that the
-per-token loop costs one launch instead of two per layer."""
+per-token loop costs one launch instead of two per layer; `SideStream` lets the two
+independent halves of a mixed step (a prompt chunk, one new token of the other
+sequences) run side by side."""
 import ctypes
 
 from ._lib import check, load_library
@@ -34,6 +36,46 @@ def positions_advance(positions, by=1, stream=None):
 
     check(load_library().ellm_positions_advance(ctypes.c_void_p(positions.data_ptr()),
                                                 positions.numel(), by, _stream_ptr(stream)))
+
+
+class SideStream:
+    """A second stream of the library's (ellm_side_stream_*).  Pass the object as `stream=` to
+    the operators whose launches may run beside those of the caller's stream:
+
+        side.fork(stream); chunk_op.run(..., stream=stream); token_op.run_ragged(..., stream=side)
+        side.join(stream)
+
+    also between StepGraph's begin and end, where the side launches become a parallel branch."""
+
+    def __init__(self):
+        self._lib = load_library()
+        self._handle = ctypes.c_void_p()
+        check(self._lib.ellm_side_stream_create(ctypes.byref(self._handle)))
+
+    @property
+    def cuda_stream(self):
+        return self._lib.ellm_side_stream_get(self._handle) or 0
+
+    def fork(self, stream=None):
+        from .attention import _stream_ptr
+
+        check(self._lib.ellm_side_stream_fork(self._handle, _stream_ptr(stream)))
+
+    def join(self, stream=None):
+        from .attention import _stream_ptr
+
+        check(self._lib.ellm_side_stream_join(self._handle, _stream_ptr(stream)))
+
+    def close(self):
+        if self._handle:
+            check(self._lib.ellm_side_stream_destroy(self._handle))
+            self._handle = ctypes.c_void_p()
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
 
 
 class StepGraph:

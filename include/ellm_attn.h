@@ -354,6 +354,31 @@ int ellm_graph_end(void* stream, ellm_graph** out_graph);
 int ellm_graph_launch(ellm_graph* graph, void* stream);
 int ellm_graph_destroy(ellm_graph* graph);
 
+/*
+ * A second stream for launches that may run beside those on the caller's stream.
+ * A mixed step holds two independent halves, the chunk of a prompt (MFMA-bound) and
+ * one new token of the other sequences (HBM-bound); issued one after the other on
+ * one stream each waits for the other's last workgroups, side by side they fill
+ * each other's tails (16384-token chunk + 32 sequences of 1k-128k cached tokens,
+ * one layer: 3.05 -> 2.89 ms).  The reference has no counterpart: its operators
+ * run one after another, every thread on each (src/serving/start.rs:59-77).
+ *     ellm_side_stream_fork(s, stream);     the side stream waits for what `stream` holds so far
+ *     ... launches with ellm_side_stream_get(s) as their stream ...
+ *     ... launches on `stream` ...
+ *     ellm_side_stream_join(s, stream);     `stream` waits for what the side stream holds so far
+ * Works under ellm_graph_begin / ellm_graph_end too (the side stream's launches
+ * become a parallel branch of the graph; join before ellm_graph_end).  The two
+ * halves must use different handles and write different memory (a handle has one
+ * call in flight), and a fork must be joined before the next fork.  The stream has
+ * the default priority; destroy waits for its work.
+ */
+typedef struct ellm_side_stream ellm_side_stream;
+int ellm_side_stream_create(ellm_side_stream** out_side);
+void* ellm_side_stream_get(ellm_side_stream* side);
+int ellm_side_stream_fork(ellm_side_stream* side, void* stream);
+int ellm_side_stream_join(ellm_side_stream* side, void* stream);
+int ellm_side_stream_destroy(ellm_side_stream* side);
+
 /* positions[i] += by for i < batch_size (device array), in stream order. */
 int ellm_positions_advance(uint32_t* positions, size_t batch_size, uint32_t by, void* stream);
 
