@@ -20,7 +20,8 @@ namespace {
 // Capacity of the static scratch, in the units of ellm::DecodeWorkspace.  A launch with
 // more than one split per K/V plane has at most 2 x compute units workgroups, so
 // (sequences x query heads x splits) <= group size x 2 x compute units partial rows:
-// 8192 rows cover GQA groups of up to 16 query heads on a 256-unit part.
+// 8192 rows cover GQA groups of up to 16 query heads on a 256-unit part whatever the plan,
+// and groups of up to 32 where the plan has one workgroup per unit (most shapes).
 constexpr size_t kRows = 8192;       // split partials   [row][128] + [row][2] floats
 constexpr size_t kRows2 = 1536;      // cluster partials [row][128] + [row][2] floats
 constexpr size_t kCounters = 4096;   // uint32 arrival counters

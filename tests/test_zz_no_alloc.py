@@ -94,8 +94,8 @@ def test_noalloc_rejects_what_the_scratch_cannot_hold():
 
     import ellm_amd
 
-    # GQA groups of 32 query heads on two long planes: 2 x 32 heads x 256 splits = 16384 rows
-    hq, hkv, cap, batch = 32, 1, 65536, 2
+    # GQA groups of 64 query heads on two long planes: 2 x 64 heads x 128 splits = 16384 rows
+    hq, hkv, cap, batch = 64, 1, 65536, 2
     dq = torch.zeros((1, batch, hq, D), dtype=torch.float16, device="cuda")
     dk = torch.zeros((batch, hkv, cap, D), dtype=torch.float16, device="cuda")
     dout = torch.zeros_like(dq)
