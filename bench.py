@@ -32,10 +32,10 @@ HBM_PEAK_GBS = 8000.0       # MI355X HBM3E, published
 # copy of known size; summaries and commands under profiles/).  Not measurable from inside
 # this script; null for workloads without a counter run.
 TRAFFIC_BYTES = {
-    "decode": (2 * 132699 + 4372) * 1024,      # 16 x 8192
-    "decode128k": (2 * 132286 + 4489) * 1024,  # 1 x 131072
+    "decode": (2 * 131928 + 2252) * 1024,      # 16 x 8192
+    "decode128k": (2 * 131745 + 2261) * 1024,  # 1 x 131072
     "lastchunk": (2 * (198592 + 15674) + 31309 + 3120) * 1024,   # 16 tokens x 24: stream kernel + merge launch
-    "mixed_decode": (2 * 2258263 + 5415) * 1024,                 # 32 sequences U{1024..131072}, seed 7
+    "mixed_decode": (2 * 2257752 + 3286) * 1024,                 # 32 sequences U{1024..131072}, seed 7
     "prefill": (1363516 + 319881) * 1024,
     "kvwrite": (73808 + 65536) * 1024,
     "qkv": (1130126 + 327680) * 1024,          # fetched past the L2s (mostly from the last-level cache) + written
