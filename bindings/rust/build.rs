@@ -29,7 +29,7 @@ fn main() {
     for f in [
         "api.hip", "noalloc.hip", "decode.hip", "decode_balanced.hip", "prefill.hip", "kv_cache.hip",
         "project.hip", "project_mid.hip", "project_small.hip", "project_api.hip", "common.hpp",
-        "kernels.hpp", "decode_common.hpp", "decode_shares.hpp", "chunk_plan.hpp", "project_common.hpp",
+        "kernels.hpp", "decode_common.hpp", "decode_plan.hpp", "decode_shares.hpp", "chunk_plan.hpp", "project_common.hpp",
         "project_epilogue.hpp", "Makefile",
     ] {
         println!("cargo:rerun-if-changed={}", csrc.join(f).display());

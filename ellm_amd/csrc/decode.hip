@@ -112,65 +112,6 @@ __global__ __launch_bounds__(kDecThreads, 4) void decode_split_kernel(DecodeKern
 
 }  // namespace
 
-DecodePlan decode_plan(uint32_t max_len, uint32_t batch, uint32_t n_kv_heads, uint32_t n_cu) {
-  // Every plane is cut into the same number of splits.  Each workgroup has fixed costs (query
-  // load, wave merge, partial write, arrival) that more, shorter workgroups pay more often, and
-  // one workgroup alone on a compute unit streams a little faster than each of two that share
-  // it, so one workgroup per unit is the first choice (measured against two per unit: 16 x 8192
-  // keys 45.5 against 46.4 us, 1 x 131072 46.4 against 48.1, 4 x 32768 44.8 against 47.8,
-  // 64 x 2048 42.8 against 46.6).  Where the planes do not divide the units well, two per unit
-  // waste less (24 x 8192: 96 planes, 2 splits = 192 workgroups on 256 units, or 5 splits = 480
-  // on 2 x 256): the plan with the shorter estimated time is taken, time = keys per split x
-  // workgroups on the busiest unit (x 1.03 when units are shared).  Splits are rounded down in
-  // number: a few workgroups beyond a whole round make some units host one more, and those
-  // finish that much later (20 x 8192: 67 us with 560 workgroups, 57 us with 480).  Never
-  // shorter than four 64-key steps.
-  const uint32_t planes = batch * n_kv_heads;
-  // both merge levels fold at most 16 partials: at most 16 * 16 splits per plane
-  const uint32_t floor_len =
-      ((max_len + kMergeFan * kMergeFan - 1) / (kMergeFan * kMergeFan) + kDecodeStepKeys - 1) /
-      kDecodeStepKeys * kDecodeStepKeys;
-  auto plan_for = [&](uint32_t per_cu, uint64_t* cost) {
-    const uint32_t target = n_cu * per_cu;
-    const uint32_t want = target / planes > 0 ? target / planes : 1;
-    uint32_t split_len = (max_len + want - 1) / want;
-    split_len = (split_len + kDecodeStepKeys - 1) / kDecodeStepKeys * kDecodeStepKeys;
-    if (split_len < 4 * kDecodeStepKeys) split_len = 4 * kDecodeStepKeys;
-    if (split_len < floor_len) split_len = floor_len;
-    DecodePlan plan;
-    plan.split_len = split_len;
-    plan.n_split = (max_len + split_len - 1) / split_len;
-    const uint64_t on_busiest = ((uint64_t)planes * plan.n_split + n_cu - 1) / n_cu;
-    *cost = (uint64_t)split_len * on_busiest * (on_busiest > 1 ? 103 : 100);
-    return plan;
-  };
-  uint64_t cost_one = 0, cost_two = 0;
-  const DecodePlan one = plan_for(1, &cost_one), two = plan_for(2, &cost_two);
-  return cost_one <= cost_two ? one : two;
-}
-
-DecodeWorkspace decode_workspace(uint32_t batch_capacity, uint32_t n_q_heads, uint32_t n_kv_heads,
-                                 uint32_t n_cu) {
-  // rows = batch * heads * n_split with n_split <= ceil(4*n_cu / (batch*kv_heads))
-  const size_t group = n_q_heads / n_kv_heads;
-  DecodeWorkspace w;
-  w.rows = (size_t)batch_capacity * n_q_heads + (size_t)n_cu * 16 * group;
-  // cluster partials: ceil(n_split / 16) per row of batch * heads
-  w.rows2 = w.rows / kMergeFan + (size_t)batch_capacity * n_q_heads;
-  // counters: (1 + clusters) per plane, planes <= batch * heads
-  w.counters = w.rows2 + (size_t)batch_capacity * n_q_heads;
-  return w;
-}
-
-bool decode_plan_fits(const DecodeWorkspace& w, uint32_t batch, uint32_t n_q_heads,
-                      uint32_t n_kv_heads, uint32_t group, uint32_t n_split) {
-  const size_t n_cluster = (n_split + kMergeFan - 1) / kMergeFan;
-  const size_t head_groups = (group + kMaxHeadsPerGroup - 1) / kMaxHeadsPerGroup;
-  return (size_t)batch * n_q_heads * n_split <= w.rows &&
-         (size_t)batch * n_q_heads * n_cluster <= w.rows2 &&
-         (size_t)batch * n_kv_heads * head_groups * (1 + n_cluster) <= w.counters;
-}
-
 hipError_t launch_decode(const AttnArgs& a, hipStream_t stream) {
   DecodeKernelArgs p;
   p.q = (const uint16_t*)a.q;

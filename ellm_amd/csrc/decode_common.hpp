@@ -17,7 +17,9 @@ constexpr int kKPitch = kHeadDim + 8;           // halves per K row in LDS (272 
 constexpr int kVtPitch = kChunk + 4;            // halves per V^T row in LDS (40 B)
 constexpr int kWaveLdsHalves = kChunk * kKPitch + kHeadDim * kVtPitch;
 constexpr int kMaxHeadsPerGroup = 16;
+static_assert(kMaxHeadsPerGroup == (int)kPlanMaxHeadsPerGroup, "decode_plan.hpp sizes the workspace for this group");
 constexpr int kMergeFan = 16;                   // partials folded per merge step
+static_assert(kMergeFan == (int)kPlanMergeFan, "decode_plan.hpp sizes the workspace for this fan");
 constexpr int kQuads = kHeadDim / 4;
 constexpr int kItems = kMaxHeadsPerGroup * kQuads / kDecThreads;  // (head, four columns) items per thread
 constexpr int kRedPitch = kHeadDim + 4;         // floats per (wave, head) row of the wave merge, 16-byte aligned

@@ -5,6 +5,8 @@
 #include <stddef.h>
 #include <stdint.h>
 
+#include "decode_plan.hpp"
+
 struct ellm_attn_desc;
 
 namespace ellm {
@@ -53,26 +55,6 @@ struct AttnArgs {
 // Partial rows the chunk path's workspace holds for an operator of this shape (0: none needed).
 size_t prefill_workspace_rows(uint32_t max_interval, uint32_t batch_capacity, uint32_t n_q_heads,
                               uint32_t n_cu);
-
-// Keys handled by one workgroup step of the single-token kernel.
-constexpr uint32_t kDecodeStepKeys = 64;
-struct DecodePlan {
-  uint32_t split_len;
-  uint32_t n_split;
-};
-DecodePlan decode_plan(uint32_t max_len, uint32_t batch, uint32_t n_kv_heads, uint32_t n_cu);
-
-// Sizes (in partial rows / counters) that cover every plan decode_plan() can
-// return for up to batch_capacity sequences.
-struct DecodeWorkspace {
-  size_t rows;      // first-level partials  (x 128 and x 2 floats)
-  size_t rows2;     // cluster partials      (x 128 and x 2 floats)
-  size_t counters;  // uint32 arrival counters
-};
-DecodeWorkspace decode_workspace(uint32_t batch_capacity, uint32_t n_q_heads, uint32_t n_kv_heads,
-                                 uint32_t n_cu);
-bool decode_plan_fits(const DecodeWorkspace& w, uint32_t batch, uint32_t n_q_heads,
-                      uint32_t n_kv_heads, uint32_t group, uint32_t n_split);
 
 hipError_t launch_decode(const AttnArgs& a, hipStream_t stream);
 // Per-sequence positions, the planes' keys dealt evenly to `wgs` workgroups (decode_balanced.hip):
