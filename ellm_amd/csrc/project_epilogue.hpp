@@ -13,8 +13,10 @@ typedef __attribute__((address_space(3))) u32x4 LdsVec4;
 typedef __attribute__((address_space(3))) u32x2 LdsVec2;
 typedef __attribute__((address_space(3))) uint64_t LdsU64;
 
-constexpr int kEpPitch = kHeadDim * 2 + 16;           // output row in LDS
-constexpr int kEpWaveBytes = 32 * kEpPitch + 32 * 8;  // 32 rows and their destinations, per wave
+constexpr int kEpPitch = kHeadDim * 2 + 16;           // a 256-byte row in LDS
+constexpr int kEpWaveBytes = 2 * 32 * kEpPitch;       // per wave: 32 output rows and 32 rows of the extra operand
+
+typedef __attribute__((address_space(1))) u32x4 GlobalVec4;
 
 // acc[nb][mb]: column block nb (32 columns) x token block mb (32 tokens) of head `hh`;
 // `first_row` is the row of the activations that token block 0, lane row 0 stands for;
@@ -22,30 +24,55 @@ constexpr int kEpWaveBytes = 32 * kEpPitch + 32 * 8;  // 32 rows and their desti
 // In the accumulator layout lane (j, g) holds, for token 32 mb + j, the
 // columns 32 nb + 8 b + 4 g + (0..3) of the head: four consecutive columns = two rotation
 // pairs = one 8-byte piece of the rotary row, of the residual row and of the output
-// row; lanes l and l ^ 32 together own the token's 128 columns.  The extra operand
-// (table or residual) of token block mb + 1 is requested before block mb is worked on.
+// row; lanes l and l ^ 32 together own the token's 128 columns.
+// Memory is touched in whole rows only, in both directions: a wave instruction moves four
+// 256-byte rows (16 lanes a row), and LDS turns rows into the accumulator layout and back.
+// (Fetching the extra operand in the accumulator layout directly, 8 bytes a lane from 32
+// different rows per instruction, cost the vector cache 32 line look-ups an instruction and
+// 200 cycles each: 1.3 us a token block on a wave that has nothing else to run.)  Which row
+// a lane moves is lane / 16 + 4 i; the row's address comes from the lane that owns the token
+// through a lane permute.  The extra operand (table or residual) of token block mb + 2 is
+// requested while block mb is worked on, ahead of block mb's stores.
 // One code path: a head that is not normalised and rotated runs the same arithmetic
 // with scale 1 and the rotation (cos, sin) = (1, 0), which leaves every value as it is.
-// Where the rows of one head x 32 MB tokens go and what is combined with them, plus the extra
-// operand of token block 0, already requested: a kernel with registers to spare calls
+// HeadRows: where the rows of one head x 32 MB tokens go and what is combined with them, plus
+// the extra operand of token block 0, already requested: a kernel with registers to spare calls
 // prepare_head() ahead of its main loop, so that neither the positions nor the first table /
 // residual rows are waited for after it.
 template <int MB>
 struct HeadRows {
-  uint16_t* out_row[MB];
-  const uint16_t* ext_row[MB];
-  bool live[MB];
+  uint16_t* out_row[MB];        // this lane's token: destination row (g == 0 and g == 1 alike)
+  const uint16_t* ext_row[MB];  // ... and row of the extra operand; null: none (scale 1, no rotation)
   bool present;    // false: the head lies beyond the last one (odd head count), nothing to do
   bool finalize;   // normalise + rotate
-  u32x2 ext0[16];
+  u32x4 ext0[8];   // token block 0's extra rows as fetched: piece lane % 16 of rows lane / 16 + 4 i
 };
+
+// The 64-bit value that lane `from` holds (every lane names its own source lane).
+__device__ __forceinline__ uint64_t from_lane(uint64_t v, int from) {
+  const uint32_t lo = (uint32_t)__builtin_amdgcn_ds_bpermute(4 * from, (int)(uint32_t)v);
+  const uint32_t hi = (uint32_t)__builtin_amdgcn_ds_bpermute(4 * from, (int)(uint32_t)(v >> 32));
+  return ((uint64_t)hi << 32) | lo;
+}
+
+// Rows lane / 16 + 4 i, i = 0..7, of the extra operand of one token block; rows without one
+// read as (1, 0) pairs.
+template <typename S>
+__device__ __forceinline__ void fetch_ext_rows(const uint16_t* my_row, int lane, u32x4 (&v)[8]) {
+  const uint32_t one_zero = Mfma<S>::pack2(1.0f, 0.0f);
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    const uint64_t row = from_lane((uint64_t)my_row, 4 * i + (lane >> 4));
+    v[i] = u32x4{one_zero, one_zero, one_zero, one_zero};
+    if (row) v[i] = *(const GlobalVec4*)(row + 16 * (lane & 15));
+  }
+}
 
 template <typename S, int MODE, int MB>
 __device__ __forceinline__ HeadRows<MB> prepare_head(const ProjectKernelArgs& p, uint32_t hh,
                                                      uint32_t first_row, int lane) {
-  using M = Mfma<S>;
   HeadRows<MB> h;
-  const int j = lane & 31, g = lane >> 5;
+  const int j = lane & 31;
   const uint32_t heads_total = p.heads0 + 2 * p.heads_kv;
   h.present = hh < heads_total;
   const uint32_t seg = (hh < p.heads0) ? 0u : (hh < p.heads0 + p.heads_kv ? 1u : 2u);
@@ -56,30 +83,24 @@ __device__ __forceinline__ HeadRows<MB> prepare_head(const ProjectKernelArgs& p,
   for (int mb = 0; mb < MB; ++mb) {
     const uint32_t R = first_row + 32 * mb + j;
     const uint32_t t = R / p.batch_pitch, b = R % p.batch_pitch;
-    h.live[mb] = h.present && R < p.rows && b < p.batch;
+    const bool live = h.present && R < p.rows && b < p.batch;
     uint32_t pos = t;
     if (p.positions)
-      pos += h.live[mb] ? min(p.positions[b], p.max_start) : 0u;
+      pos += live ? min(p.positions[b], p.max_start) : 0u;
     else
       pos += p.position_index;
     const size_t col = hs * kHeadDim;
-    if (seg == 0)
-      h.out_row[mb] = dst + (size_t)R * p.ld0 + col;
-    else
-      h.out_row[mb] = dst + (h.live[mb] ? kv_row_offset(p, b, hs, pos) : (size_t)0);
-    if (MODE == kModeQkv)
-      h.ext_row[mb] = p.rope + (size_t)pos * p.rope_pos_stride + (size_t)hs * p.rope_head_stride + 4 * g;
-    else
-      h.ext_row[mb] = p.residual + (size_t)R * p.ld0 + col + 4 * g;
+    h.out_row[mb] = nullptr;
+    h.ext_row[mb] = nullptr;
+    if (live) {
+      h.out_row[mb] = (seg == 0) ? dst + (size_t)R * p.ld0 + col : dst + kv_row_offset(p, b, hs, pos);
+      if (MODE == kModeAdd)
+        h.ext_row[mb] = p.residual + (size_t)R * p.ld0 + col;
+      else if (h.finalize)
+        h.ext_row[mb] = p.rope + (size_t)pos * p.rope_pos_stride + (size_t)hs * p.rope_head_stride;
+    }
   }
-  const uint32_t one_zero = M::pack2(1.0f, 0.0f);
-  if ((MODE == kModeAdd || h.finalize) && h.live[0]) {
-#pragma unroll
-    for (int i = 0; i < 16; ++i) h.ext0[i] = *(const u32x2*)(h.ext_row[0] + 32 * (i >> 2) + 8 * (i & 3));
-  } else {
-#pragma unroll
-    for (int i = 0; i < 16; ++i) h.ext0[i] = u32x2{one_zero, one_zero};
-  }
+  fetch_ext_rows<S>(h.ext_row[0], lane, h.ext0);
   return h;
 }
 
@@ -90,28 +111,26 @@ __device__ __forceinline__ void finish_head(const ProjectKernelArgs& p, f32x16 (
   const int j = lane & 31, g = lane >> 5;
   if (!h.present) return;
   const bool finalize = h.finalize;
-  const auto& out_row = h.out_row;
-  const auto& ext_row = h.ext_row;
-  const auto& live = h.live;
-  const uint32_t ep_table = ep_rows + 32 * kEpPitch;
-  const uint32_t one_zero = M::pack2(1.0f, 0.0f);
-  u32x2 ext[2][16];
-  auto fetch_ext = [&](auto set, int mb) {
-    if ((MODE == kModeAdd || finalize) && live[mb]) {
+  const uint32_t ep_ext = ep_rows + 32 * kEpPitch;
+  // this lane's place as a mover of whole rows (row lane / 16 + 4 i, piece lane % 16) and as the
+  // owner of token j (8-byte pieces at columns 32 nb + 8 b + 4 g)
+  const uint32_t row_piece = (lane >> 4) * kEpPitch + 16 * (lane & 15);
+  const uint32_t own_piece = j * kEpPitch + 8 * g;
+  u32x4 raw[8];
 #pragma unroll
-      for (int i = 0; i < 16; ++i) ext[set][i] = *(const u32x2*)(ext_row[mb] + 32 * (i >> 2) + 8 * (i & 3));
-    } else {
+  for (int i = 0; i < 8; ++i) raw[i] = h.ext0[i];
+  // the extra rows of a block go into LDS as soon as the block before has read its own out of it,
+  // and the block after is requested: both ahead of that block's stores, so that a wait for
+  // the rows never includes stores (the compiler cannot count conditional stores and waits for all)
+  auto stage_ext = [&](int next) __attribute__((always_inline)) {
 #pragma unroll
-      for (int i = 0; i < 16; ++i) ext[set][i] = u32x2{one_zero, one_zero};
-    }
+    for (int i = 0; i < 8; ++i) *(LdsVec4*)(ep_ext + row_piece + 4 * i * kEpPitch) = raw[i];
+    if (next < MB) fetch_ext_rows<S>(h.ext_row[next < MB ? next : 0], lane, raw);
   };
-#pragma unroll
-  for (int i = 0; i < 16; ++i) ext[0][i] = h.ext0[i];
+  stage_ext(1);
   static_for<MB>([&](auto mb_) {
     constexpr int mb = decltype(mb_)::value;
-    constexpr int set = mb & 1;
     __builtin_amdgcn_sched_barrier(0);  // one token block's accumulators at a time leave the AGPRs
-    if constexpr (mb + 1 < MB) fetch_ext(std::integral_constant<int, 1 - set>{}, mb + 1);
     float inv = 1.0f;
     if (MODE == kModeQkv) {
       float ss = 0.0f;
@@ -122,13 +141,16 @@ __device__ __forceinline__ void finish_head(const ProjectKernelArgs& p, f32x16 (
       ss = sum_with_partner_half(ss);
       inv = finalize ? 1.0f / (sqrtf(ss / (float)kHeadDim) + p.eps) : 1.0f;
     }
+    u32x2 ext[16];
+#pragma unroll
+    for (int i = 0; i < 16; ++i) ext[i] = *(const LdsVec2*)(ep_ext + own_piece + 2 * (32 * (i >> 2) + 8 * (i & 3)));
     u32x2 packed[16];
 #pragma unroll
     for (int i = 0; i < 16; ++i) {
       const int nb = i >> 2, b4 = i & 3;
       float o0 = acc[nb][mb][4 * b4], o1 = acc[nb][mb][4 * b4 + 1];
       float o2 = acc[nb][mb][4 * b4 + 2], o3 = acc[nb][mb][4 * b4 + 3];
-      const u32x2 rr = ext[set][i];
+      const u32x2 rr = ext[i];
       const float e0 = M::to_float((uint16_t)(rr[0] & 0xffffu)), e1 = M::to_float((uint16_t)(rr[0] >> 16));
       const float e2 = M::to_float((uint16_t)(rr[1] & 0xffffu)), e3 = M::to_float((uint16_t)(rr[1] >> 16));
       if (MODE == kModeQkv) {
@@ -145,19 +167,22 @@ __device__ __forceinline__ void finish_head(const ProjectKernelArgs& p, f32x16 (
       }
       packed[i] = u32x2{M::pack2(o0, o1), M::pack2(o2, o3)};
     }
-    // out through LDS so that a store instruction covers whole 256-byte rows: the lane
-    // that owns token j also leaves the row's destination (0: nothing to write)
-    if (g == 0) *(LdsU64*)(ep_table + 8 * j) = live[mb] ? (uint64_t)out_row[mb] : 0ull;
+    // out through LDS: the owner of a token leaves its row there, the movers of whole rows pick
+    // up all eight of theirs before the first store
 #pragma unroll
     for (int i = 0; i < 16; ++i)
-      *(LdsVec2*)(ep_rows + j * kEpPitch + 2 * (32 * (i >> 2) + 8 * (i & 3) + 4 * g)) = packed[i];
+      *(LdsVec2*)(ep_rows + own_piece + 2 * (32 * (i >> 2) + 8 * (i & 3))) = packed[i];
+    if constexpr (mb + 1 < MB) stage_ext(mb + 2);
+    uint64_t to[8];
+    u32x4 v[8];
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
-      const uint32_t row = 4 * i + (lane >> 4);
-      uint16_t* const to = (uint16_t*)*(const LdsU64*)(ep_table + 8 * row);
-      const u32x4 v = *(const LdsVec4*)(ep_rows + row * kEpPitch + 16 * (lane & 15));
-      if (to) store16(to + 8 * (lane & 15), v);
+      to[i] = from_lane((uint64_t)h.out_row[mb], 4 * i + (lane >> 4));   // 0: nothing to write
+      v[i] = *(const LdsVec4*)(ep_rows + row_piece + 4 * i * kEpPitch);
     }
+#pragma unroll
+    for (int i = 0; i < 8; ++i)
+      if (to[i]) *(GlobalVec4*)(to[i] + 16 * (lane & 15)) = v[i];
   });
 }
 
