@@ -336,7 +336,8 @@ static void fill_args(const ellm_attn* h, ellm::AttnArgs* a) {
   a->seq_caps = h->seq_caps;
 }
 
-// sequences of different lengths: equal shares of all keys, two workgroups per compute unit
+// sequences of different lengths: equal shares of all keys; two workgroups per compute unit are
+// launched, and the kernel lets one or two per unit take part (it knows the lengths)
 static bool takes_balanced(const ellm_attn* h, size_t batch, size_t max_position, uint32_t* wgs) {
   *wgs = 2 * (uint32_t)h->n_cu;
   const ellm_attn_desc& d = h->desc;
