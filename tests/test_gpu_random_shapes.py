@@ -1,7 +1,9 @@
 """Seeded sweep of chunk attention shapes against the CPU oracle through the C ABI: head layouts,
 batch below capacity, chunk lengths either side of the kernels' row limits (128 / 256 / 384 query
 rows per K/V plane), cached lengths on and off tile edges.  The shapes are drawn so that the
-planner splits the key range evenly, unevenly and not at all."""
+planner splits the key range evenly, unevenly and not at all.  Below them: single-token steps over
+sequences of different lengths, and uniform single-token steps over the split plans (one or two
+workgroups per compute unit, one to hundreds of splits per plane, one and two fold levels)."""
 import numpy as np
 import pytest
 
@@ -102,3 +104,34 @@ def test_random_ragged_single_token_steps_match_oracle(block):
         res = compare(got, orc.from_storage(want, dtype), dtype)
         assert res["ok"], (c, res)
         assert float(np.abs(got_lse - want_lse).max()) <= LSE_TOL, c
+
+
+# (sequences, kv heads, group, cached positions): shapes whose planes divide the compute units
+# and shapes that do not, one to hundreds of splits per plane, one and two fold levels
+UNIFORM_STEPS = [
+    (20, 4, 2, 8192),    # 80 planes: 3 splits, one workgroup per unit
+    (24, 4, 2, 4096),    # 96 planes: 5 splits, two per unit
+    (3, 1, 8, 40000),    # 3 planes: 79 splits, five clusters to fold
+    (7, 2, 4, 5000),     # 14 planes: a full cluster of 16 splits
+    (1, 2, 4, 70000),    # 2 planes: 122 splits
+    (33, 4, 2, 3000),    # 132 planes: 3 splits, two per unit
+    (100, 4, 1, 1024),   # more planes than units: no split
+    (64, 1, 16, 2048),   # 64 planes x 4, sixteen heads a group
+]
+
+
+@pytest.mark.parametrize("case", UNIFORM_STEPS, ids=["%dx%dx%d_%d" % c for c in UNIFORM_STEPS])
+def test_uniform_single_token_steps_over_split_plans(case):
+    b, hkv, g, cached = case
+    dtype = orc.F16 if (b + cached) % 2 == 0 else orc.BF16
+    hq = hkv * g
+    print("case", case, "f16" if dtype == orc.F16 else "bf16", flush=True)
+    q = rand_storage((1, b, hq, D), 31, dtype)
+    k = rand_storage((b, hkv, cached, D), 32, dtype)
+    v = rand_storage((b, hkv, cached, D), 33, dtype)
+    scale = 1.0 / np.sqrt(D)
+    want, want_lse = orc.attention(q, k, v, scale, dtype, position_index=cached - 1)
+    got, got_lse = gpu_attention(q, k, v, scale, dtype, position_index=cached - 1)
+    res = compare(got, orc.from_storage(want, dtype), dtype)
+    assert res["ok"], (case, res)
+    assert float(np.abs(got_lse - want_lse).max()) <= LSE_TOL, case
