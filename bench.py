@@ -577,65 +577,106 @@ def bench_step_projections(batch, steps, warmup, hidden=2048, hq=32, hkv=4, copi
             "o_ms": o_ms, "o_kernel_ms": per[0], "o_bytes": o_bytes}
 
 
-def bench_layer_step(layers, batch, length, steps, warmup, hidden=2048, hq=32, hkv=4):
+def bench_layer_steps(layers, cases, steps, warmup, hidden=2048, hq=32, hkv=4):
     """The attention block of every layer for one new token per sequence: fused Q/K/V projection
     (norm + rotation, K/V written into the cache), attention over the cache, output projection +
     residual; every layer has its own weights and cache; positions advance on the device.
-    Issued launch by launch and replayed from a graph recorded once through the library."""
+    Issued launch by launch and replayed from a graph recorded once through the library.
+    cases: (sequences, cached tokens) pairs; the layers' weights are made once and shared by the
+    cases, every case has its own caches."""
     import torch
 
     import ellm_amd
 
     dt = torch.float16
-    cap = length + 2 * (steps + warmup) + 8
     scale = 1.0 / D ** 0.5
     stream = torch.cuda.Stream()
-    cache = ellm_amd.KVCache(layers, batch, hkv, cap, ellm_amd.DTYPE_F16)
-    j = torch.arange(D // 2, device="cuda", dtype=torch.float64)
-    ang = torch.arange(cap, device="cuda", dtype=torch.float64)[:, None] * (1.0e6 ** (-2.0 * j / D))[None, :]
-    rope = torch.stack((torch.cos(ang), torch.sin(ang)), dim=-1).reshape(cap, D).to(dt)
-    x = [_dev_normal((1, batch, hidden), dt, 501), torch.zeros((1, batch, hidden), dtype=dt, device="cuda")]
-    q = torch.zeros((1, batch, hq, D), dtype=dt, device="cuda")
-    att = torch.zeros_like(q)
-    ops, keep = [], []
+    keep = []
     for layer in range(layers):
-        kt, vt = cache.layer_tensors(layer, dt)
-        kt.normal_()
-        vt.normal_()
-        _, _, strides = cache.layer(layer)
         w = [_dev_normal((h * D, hidden), dt, 600 + 4 * layer + i, scale=hidden ** -0.5) for i, h in enumerate((hq, hkv, hkv))]
         wo = _dev_normal((hidden, hq * D), dt, 603 + 4 * layer, scale=(hq * D) ** -0.5)
         keep.append((w, wo))
-        src, dst = x[layer & 1], x[1 - (layer & 1)]
-        ops.append((ellm_amd.MatMul3(src, w[0], q, w[1], kt, w[2], vt, rope, D, batch, hq, hkv, strides, cap),
-                    ellm_amd.Attention(q, kt, vt, att, batch, hq, hkv, D, strides, scale,
-                                       sequence_capacity=cap, max_position_interval=1),
-                    ellm_amd.MatMulAdd(att.view(1, batch, hq * D), wo, src, dst)))
-    pos = torch.full((batch,), length - 1, dtype=torch.int32, device="cuda")
-    torch.cuda.synchronize()
+    results = {}
+    for batch, length in cases:
+        n_steps = min(steps, 20)
+        cap = length + 512     # positions advance once per step; the kernels clamp them to cap - 1
+        cache = ellm_amd.KVCache(layers, batch, hkv, cap, ellm_amd.DTYPE_F16)
+        j = torch.arange(D // 2, device="cuda", dtype=torch.float64)
+        ang = torch.arange(cap, device="cuda", dtype=torch.float64)[:, None] * (1.0e6 ** (-2.0 * j / D))[None, :]
+        rope = torch.stack((torch.cos(ang), torch.sin(ang)), dim=-1).reshape(cap, D).to(dt)
+        x = [_dev_normal((1, batch, hidden), dt, 501), torch.zeros((1, batch, hidden), dtype=dt, device="cuda")]
+        q = torch.zeros((1, batch, hq, D), dtype=dt, device="cuda")
+        att = torch.zeros_like(q)
+        ops = []
+        for layer in range(layers):
+            kt, vt = cache.layer_tensors(layer, dt)
+            kt.normal_()
+            vt.normal_()
+            _, _, strides = cache.layer(layer)
+            w, wo = keep[layer]
+            src, dst = x[layer & 1], x[1 - (layer & 1)]
+            ops.append((ellm_amd.MatMul3(src, w[0], q, w[1], kt, w[2], vt, rope, D, batch, hq, hkv, strides, cap),
+                        ellm_amd.Attention(q, kt, vt, att, batch, hq, hkv, D, strides, scale,
+                                           sequence_capacity=cap, max_position_interval=1),
+                        ellm_amd.MatMulAdd(att.view(1, batch, hq * D), wo, src, dst)))
+        pos = torch.full((batch,), length - 1, dtype=torch.int32, device="cuda")
+        torch.cuda.synchronize()
 
-    def step(_=None):
-        for qkv, attn, oproj in ops:
-            qkv.run_ragged(pos, cap - 1, batch)
-            attn.run_ragged(pos, cap - 1, batch)
-            oproj.run(0, 1, batch)
-        ellm_amd.positions_advance(pos, 1)
+        def step(_=None):
+            for qkv, attn, oproj in ops:
+                qkv.run_ragged(pos, cap - 1, batch)
+                attn.run_ragged(pos, cap - 1, batch)
+                oproj.run(0, 1, batch)
+            ellm_amd.positions_advance(pos, 1)
 
-    with torch.cuda.stream(stream):
-        _, eager_ms = _time_steps(step, steps, warmup)
-        pos.fill_(length - 1)
-        stream.synchronize()
-        with ellm_amd.StepGraph(stream) as graph:
-            step()
-        _, graph_ms = _time_steps(lambda _i: graph.launch(), steps, warmup)
-    graph.close()
-    for group in ops:
-        for op in group:
-            op.close()
-    cache.close()
-    kv_bytes = layers * (2 * batch * hkv * length * D * 2)
-    w_bytes = layers * ((hq + 2 * hkv) * D * hidden * 2 + hidden * hq * D * 2)
-    return {"eager_ms": eager_ms, "graph_ms": graph_ms, "kv_bytes": kv_bytes, "w_bytes": w_bytes}
+        # short steps: fewer timed passes, so that the positions stay near `length`
+        min_ms = MIN_TIMED_MS if length >= 4096 else 30.0
+        with torch.cuda.stream(stream):
+            _, eager_ms = _time_steps(step, n_steps, warmup, min_ms=min_ms)
+            pos.fill_(length - 1)
+            stream.synchronize()
+            with ellm_amd.StepGraph(stream) as graph:
+                step()
+            dev, graph_ms = _time_steps(lambda _i: graph.launch(), n_steps, warmup, min_ms=min_ms)
+        graph.close()
+        for group in ops:
+            for op in group:
+                op.close()
+        cache.close()
+        del rope, ang
+        kv_bytes = layers * (2 * batch * hkv * length * D * 2)
+        w_bytes = layers * ((hq + 2 * hkv) * D * hidden * 2 + hidden * hq * D * 2)
+        results[(batch, length)] = {"eager_ms": eager_ms, "graph_ms": graph_ms, "graph_dev_ms": dev[0],
+                                    "kv_bytes": kv_bytes, "w_bytes": w_bytes, "steps": n_steps}
+    return results
+
+
+def cpu_baseline_layer_step(batch, length, layers=48, hidden=2048, hq=32, hkv=4):
+    """One layer's attention block of a single-token step on the CPU oracle (fused Q/K/V projection,
+    attention over the cache, output projection + residual: the oracle's scalar restatements, one
+    thread), times the layer count."""
+    import numpy as np
+    import oracle_lib as orc
+
+    cap = length
+    x = _cpu_normal((1, batch, hidden), "f16", 31)
+    w = [_cpu_normal((h * D, hidden), "f16", 32 + i) for i, h in enumerate((hq, hkv, hkv))]
+    wo = _cpu_normal((hidden, hq * D), "f16", 36)
+    k = _cpu_normal((batch, hkv, cap, D), "f16", 37)
+    v = _cpu_normal((batch, hkv, cap, D), "f16", 38)
+    ang = np.arange(cap)[:, None] * (1.0e6 ** (-2.0 * np.arange(D // 2) / D))[None, :]
+    rope32 = np.empty((cap, D), dtype=np.float32)
+    rope32[:, 0::2], rope32[:, 1::2] = np.cos(ang), np.sin(ang)
+    rope = orc.to_storage(rope32, orc.F16)
+    q = np.zeros((1, batch, hq, D), dtype=np.float16)
+    strides = [hkv * cap * D, cap * D, D, 1]
+    t0 = time.perf_counter()
+    assert orc.matmul3(x, w[0], w[1], w[2], q, k, v, rope, strides, cap, length - 1, 1, orc.F16) == 0
+    att, _ = orc.attention(q, k, v, 1.0 / D ** 0.5, orc.F16, position_index=length - 1, n_threads=1)
+    orc.matmul_add(att.reshape(1, batch, hq * D), wo, x, orc.F16)
+    t = time.perf_counter() - t0
+    return {"value": round(t * layers * 1e3, 2), "unit": "ms", "cores": 1, "kind": "port",
+            "sample": f"one layer of {layers} on one thread ({t * 1e3:.1f} ms), x {layers}"}
 
 
 def bench_chunk_block(positions, batch, p0, steps, warmup, hidden=2048, hq=32, hkv=4):
@@ -749,8 +790,7 @@ def cpu_baseline_decode(batch, length, hq=32, hkv=4, budget_s=1.5):
         "cores": cores,
         "kind": "port",
         "pinned": True,
-        "sample": f"full workload ({batch} seq x {length} keys x {hq} heads), {repeats} passes, "
-                  f"{t * 1e3:.1f} ms per pass, one pinned thread per core with the reference's static split",
+        "sample": f"full workload, {repeats} passes, {t * 1e3:.1f} ms per pass, one pinned thread per core",
     }
 
 
@@ -807,9 +847,8 @@ def cpu_baseline_chunk(seq, p0, hq, hkv, dtype_name, budget_s=1.5, seed=17):
         "cores": cores,
         "kind": "port",
         "pinned": True,
-        "sample": f"{n} seeded (token, head) rows of the {seq}-token chunk, {macs / 1e9:.2f} of "
-                  f"{full_macs / 1e9:.0f} G multiply-adds in {t:.2f} s on {cores} pinned threads; the whole "
-                  f"chunk extrapolated by multiply-add count (x {factor:.0f}) would take {t * factor:.0f} s",
+        "sample": f"{n} seeded (token, head) rows, {macs / 1e9:.2f} of {full_macs / 1e9:.0f} G multiply-adds in "
+                  f"{t:.2f} s; x {factor:.0f} by multiply-add count",
         "extrapolation_factor": factor,
         "seconds_extrapolated": t * factor,
     }
@@ -844,8 +883,7 @@ def cpu_baseline_ragged_decode(lengths, hq=32, hkv=4, sample_seqs=4, seed=19):
         "cores": cores,
         "kind": "port",
         "pinned": True,
-        "sample": f"{b} of the {len(lengths)} sequences (cache lengths {lens.tolist()}), all {hq} heads, "
-                  f"{t * 1e3:.0f} ms on {cores} pinned threads; extrapolated by cached-token count (x {factor:.2f})",
+        "sample": f"{b} of {len(lengths)} sequences, all heads, {t * 1e3:.0f} ms; x {factor:.2f} by cached-token count",
         "extrapolation_factor": factor,
         "seconds_extrapolated": t * factor,
     }
@@ -925,10 +963,15 @@ def main():
         del src, dst
 
     also = []
+    last_entries = []   # the two headline targets: appended last, where a truncated record still shows them
+    targets = {}        # compact copies of the headline figures, inside the line's `roofline` object
     dec = None
     host = _host_info()
     if args.only in ("", "decode"):
         dec = bench_decode(16, 8192, args.steps, args.warmup)
+        targets["decode_16x8192"] = {
+            "us": round(dec["kernel_ms"] * 1e3, 2), "gbs": round(dec["kernel_gbs"], 1),
+            "frac": round(dec["kernel_gbs"] / HBM_PEAK_GBS, 4), "target_frac": 0.7}
     if args.only in ("", "prefill"):
         pf_steps = max(3, min(args.steps, 10))
         pf = bench_prefill(32768, pf_steps, min(args.warmup, 2), zero_kv=args.prefill_zero_kv, power_seconds=1.0)
@@ -945,27 +988,27 @@ def main():
         stream_reg0 = bench_mfma_stream(0, "f16", n_cu, seconds=0.3, zeros=True)
         stream_lds0 = bench_mfma_stream(1, "f16", n_cu, seconds=0.3, zeros=True)
         pf_cpu = None if args.skip_cpu else cpu_baseline_chunk(32768, 0, 32, 4, "f16")
-        also.append({
-            "workload": "prefill: 1 seq x 32768 tokens, 32q/4kv heads, fp16, causal"
+        last_entries.append({
+            "workload": "prefill: 1 seq x 32768 tokens, 32q/4kv heads, fp16, causal (configs[2])"
                         + (" [DIAGNOSTIC: K = V = 0]" if args.prefill_zero_kv else ""),
             "metric": "prefill attn TFLOP/s", "value": round(pf["tflops"], 2), "unit": "TFLOP/s",
-            "ms_per_step": round(pf["ms_per_step"], 4), "steps": pf_steps,
+            "ms_per_step": round(pf["ms_per_step"], 4), "kernel_ms": round(pf["kernel_ms"], 4), "steps": pf_steps,
             "roofline": {"bound": "mfma", "achieved": round(pf["kernel_tflops"], 2),
                          "peak": MFMA_F16_PEAK_TFLOPS, "unit": "TFLOP/s",
                          "frac": round(pf["kernel_tflops"] / MFMA_F16_PEAK_TFLOPS, 4),
                          "traffic": TRAFFIC_BYTES["prefill"]},
             "passes": pf["passes"],
+            # board power / engine clock (hwmon, 20 ms samples, 1 s after the timed passes) for this
+            # launch and for the same launch on K = V = 0
             "board_power": {
-                "what": "board power and engine clock from the driver's hwmon files, sampled every 20 ms while the "
-                        "launch is repeated for a second right after the timed passes; and the same launch on "
-                        "K = V = 0 (same instruction stream, operands that toggle nothing)",
                 "this_workload": pf["power"],
                 "zero_kv": None if pf_zero is None else dict(pf_zero["power"] or {}, ms_per_step=round(pf_zero["ms_per_step"], 4),
                                                              tflops=round(pf_zero["tflops"], 1)),
             },
+            # pure v_mfma_f32_32x32x16_f16 streams on N(0,1) operands on every compute unit, timed in
+            # this run (libellm_diag.so): operands in registers / A operand from LDS / LDS-fed plus
+            # the vector instructions of a soft-max of the same tile shape
             "mfma_stream_on_n01_fp16": {
-                "what": "pure v_mfma_f32_32x32x16_f16 stream on N(0,1) operands, one wave per SIMD on every "
-                        "compute unit, no memory access in the loop, timed in this run (libellm_diag.so)",
                 "register_operands_tflops": round(stream_reg, 1),
                 "a_operand_from_lds_tflops": round(stream_lds, 1),
                 "lds_fed_with_softmax_vector_mix_tflops": round(stream_mix, 1),
@@ -978,12 +1021,22 @@ def main():
             },
             "cpu_baseline": pf_cpu,
         })
+        targets["prefill_32k"] = {
+            "ms": round(pf["kernel_ms"], 4), "tflops": round(pf["kernel_tflops"], 1),
+            "frac": round(pf["kernel_tflops"] / MFMA_F16_PEAK_TFLOPS, 4), "target_frac": 0.5,
+            "mix_stream_tflops": round(stream_mix, 1), "register_stream_tflops": round(stream_reg, 1),
+            "frac_of_mix_stream": round(pf["kernel_tflops"] / stream_mix, 4),
+            "engine_mhz": (pf["power"] or {}).get("engine_mhz"), "watts": (pf["power"] or {}).get("watts"),
+        }
     if args.only in ("", "decode128k"):
         d128 = bench_decode(1, 131072, args.steps, args.warmup)
-        also.append({
+        targets["decode_1x131072"] = {
+            "us": round(d128["kernel_ms"] * 1e3, 2), "gbs": round(d128["kernel_gbs"], 1),
+            "frac": round(d128["kernel_gbs"] / HBM_PEAK_GBS, 4), "target_frac": 0.7}
+        last_entries.append({
             "workload": "decode: 1 seq x 131072 cached tokens, 32q/4kv heads, fp16",
             "metric": "decode attn HBM GB/s", "value": round(d128["gbs"], 1), "unit": "GB/s",
-            "ms_per_step": round(d128["ms_per_step"], 5), "steps": args.steps,
+            "ms_per_step": round(d128["ms_per_step"], 5), "kernel_ms": round(d128["kernel_ms"], 5), "steps": args.steps,
             "roofline": {"bound": "hbm", "achieved": round(d128["kernel_gbs"], 1),
                          "peak": HBM_PEAK_GBS, "unit": "GB/s",
                          "frac": round(d128["kernel_gbs"] / HBM_PEAK_GBS, 4),
@@ -995,6 +1048,9 @@ def main():
         # every cache, so one set of buffers is enough
         b128_steps = max(3, min(args.steps, 20))
         b128 = bench_decode(16, 131072, b128_steps, min(args.warmup, 3), copies=1)
+        targets["decode_16x131072"] = {
+            "us": round(b128["kernel_ms"] * 1e3, 1), "gbs": round(b128["kernel_gbs"], 1),
+            "frac": round(b128["kernel_gbs"] / HBM_PEAK_GBS, 4)}
         also.append({
             "workload": "decode: 16 seq x 131072 cached tokens, 32q/4kv heads, fp16",
             "metric": "decode attn HBM GB/s", "value": round(b128["gbs"], 1), "unit": "GB/s",
@@ -1011,8 +1067,7 @@ def main():
                            p0=120000)
         ck_cpu = None if args.skip_cpu else cpu_baseline_chunk(8192, 120000, 64, 8, "bf16")
         also.append({
-            "workload": "chunked prefill: 8192 new tokens on a 120000-token cache, 64q/8kv heads, "
-                        "bf16 (BASELINE configs[3])",
+            "workload": "chunk: 8192 tokens on a 120000-token cache, 64q/8kv, bf16 (configs[3])",
             "metric": "prefill attn TFLOP/s", "value": round(ck["tflops"], 2), "unit": "TFLOP/s",
             "ms_per_step": round(ck["ms_per_step"], 4), "steps": ck_steps,
             "roofline": {"bound": "mfma", "achieved": round(ck["kernel_tflops"], 2),
@@ -1027,8 +1082,7 @@ def main():
         # is split over workgroups and merged by a second small launch
         sc = bench_prefill(64, args.steps, min(args.warmup, 5), p0=8192)
         also.append({
-            "workload": "chunk of 64 new tokens of one sequence on an 8192-token cache, 32q/4kv heads, fp16 "
-                        "(key range split over workgroups + merge launch)",
+            "workload": "chunk: 64 tokens x 1 seq on an 8192-token cache, 32q/4kv, fp16 (keys split + merge)",
             "metric": "prefill attn TFLOP/s", "value": round(sc["tflops"], 2), "unit": "TFLOP/s",
             "ms_per_step": round(sc["ms_per_step"], 5), "steps": args.steps,
             "kv_gbs": round(2 * 4 * (8192 + 64) * D * 2 / (sc["ms_per_step"] * 1e-3) / 1e9, 1),
@@ -1038,13 +1092,10 @@ def main():
         # the reference's serving loop ends a prompt with a chunk of (prompt % 64) positions x 24 sequences
         # (src/serving/start copy.rs:71-101): few query rows per K/V plane over thousands of cached tokens
         lc_dec = bench_decode(24, 8192, args.steps, min(args.warmup, 5), copies=3)
-        lc = {t: bench_prefill(t, args.steps, min(args.warmup, 5), p0=8192, batch=24, copies=3) for t in (2, 8, 16, 24, 33, 48)}
+        lc = {t: bench_prefill(t, args.steps, min(args.warmup, 5), p0=8192, batch=24, copies=3) for t in (2, 8, 16, 24, 33, 48, 64)}
         kv_bytes = 2 * 24 * 4 * 8192 * D * 2
         also.append({
-            "workload": "short last chunk of a prompt: 2 / 8 / 16 / 24 / 33 / 48 new tokens x 24 sequences on 8192-token "
-                        "caches, 32q/4kv heads, fp16 (the streaming chunk kernel: one workgroup of 4, 8 or 12 waves "
-                        "per GQA group's rows, up to 16, 32 or 48 tokens, keys split over workgroups + merge launch); "
-                        "beside it the single-token kernel on the same caches",
+            "workload": "last chunk: 2-64 tokens x 24 seq on 8192-token caches, 32q/4kv, fp16; value = 16 tokens",
             "metric": "chunk attention us per call", "unit": "us",
             "value": round(lc[16]["ms_per_step"] * 1e3, 1),
             "us_by_tokens": {str(t): round(r["ms_per_step"] * 1e3, 1) for t, r in lc.items()},
@@ -1056,6 +1107,8 @@ def main():
                          "frac": round(kv_bytes / (lc[16]["kernel_ms"] * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
                          "traffic": TRAFFIC_BYTES["lastchunk"]},
         })
+        targets["lastchunk_24x8192"] = {"us_by_tokens": {str(t): round(r["kernel_ms"] * 1e3, 1) for t, r in lc.items()},
+                                        "single_token_us": round(lc_dec["kernel_ms"] * 1e3, 1)}
 
     if args.only in ("", "mixed"):
         # one layer of the mixed-step configuration: a 16384-token prefill and a single-token step over 32
@@ -1073,12 +1126,10 @@ def main():
             cd = cpu_baseline_ragged_decode(lengths)
             mx_cpu = {"value": round((cp["seconds_extrapolated"] + cd["seconds_extrapolated"]) * 1e3, 1),
                       "unit": "ms", "cores": cp["cores"], "kind": "port", "pinned": True,
-                      "sample": "prefill side: " + cp["sample"] + "; single-token side: " + cd["sample"],
+                      "sample": "prefill: " + cp["sample"] + "; single token: " + cd["sample"],
                       "prefill_tflops": cp["value"], "decode_gbs": cd["value"]}
         also.append({
-            "workload": "mixed step, one of 48 layers (BASELINE configs[4]), kernel by kernel: Q/K/V projection + "
-                        "attention of a 16384-token prefill, Q/K/V projection + attention of one new token of 32 "
-                        "sequences, cache lengths U{1024..131072} (seed 7)",
+            "workload": "mixed step, 1 of 48 layers (configs[4]): 16384-token prefill + 32 seq U{1024..131072}",
             "metric": "attention ms per layer",
             "value": round(mp["ms_per_step"] + md["ms_per_step"], 4), "unit": "ms",
             "prefill_ms": round(mp["ms_per_step"], 4), "prefill_tflops": round(mp["tflops"], 1),
@@ -1104,30 +1155,25 @@ def main():
             ms = None
             also.append({"workload": "mixed step end to end (BASELINE configs[4])", "error": str(e)[:300]})
         if ms is not None:
+            # every flop at the MFMA peak plus every cache byte at the HBM peak, one after the other
+            floor_ms = ((ms["flops"] + ms["proj_flops"]) / (MFMA_F16_PEAK_TFLOPS * 1e12) + ms["bytes"] / (HBM_PEAK_GBS * 1e9)) * 1e3
             also.append({
-                "workload": "mixed step end to end (BASELINE configs[4]): 48 layers x (Q/K/V projection + attention "
-                            "of a 16384-token prefill, Q/K/V projection + attention of one new token of 32 "
-                            "sequences with cache lengths U{1024..131072}, seed 7), random-init fp16 projection "
-                            "weights per layer, K/V written into the caches by the projections; every layer has "
-                            "its own K/V in one cache object with per-sequence capacities "
-                            f"({ms['resident_bytes'] / 1e9:.1f} GB resident); 192 launches: on one stream issued "
-                            "one by one (eager_ms), replayed from one recorded graph (graph_ms), and with the "
-                            "single-token half of every layer recorded as a parallel branch on the library's "
-                            "side stream (side_by_side_ms = value: the MFMA-bound and the HBM-bound half fill "
-                            "each other's tails)",
-                "metric": "attention ms per step", "value": round(ms["side_by_side_ms"], 3), "unit": "ms",
+                "workload": "mixed step, 48 layers, projections + attention (configs[4]); value = one stream, one graph",
+                "metric": "attention ms per step", "value": round(ms["graph_ms"], 3), "unit": "ms",
                 "eager_ms": round(ms["eager_ms"], 3), "graph_ms": round(ms["graph_ms"], 3),
                 "side_by_side_ms": round(ms["side_by_side_ms"], 3),
                 "steps": 3, "prefill_tflop_per_step": round(ms["flops"] / 1e12, 2),
                 "projection_tflop_per_step": round(ms["proj_flops"] / 1e12, 2),
                 "decode_gb_per_step": round(ms["bytes"] / 1e9, 1),
                 "cache_resident_gb": round(ms["resident_bytes"] / 1e9, 1),
+                "floor_ms_at_both_peaks": round(floor_ms, 2), "frac_of_floor": round(floor_ms / ms["graph_ms"], 4),
             })
+            targets["mixed48"] = {"ms_one_stream": round(ms["graph_ms"], 2), "ms_two_streams": round(ms["side_by_side_ms"], 2),
+                                  "floor_ms": round(floor_ms, 2), "frac_of_floor": round(floor_ms / ms["graph_ms"], 4)}
     if args.only in ("", "kvwrite"):
         kw = bench_kv_write(32768, args.steps, args.warmup)
         also.append({
-            "workload": "cache write with key RMS norm + rotary rotation: 32768 tokens x 4 kv heads, "
-                        "fp16 (the K/V rows of the 32k prefill)",
+            "workload": "cache write, key RMS norm + rotation: 32768 tokens x 4 kv heads, fp16",
             "metric": "kv write HBM GB/s", "value": round(kw["gbs"], 1), "unit": "GB/s",
             "ms_per_step": round(kw["ms_per_step"], 5), "steps": args.steps,
             "roofline": {"bound": "hbm", "achieved": round(kw["kernel_gbs"], 1),
@@ -1140,21 +1186,20 @@ def main():
         for (tb, tl) in ((16, 8192), (4, 1024)):
             ts = bench_token_step(48, tb, tl, min(args.steps, 20), min(args.warmup, 3))
             also.append({
-                "workload": f"single-token step over 48 layers: per layer the fused cache write of {tb} new "
-                            f"K/V rows x 4 heads + attention over {tb} seq x {tl} cached tokens, positions "
-                            "advanced on the device; 97 launches issued one by one vs one recorded graph",
+                "workload": f"token step, 48 layers: cache write + attention, {tb} seq x {tl} cached tokens; value = graph",
                 "metric": "attention ms per token step", "value": round(ts["graph_ms"], 4), "unit": "ms",
                 "eager_ms": round(ts["eager_ms"], 4), "graph_ms": round(ts["graph_ms"], 4),
                 "steps": min(args.steps, 20),
                 "gbs": round(ts["bytes"] / (ts["graph_ms"] * 1e-3) / 1e9, 1),
             })
+            targets[f"tokenstep_{tb}x{tl}"] = {"ms": round(ts["graph_ms"], 4),
+                                               "frac": round(ts["bytes"] / (ts["graph_ms"] * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)}
 
     if args.only in ("", "qkv"):
         pj_steps = max(3, min(args.steps, 20))
         pj = bench_qkv_projection(32768, pj_steps, min(args.warmup, 3))
         also.append({
-            "workload": "fused Q/K/V projection: 32768 tokens x hidden 2048 -> 32q + 4k + 4v heads x 128, fp16, "
-                        "RMS norm + rotary rotation of Q and K heads, K/V written to the cache",
+            "workload": "fused Q/K/V projection: 32768 rows x 2048 -> 5120, norm + rotation, K/V to the cache, fp16",
             "metric": "projection TFLOP/s", "value": round(pj["tflops"], 2), "unit": "TFLOP/s",
             "ms_per_step": round(pj["ms_per_step"], 4), "steps": pj_steps,
             "roofline": {"bound": "mfma", "achieved": round(pj["kernel_tflops"], 2),
@@ -1179,9 +1224,7 @@ def main():
         cq = bench_qkv_projection(64, args.steps, min(args.warmup, 5), batch=24)
         co = bench_output_projection(64 * 24, args.steps, min(args.warmup, 5))
         also.append({
-            "workload": "projections of a prompt chunk of 64 positions x 24 sequences (1536 rows, the reference's "
-                        "serving shape): fused Q/K/V 2048 -> 5120 and output + residual 4096 -> 2048, fp16 "
-                        "(128-token x one-head tiles)",
+            "workload": "projections at 1536 rows (64 positions x 24 seq): Q/K/V 2048 -> 5120, output 4096 -> 2048, fp16",
             "metric": "projection TFLOP/s (Q/K/V)", "value": round(cq["tflops"], 2), "unit": "TFLOP/s",
             "ms_per_step": round(cq["ms_per_step"], 5), "steps": args.steps,
             "output_projection_ms": round(co["ms_per_step"], 5),
@@ -1190,13 +1233,15 @@ def main():
                          "peak": MFMA_F16_PEAK_TFLOPS, "unit": "TFLOP/s",
                          "frac": round(cq["kernel_tflops"] / MFMA_F16_PEAK_TFLOPS, 4), "traffic": None},
         })
+        targets["chunkproj_1536"] = {
+            "qkv_us": round(cq["kernel_ms"] * 1e3, 2), "output_us": round(co["kernel_ms"] * 1e3, 2),
+            "qkv_frac": round(cq["kernel_tflops"] / MFMA_F16_PEAK_TFLOPS, 4),
+            "output_frac": round(co["kernel_tflops"] / MFMA_F16_PEAK_TFLOPS, 4)}
 
     if args.only in ("", "chunkblock"):
         cb = bench_chunk_block(64, 24, 4096, min(args.steps, 30), min(args.warmup, 5))
         also.append({
-            "workload": "attention block of one layer for a prompt chunk of 64 positions x 24 sequences (the "
-                        "reference's serving shape) on caches of 4096 tokens: fused Q/K/V projection (K/V into the "
-                        "cache) + chunk attention + output projection with residual, fp16, three launches",
+            "workload": "layer block, chunk of 64 positions x 24 seq on 4096-token caches: Q/K/V + attention + output",
             "metric": "attention-block ms per chunk", "value": round(cb["block_ms"], 5), "unit": "ms",
             "steps": min(args.steps, 30),
             "qkv_ms": round(cb["parts_ms"]["qkv"], 5), "attention_ms": round(cb["parts_ms"]["attention"], 5),
@@ -1207,9 +1252,7 @@ def main():
     if args.only in ("", "stepproj"):
         sp = bench_step_projections(16, args.steps, args.warmup)
         also.append({
-            "workload": "projections of a single-token step, 16 sequences: fused Q/K/V (2048 -> 5120, norm + "
-                        "rotation, K/V to the cache) and output + residual (4096 -> 2048), fp16, weights "
-                        "streamed from HBM (8 rotating sets)",
+            "workload": "projections of a token step, 16 seq: Q/K/V 2048 -> 5120, output 4096 -> 2048, weights from HBM",
             "metric": "weight stream GB/s (Q/K/V projection)", "unit": "GB/s",
             "value": round(sp["qkv_bytes"] / (sp["qkv_ms"] * 1e-3) / 1e9, 1),
             "ms_per_step": round(sp["qkv_ms"], 5), "steps": args.steps,
@@ -1220,27 +1263,47 @@ def main():
                          "frac": round(sp["qkv_bytes"] / (sp["qkv_kernel_ms"] * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
                          "traffic": TRAFFIC_BYTES["stepproj"]},
         })
+        targets["stepproj_16"] = {
+            "qkv_us": round(sp["qkv_kernel_ms"] * 1e3, 2), "output_us": round(sp["o_kernel_ms"] * 1e3, 2),
+            "qkv_frac": round(sp["qkv_bytes"] / (sp["qkv_kernel_ms"] * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
+            "output_frac": round(sp["o_bytes"] / (sp["o_kernel_ms"] * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)}
 
     if args.only in ("", "layerstep"):
-        ls_steps = min(args.steps, 20)
-        ls = bench_layer_step(48, 16, 8192, ls_steps, min(args.warmup, 3))
-        also.append({
-            "workload": "attention blocks of a 48-layer single-token step, 16 seq x 8192 cached tokens: per layer "
-                        "fused Q/K/V projection (K/V written into the cache) + attention + output projection "
-                        "with residual, own weights and cache per layer, positions on the device; 145 launches "
-                        "issued one by one vs one recorded graph",
-            "metric": "attention-block ms per token step", "value": round(ls["graph_ms"], 4), "unit": "ms",
-            "eager_ms": round(ls["eager_ms"], 4), "graph_ms": round(ls["graph_ms"], 4), "steps": ls_steps,
-            "cache_gb_per_step": round(ls["kv_bytes"] / 1e9, 2), "weight_gb_per_step": round(ls["w_bytes"] / 1e9, 2),
-            "gbs": round((ls["kv_bytes"] + ls["w_bytes"]) / (ls["graph_ms"] * 1e-3) / 1e9, 1),
-        })
+        # 16 x 8192: BASELINE configs[1] with its projections; 4 x 1024: a small batch; 1 x 512 / 256 / 128:
+        # the operating point of the reference's own published numbers (decode at batch 1 after a prompt
+        # of 128 / 256 / 512 tokens, README.md:92-116; its figures include the MoE blocks, these do not)
+        cases = [(16, 8192), (4, 1024), (1, 512), (1, 256), (1, 128)]
+        lsr = bench_layer_steps(48, cases, args.steps, min(args.warmup, 3))
+        for (lb, ll) in cases:
+            ls = lsr[(lb, ll)]
+            nbytes = ls["kv_bytes"] + ls["w_bytes"]
+            ls_cpu = None
+            if not args.skip_cpu and (lb == 1 or (lb, ll) == (16, 8192)):
+                ls_cpu = cpu_baseline_layer_step(lb, ll)
+            also.append({
+                "workload": f"layer step, 48 layers: Q/K/V projection + attention + output projection, {lb} seq x {ll} cached tokens",
+                "metric": "attention-block ms per token step", "value": round(ls["graph_ms"], 4), "unit": "ms",
+                "eager_ms": round(ls["eager_ms"], 4), "graph_ms": round(ls["graph_ms"], 4),
+                "kernel_ms": round(ls["graph_dev_ms"], 4), "us_per_layer": round(ls["graph_dev_ms"] * 1e3 / 48, 2),
+                "steps": ls["steps"],
+                "cache_gb_per_step": round(ls["kv_bytes"] / 1e9, 3), "weight_gb_per_step": round(ls["w_bytes"] / 1e9, 3),
+                "roofline": {"bound": "hbm", "achieved": round(nbytes / (ls["graph_dev_ms"] * 1e-3) / 1e9, 1),
+                             "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                             "frac": round(nbytes / (ls["graph_dev_ms"] * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
+                             "traffic": None},
+                "cpu_baseline": ls_cpu,
+            })
+            targets[f"layerstep_{lb}x{ll}"] = {
+                "ms": round(ls["graph_dev_ms"], 4), "us_per_layer": round(ls["graph_dev_ms"] * 1e3 / 48, 2),
+                "frac": round(nbytes / (ls["graph_dev_ms"] * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)}
 
     cpu = None
     if not args.skip_cpu and dec is not None:
         cpu = cpu_baseline_decode(16, 8192)
 
+    also += last_entries
     if dec is None:  # partial run for profiling
-        print(json.dumps({"also": also}))
+        print(json.dumps({"targets": targets, "also": also}))
         return
     line = {
         "metric": "decode attn HBM GB/s (Qwen3 GQA, 1 GPU)",
@@ -1250,17 +1313,21 @@ def main():
         "steps": args.steps,
         "warmup": args.warmup,
         "ms_per_step": round(dec["ms_per_step"], 5),
+        # value = algorithmic bytes / ms_per_step (host clock around the K steps); roofline.achieved and
+        # .frac = the same bytes / kernel_ms (HIP events on the launch stream around the same K launches)
+        "kernel_ms": round(dec["kernel_ms"], 5),
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
         "dtype": "f16",
         "data": "synthetic",
-        "config": {"workload": "decode: 16 seq x 8192 cached tokens, 32q/4kv heads, head_dim 128, "
-                               "fp16, dimension-first cache (BASELINE configs[1])",
+        "config": {"workload": "decode: 16 seq x 8192 cached tokens, 32q/4kv heads, fp16 (BASELINE configs[1])",
                    "batch": 16, "cache_len": 8192, "q_heads": 32, "kv_heads": 4},
         "roofline": {"bound": "hbm", "achieved": round(dec["kernel_gbs"], 1), "peak": HBM_PEAK_GBS,
                      "unit": "GB/s", "frac": round(dec["kernel_gbs"] / HBM_PEAK_GBS, 4),
-                     "traffic": TRAFFIC_BYTES["decode"]},
+                     "traffic": TRAFFIC_BYTES["decode"], "timer": "kernel_ms (HIP events)",
+                     # the headline figures of the other workloads (their full entries are in `also`)
+                     "targets": targets},
         "cpu_baseline": cpu,
         "passes": dec["passes"],
         "cpu_model": host["cpu_model"],

@@ -78,13 +78,32 @@ inline DecodeWorkspace decode_workspace(uint32_t batch_capacity, uint32_t n_q_he
   return w;
 }
 
-inline bool decode_plan_fits(const DecodeWorkspace& w, uint32_t batch, uint32_t n_q_heads,
-                      uint32_t n_kv_heads, uint32_t group, uint32_t n_split) {
+// Which bound of the workspace a plan exceeds: 0 none, 1 split partials, 2 cluster partials,
+// 3 arrival counters.  Cluster partials are written only when a plane has more splits than one
+// fold takes (n_split > kPlanMergeFan); with fewer the single fold goes straight to the output.
+inline int decode_plan_exceeds(const DecodeWorkspace& w, uint32_t batch, uint32_t n_q_heads,
+                               uint32_t n_kv_heads, uint32_t group, uint32_t n_split) {
   const size_t n_cluster = (n_split + kPlanMergeFan - 1) / kPlanMergeFan;
   const size_t head_groups = (group + kPlanMaxHeadsPerGroup - 1) / kPlanMaxHeadsPerGroup;
-  return (size_t)batch * n_q_heads * n_split <= w.rows &&
-         (size_t)batch * n_q_heads * n_cluster <= w.rows2 &&
-         (size_t)batch * n_kv_heads * head_groups * (1 + n_cluster) <= w.counters;
+  if ((size_t)batch * n_q_heads * n_split > w.rows) return 1;
+  if (n_cluster > 1 && (size_t)batch * n_q_heads * n_cluster > w.rows2) return 2;
+  if ((size_t)batch * n_kv_heads * head_groups * (1 + n_cluster) > w.counters) return 3;
+  return 0;
 }
+
+inline bool decode_plan_fits(const DecodeWorkspace& w, uint32_t batch, uint32_t n_q_heads,
+                      uint32_t n_kv_heads, uint32_t group, uint32_t n_split) {
+  return decode_plan_exceeds(w, batch, n_q_heads, n_kv_heads, group, n_split) == 0;
+}
+
+// Capacity of the static scratch of the entry point that allocates nothing (noalloc.hip), in
+// the units of DecodeWorkspace.  A launch with more than one split per K/V plane has at most
+// 2 x compute units workgroups, so (sequences x query heads x splits) <= group size x 2 x
+// compute units partial rows: 8192 rows cover GQA groups of up to 16 query heads on a 256-unit
+// part whatever the plan.  With more than 16 splits a plane the cluster partials are at most
+// rows / 16 + sequences x query heads < 1024 rows; the counters are (1 + clusters) per plane.
+constexpr size_t kStaticRows = 8192;       // split partials   [row][128] + [row][2] floats
+constexpr size_t kStaticRows2 = 1536;      // cluster partials [row][128] + [row][2] floats
+constexpr size_t kStaticCounters = 4096;   // uint32 arrival counters
 
 }  // namespace ellm

@@ -17,14 +17,11 @@
 
 namespace {
 
-// Capacity of the static scratch, in the units of ellm::DecodeWorkspace.  A launch with
-// more than one split per K/V plane has at most 2 x compute units workgroups, so
-// (sequences x query heads x splits) <= group size x 2 x compute units partial rows:
-// 8192 rows cover GQA groups of up to 16 query heads on a 256-unit part whatever the plan,
-// and groups of up to 32 where the plan has one workgroup per unit (most shapes).
-constexpr size_t kRows = 8192;       // split partials   [row][128] + [row][2] floats
-constexpr size_t kRows2 = 1536;      // cluster partials [row][128] + [row][2] floats
-constexpr size_t kCounters = 4096;   // uint32 arrival counters
+// Capacity of the static scratch: decode_plan.hpp (kStaticRows ...), where the host tests
+// check it against every plan the planner returns.
+constexpr size_t kRows = ellm::kStaticRows;
+constexpr size_t kRows2 = ellm::kStaticRows2;
+constexpr size_t kCounters = ellm::kStaticCounters;
 constexpr size_t kOffMl = kRows * 128;
 constexpr size_t kOffAcc2 = kOffMl + kRows * 2;
 constexpr size_t kOffMl2 = kOffAcc2 + kRows2 * 128;
@@ -52,16 +49,29 @@ __global__ void clear_counters_kernel(uint32_t* counters, uint32_t n) {
   if (i < n) counters[i] = 0u;
 }
 
-// Once per device, with that device current: the address of its copy of the array.
+// The current device's entry: its copy of the array's address and its compute-unit count.
+// The steady-state cost is one hipGetDevice; the property query and the symbol lookup (a
+// module load, which a stream capture in progress does not allow) run once per device, under
+// the mutex, the first time a device is seen.
 int prepare_current_device(const PerDevice** out) {
-  int device = 0, n_cu = 0;
-  if (int st = ellm::current_gfx950_device(&device, &n_cu)) return st;
+  int device = 0;
+  const hipError_t got = hipGetDevice(&device);
+  if (got != hipSuccess) {
+    (void)hipGetLastError();
+    return ellm::set_error(ELLM_ERR_NO_DEVICE, "hipGetDevice: %s", hipGetErrorString(got));
+  }
   if (device < 0 || device >= kMaxDevices)
     return ellm::set_error(ELLM_ERR_UNSUPPORTED, "device %d: at most %d devices are tracked", device,
                            kMaxDevices);
-  std::lock_guard<std::mutex> lock(g_mutex);
   PerDevice& d = g_devices[device];
+  if (__atomic_load_n(&d.ready, __ATOMIC_ACQUIRE)) {
+    *out = &d;
+    return ELLM_OK;
+  }
+  std::lock_guard<std::mutex> lock(g_mutex);
   if (!d.ready) {
+    int checked = 0, n_cu = 0;
+    if (int st = ellm::current_gfx950_device(&checked, &n_cu)) return st;
     float* ptr = nullptr;
     const hipError_t e = hipGetSymbolAddress((void**)&ptr, HIP_SYMBOL(scratch));
     if (e != hipSuccess || !ptr)
@@ -69,7 +79,7 @@ int prepare_current_device(const PerDevice** out) {
                              hipGetErrorString(e));
     d.ptr = ptr;
     d.n_cu = n_cu;
-    d.ready = true;
+    __atomic_store_n(&d.ready, true, __ATOMIC_RELEASE);
   }
   *out = &d;
   return ELLM_OK;
@@ -112,12 +122,21 @@ int ellm_attn_run_noalloc(const ellm_attn_desc* desc, const uint32_t* positions,
   a.n_split = plan.n_split;
   if (plan.n_split > 1) {  // an unsplit launch touches no scratch at all
     const ellm::DecodeWorkspace room{kRows, kRows2, kCounters};
-    if (!ellm::decode_plan_fits(room, a.batch, a.n_q_heads, a.n_kv_heads, a.group, a.n_split))
+    const int over = ellm::decode_plan_exceeds(room, a.batch, a.n_q_heads, a.n_kv_heads, a.group, a.n_split);
+    if (over) {
+      const size_t n_cluster = (a.n_split + ellm::kPlanMergeFan - 1) / ellm::kPlanMergeFan;
+      const size_t head_groups = (a.group + ellm::kPlanMaxHeadsPerGroup - 1) / ellm::kPlanMaxHeadsPerGroup;
+      const char* what = over == 1 ? "split partial rows" : (over == 2 ? "cluster partial rows" : "arrival counters");
+      const size_t need = over == 1 ? batch_size * a.n_q_heads * a.n_split
+                                    : (over == 2 ? batch_size * a.n_q_heads * n_cluster
+                                                 : batch_size * a.n_kv_heads * head_groups * (1 + n_cluster));
+      const size_t have = over == 1 ? kRows : (over == 2 ? kRows2 : kCounters);
       return ellm::set_error(
           ELLM_ERR_OUT_OF_RANGE,
-          "%zu sequences x %u query heads x %u splits = %zu partial rows; the static scratch holds %zu "
+          "%zu sequences x %u query heads x %u splits need %zu %s; the static scratch holds %zu "
           "(use ellm_attn_create / ellm_attn_run, whose handle sizes its own workspace)",
-          batch_size, a.n_q_heads, a.n_split, batch_size * a.n_q_heads * a.n_split, kRows);
+          batch_size, a.n_q_heads, a.n_split, need, what, have);
+    }
     float* base = dev->ptr;   // never the array's name: that is not a device address here
     a.ws_acc = base;
     a.ws_ml = base + kOffMl;

@@ -79,8 +79,12 @@ static int matmul3_create(const ellm_matmul3_desc* d, const ellm_kv_seq_table* t
                              d->batch_size, table->sequences);
     local = *d;
     size_t cap = 0;
-    for (size_t i = 0; i < d->batch_size; ++i)
+    for (size_t i = 0; i < d->batch_size; ++i) {
+      // (the kernels clamp a position to capacity - 1: a capacity of 0 would switch the clamp off)
+      if (table->seq_capacity_host[i] == 0)
+        return ellm::set_error(ELLM_ERR_INVALID_ARGUMENT, "sequence %zu of the table has capacity 0", i);
       cap = table->seq_capacity_host[i] > cap ? table->seq_capacity_host[i] : cap;
+    }
     local.sequence_capacity = cap;   // the largest: per-sequence checks follow at run time
     d = &local;
   }

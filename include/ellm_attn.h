@@ -179,14 +179,18 @@ int ellm_attn_ragged_path(const ellm_attn* handle, size_t max_position, size_t b
  * The split partials and arrival counters live in a static device array of 5,074,944
  * bytes that every device the library runs on holds until the process ends; the call
  * uses the current device's copy.  Limit: sequences x query heads x splits <= 8192
- * partial rows, which covers GQA groups of up to 16 query heads on a 256-unit part;
- * larger shapes return ELLM_ERR_OUT_OF_RANGE and must use a handle.  Every call on a
+ * partial rows, which covers GQA groups of up to 16 query heads on a 256-unit part
+ * (every split plan inside that limit also fits the cluster partials and the counters);
+ * larger shapes return ELLM_ERR_OUT_OF_RANGE, the message naming the bound, and must use
+ * a handle.  Every call on a
  * device shares that device's array: calls that overlap on one device (two streams, or
  * two graphs replayed at once) race; calls in stream order do not.  It calls no
  * hipMalloc / hipFree and launches kernels only (the counters are cleared by a small
- * fill kernel), so it may be recorded into a graph; the first call on a device looks up
- * the array's address (any ellm_attn_create / ellm_kv_create on that device has done so
- * already).
+ * fill kernel), so it may be recorded into a graph.  The first call on a device looks up
+ * the array's address and the device's properties (later calls only ask which device is
+ * current): that first call must happen outside a stream capture, or after any
+ * ellm_attn_create / ellm_kv_create on that device, which do
+ * the lookup themselves.
  */
 int ellm_attn_run_noalloc(const ellm_attn_desc* desc, const uint32_t* positions, size_t position,
                           size_t batch_size, void* stream);

@@ -21,6 +21,11 @@ LSE_TOL = 1e-4
 # (cancellation), which is what the absolute bound is for.  Measured on MI355X: max-rel
 # 3.7e-3 over |ref| >= 2^-4 and 1.5e-2 over |ref| >= 2^-6 (binary16, rows with few keys).
 REL_FLOOR = 2.0 ** -4
+# A second, wider bound two octaves further down, so that a regression among the small outputs
+# fails a test instead of only showing in a printed figure: 2x RTOL over |ref| >= 2^-6
+# (measured worst case 1.8e-2, the 32768-token prefill of BASELINE configs[2]).
+REL_FLOOR_LOW = 2.0 ** -6
+RTOL_LOW = {orc.F16: 2e-2, orc.BF16: 1.6e-1}
 
 
 def storage_ulp(ref, dtype):
@@ -38,8 +43,8 @@ def compare(got, want, dtype):
     round binary32 results to storage values that are further apart than ATOL, so results
     that differ by 1e-6 before rounding can land on adjacent values: there, and only there,
     the bound is one unit in the last place (`n_beyond_atol_within_1ulp` counts the elements
-    that needed it).  The relative bound RTOL is taken over |ref| >= REL_FLOOR; the figure
-    over |ref| >= 2^-6 is reported beside it."""
+    that needed it).  The relative bound RTOL is taken over |ref| >= REL_FLOOR, and RTOL_LOW
+    (twice as wide) over |ref| >= REL_FLOOR_LOW = 2^-6."""
     err = np.abs(got - want)
     ulp = storage_ulp(want, dtype)
     coarse = ulp > ATOL[dtype]                  # storage spacing wider than the absolute bound
@@ -52,13 +57,14 @@ def compare(got, want, dtype):
         return float((err[sel] / np.abs(want[sel])).max()) if sel.any() else 0.0
 
     rel = rel_at(REL_FLOOR)
+    rel_low = rel_at(REL_FLOOR_LOW)
     return {
         "max_abs": float(err.max()),
         "max_abs_where_1ulp_below_atol": max_abs_fine,
         "n_beyond_atol_within_1ulp": int((err[coarse] > ATOL[dtype]).sum()),
         "max_rel": rel,
-        "max_rel_floor_2^-6": rel_at(2.0 ** -6),
-        "ok": ok_abs and rel <= RTOL[dtype] and not np.isnan(got).any(),
+        "max_rel_floor_2^-6": rel_low,
+        "ok": ok_abs and rel <= RTOL[dtype] and rel_low <= RTOL_LOW[dtype] and not np.isnan(got).any(),
     }
 
 

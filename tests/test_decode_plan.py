@@ -73,3 +73,56 @@ def test_one_workgroup_per_unit_where_the_planes_divide_the_units(rows):
     assert by[(256, 32, 4, 12, 8192)] == (1664, 5)         # 48 planes x 5 = 240
     assert by[(256, 32, 4, 98, 8192)] == (8192, 1)         # more planes than units: no split
     assert by[(256, 32, 4, 1, 255)] == (256, 1)
+
+
+STATIC_PROBE = r"""
+#include "decode_plan.hpp"
+#include <cstdio>
+using namespace ellm;
+int main() {
+  const DecodeWorkspace room{kStaticRows, kStaticRows2, kStaticCounters};
+  const uint32_t lens[] = {1, 255, 256, 257, 511, 512, 1000, 2048, 4096, 6000, 8192, 20000, 40000, 65536,
+                           131072, 1u << 20, 1u << 24, 0x7fffffffu};
+  const uint32_t groups[] = {1, 2, 4, 8, 16};
+  const uint32_t kv[] = {1, 2, 4, 8, 16, 32};
+  unsigned long n = 0, refused = 0;
+  for (uint32_t g : groups)
+    for (uint32_t hkv : kv)
+      for (uint32_t batch = 1; batch <= 512; batch += (batch < 130 ? 1 : 16))
+        for (uint32_t len : lens) {
+          const uint32_t hq = g * hkv;
+          const DecodePlan p = decode_plan(len, batch, hkv, 256);
+          if (p.n_split == 1) continue;   // an unsplit launch touches no scratch
+          const size_t rows = (size_t)batch * hq * p.n_split;
+          if (rows > kStaticRows) continue;   // the documented limit
+          ++n;
+          const int over = decode_plan_exceeds(room, batch, hq, hkv, g, p.n_split);
+          if (over) {
+            ++refused;
+            printf("refused %u seq x %uq/%ukv len %u: n_split %u rows %zu bound %d\n", batch, hq, hkv, len, p.n_split,
+                   rows, over);
+          }
+        }
+  printf("checked %lu refused %lu\n", n, refused);
+  return 0;
+}
+"""
+
+
+def test_static_scratch_holds_every_plan_within_its_documented_limit(tmp_path):
+    """ellm_attn_run_noalloc documents one limit: sequences x query heads x splits <= 8192 partial
+    rows, GQA groups of up to 16 heads.  Every plan of a 256-unit part inside that limit must fit the
+    static sizes (cluster partials and counters included), or the entry point refuses shapes its
+    header says it takes."""
+    gxx = shutil.which("g++")
+    if not gxx:
+        pytest.skip("no g++")
+    src = tmp_path / "probe.cpp"
+    src.write_text(STATIC_PROBE)
+    exe = tmp_path / "probe"
+    subprocess.run([gxx, "-O2", "-std=c++17", "-Wall", "-Werror", "-I", CSRC, str(src), "-o", str(exe)],
+                   check=True, timeout=300)
+    out = subprocess.run([str(exe)], check=True, capture_output=True, text=True, timeout=300).stdout
+    last = out.strip().splitlines()[-1].split()
+    assert int(last[1]) > 3000, out[-500:]
+    assert int(last[3]) == 0, out[:2000]

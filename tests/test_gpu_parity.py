@@ -236,6 +236,33 @@ def test_causality_rows_ignore_later_keys():
     assert not np.array_equal(base[100:], pert[100:])
 
 
+@pytest.mark.parametrize("shape", [("tile", 130, 60, 256, 8, 1), ("stream", 24, 900, 1024, 8, 2)],
+                         ids=lambda sh: sh[0])
+def test_value_rows_rule_at_the_boundary_the_header_states(shape):
+    """ellm_attn_run's rule for K/V contents, pinned where it bites, in the tile kernel and in the
+    streaming chunk kernel: (1) rows of the call's own later tokens are read by earlier query rows
+    with a probability of exactly 0, so while they are FINITE (whatever their values) the earlier
+    rows' bits do not depend on them; (2) rows strictly beyond the call's last position are never
+    read: NaN / Inf there change nothing.  (The reference reads neither: flash_attention.rs:57-58.)"""
+    _, s, p0, cap, hq, hkv = shape
+    dtype = orc.F16
+    q = rand_storage((s, 1, hq, D), 91, dtype)
+    k = rand_storage((1, hkv, cap, D), 92, dtype)
+    v = rand_storage((1, hkv, cap, D), 93, dtype)
+    base, base_lse = gpu_attention(q, k, v, 0.09, dtype, position_index=p0)
+    cut = s // 2                                         # tokens cut.. of the chunk are "later" for rows < cut
+    k2, v2 = k.copy(), v.copy()
+    k2.view(np.float16)[:, :, p0 + cut:p0 + s] = 60000.0    # finite, huge
+    v2.view(np.float16)[:, :, p0 + cut:p0 + s] = -65504.0
+    k2.view(np.uint16)[:, :, p0 + s:] = 0x7e00              # NaN beyond the call's last position
+    v2.view(np.uint16)[:, :, p0 + s:] = 0x7c00              # +Inf
+    pert, pert_lse = gpu_attention(q, k2, v2, 0.09, dtype, position_index=p0)
+    assert np.array_equal(base[:cut], pert[:cut]) and np.array_equal(base_lse[:cut], pert_lse[:cut])
+    assert np.isfinite(pert[:cut]).all()
+    want, _ = orc.attention(q, k, v, 0.09, dtype, position_index=p0)
+    assert compare(base, orc.from_storage(want, dtype), dtype)["ok"]
+
+
 def test_chunked_prefill_and_decode_agree_with_one_pass():
     """The position loop of the serving layer (src/serving/'start copy.rs':86-111): full
     chunks, a partial chunk, then single-token steps give the rows of one pass."""

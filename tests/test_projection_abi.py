@@ -48,6 +48,21 @@ def test_matmul3_create(over, status):
     assert not h.value
 
 
+def test_matmul3_create_ragged_rejects_a_zero_capacity():
+    """The kernels clamp a position to capacity - 1; a capacity of 0 would wrap and switch the clamp
+    off.  Refused before anything touches a device, as ellm_attn_create_ragged does."""
+    lib = ellm_amd.load_library()
+    caps = (ctypes.c_size_t * 2)(64, 0)
+    table = _lib.KvSeqTable()
+    table.seq_offsets = 0x1000
+    table.seq_capacity = 0x2000
+    table.seq_capacity_host = ctypes.cast(caps, ctypes.POINTER(ctypes.c_size_t))
+    table.sequences = 2
+    h = ctypes.c_void_p()
+    assert lib.ellm_matmul3_create_ragged(ctypes.byref(_m3()), ctypes.byref(table), ctypes.byref(h)) == INVALID
+    assert b"capacity 0" in lib.ellm_last_error_string() and not h.value
+
+
 def test_create_without_a_device_says_so():
     lib = ellm_amd.load_library()
     if lib.ellm_device_count() > 0:

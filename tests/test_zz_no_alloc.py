@@ -109,3 +109,78 @@ def test_noalloc_rejects_what_the_scratch_cannot_hold():
     op.run(cap - 1, 1, batch)                # the handle's path takes the same shape
     torch.cuda.synchronize()
     op.close()
+
+
+def test_noalloc_takes_shapes_near_its_documented_limit():
+    """97 sequences x 16 query heads on one K/V head, five splits a plane: 7760 of the 8192 partial
+    rows the header promises (an earlier fit check also demanded cluster partials that a plan with
+    at most 16 splits a plane never writes, and refused this shape)."""
+    q, k, v = _case(61, 97, 16, 1, 1280, orc.F16)
+    _check(q, k, v, orc.F16, batch=97, position=1279)
+    # 40 sequences x 64 query heads on 4 K/V heads (groups of 16), three splits: 7680 rows
+    q, k, v = _case(71, 40, 64, 4, 1024, orc.F16)
+    _check(q, k, v, orc.F16, batch=40, position=1023)
+
+
+def test_noalloc_recorded_into_a_graph_replays_like_eager():
+    """The stated use: the call recorded once into a graph (counter clear + attention, both kernel
+    nodes) and replayed while the per-sequence positions move on inside the graph; eager work and
+    synchronisations between replays.  Every replay equals the eager call bit for bit, and the last
+    one the oracle."""
+    import torch
+
+    import ellm_amd
+
+    dtype = orc.F16
+    bcap, hq, hkv, cap = 6, 32, 4, 3000
+    q, k, v = _case(81, bcap, hq, hkv, cap, dtype)
+    scale = 1.0 / np.sqrt(D)
+    dq, dk, dv = to_dev(q, dtype), to_dev(k, dtype), to_dev(v, dtype)
+    dout = torch.full_like(dq, float("nan"))
+    dlse = torch.full((1, bcap, hq), float("nan"), dtype=torch.float32, device="cuda")
+    op = ellm_amd.Attention(dq, dk, dv, dout, bcap, hq, hkv, D, [hkv * cap * D, cap * D, D, 1], scale,
+                            lse=dlse, sequence_capacity=cap, max_position_interval=1)
+    start = np.array([2500, 3, 64, 1000, 127, 1999], dtype=np.uint32)
+    steps, by = 4, 41
+    stream = torch.cuda.Stream()
+
+    def walk(use_graph):
+        pos = torch.from_numpy(start.view(np.int32).copy()).cuda()
+        outs, graph = [], None
+        with torch.cuda.stream(stream):
+            for _ in range(steps):
+                dout.fill_(float("nan"))
+
+                def step():
+                    op.run_noalloc(cap - 1, bcap, positions=pos, stream=stream)
+                    ellm_amd.positions_advance(pos, by, stream=stream)
+
+                if not use_graph:
+                    step()
+                else:
+                    if graph is None:
+                        stream.synchronize()
+                        with ellm_amd.StepGraph(stream) as graph:
+                            step()
+                    graph.launch()
+                stream.synchronize()
+                outs.append((dout.view(torch.int16).cpu().numpy().copy(), dlse.cpu().numpy().copy()))
+                _ = float(dout.float().sum())     # eager work between replays
+        if graph is not None:
+            graph.close()
+        return outs
+
+    try:
+        eager = walk(False)
+        replay = walk(True)
+        for n in range(steps):
+            assert np.array_equal(eager[n][0], replay[n][0]), n
+            assert np.array_equal(eager[n][1].view(np.uint32), replay[n][1].view(np.uint32)), n
+        last = start + (steps - 1) * by
+        want, want_lse = orc.attention(q, k, v, scale, dtype, positions=last, batch=bcap)
+        got = orc.from_storage(replay[-1][0].view(np.uint16), dtype)
+        r = compare(got, orc.from_storage(want, dtype), dtype)
+        assert r["ok"], r
+        assert np.abs(replay[-1][1] - want_lse).max() <= 1e-4
+    finally:
+        op.close()
