@@ -293,6 +293,22 @@ extern "C" {
         stream: Stream,
     ) -> c_int;
     pub fn ellm_matmul3_destroy(handle: *mut ellm_matmul3) -> c_int;
+    pub fn ellm_matmul3_attn_run(
+        proj: *mut ellm_matmul3,
+        attn: *mut ellm_attn,
+        position_index: usize,
+        batch_size: usize,
+        stream: Stream,
+    ) -> c_int;
+    pub fn ellm_matmul3_attn_run_ragged(
+        proj: *mut ellm_matmul3,
+        attn: *mut ellm_attn,
+        positions: *const u32,
+        max_position: usize,
+        batch_size: usize,
+        stream: Stream,
+    ) -> c_int;
+    pub fn ellm_matmul3_attn_path(proj: *const ellm_matmul3, attn: *const ellm_attn, batch_size: usize) -> c_int;
 
     pub fn ellm_matmul_add_create(desc: *const ellm_matmul_add_desc, out_handle: *mut *mut ellm_matmul_add) -> c_int;
     pub fn ellm_matmul_add_run(
@@ -504,6 +520,19 @@ impl MatMul3<Half> {
         check(
             unsafe { ellm_matmul3_run_ragged(self.handle, positions, max_position, batch_size, self.stream) },
             "ellm_matmul3_run_ragged",
+        );
+    }
+
+    /// This operator and the `Attention` that follows it in the queue
+    /// (src/qwen3_moe/attention.rs:126-174) for a step of one position, as one call: what
+    /// `run(position_index, 1, ..)` followed by `attention.run(position_index, 1, ..)` leaves.
+    pub fn run_with_attention(&self, attention: &Attention<T>, position_index: usize, batch_size: usize, thread_id: usize) {
+        if thread_id != 0 {
+            return;
+        }
+        check(
+            unsafe { ellm_matmul3_attn_run(self.handle, attention.handle, position_index, batch_size, self.stream) },
+            "ellm_matmul3_attn_run",
         );
     }
 }

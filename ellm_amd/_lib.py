@@ -158,6 +158,9 @@ ABI_SYMBOLS = {
     "ellm_matmul3_run": (ctypes.c_int, [_vp, _sz, _sz, _sz, _vp]),
     "ellm_matmul3_run_ragged": (ctypes.c_int, [_vp, _vp, _sz, _sz, _vp]),
     "ellm_matmul3_destroy": (ctypes.c_int, [_vp]),
+    "ellm_matmul3_attn_run": (ctypes.c_int, [_vp, _vp, _sz, _sz, _vp]),
+    "ellm_matmul3_attn_run_ragged": (ctypes.c_int, [_vp, _vp, _vp, _sz, _sz, _vp]),
+    "ellm_matmul3_attn_path": (ctypes.c_int, [_vp, _vp, _sz]),
     "ellm_matmul_add_create": (ctypes.c_int, [ctypes.POINTER(MatMulAddDesc), _pvp]),
     "ellm_matmul_add_run": (ctypes.c_int, [_vp, _sz, _sz, _sz, _vp]),
     "ellm_matmul_add_destroy": (ctypes.c_int, [_vp]),

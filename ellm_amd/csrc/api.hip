@@ -9,6 +9,7 @@
 #include <vector>
 
 #include "../../include/ellm_attn.h"
+#include "handles.hpp"
 #include "kernels.hpp"
 
 namespace {
@@ -134,28 +135,8 @@ void ellm::attn_args_from_desc(const ellm_attn_desc& d, ellm::AttnArgs* a) {
   a->positions = nullptr;
   a->seq_offsets = nullptr;
   a->seq_caps = nullptr;
+  a->pending = ellm::PendingRows{};
 }
-
-struct ellm_attn {
-  ellm_attn_desc desc;
-  int device;
-  int n_cu;
-  float* ws_acc;
-  float* ws_ml;
-  float* ws2_acc;
-  float* ws2_ml;
-  uint32_t* counters;
-  ellm::DecodeWorkspace ws;
-  // chunk calls with few row blocks on a long cache split the key range: partial rows
-  float* part_o;
-  float* part_ml;
-  size_t part_rows;
-  // sequences of different capacities (ellm_attn_create_ragged): device tables (borrowed from
-  // the cache) and a host copy of the capacities for the range checks; empty / null otherwise
-  const size_t* seq_offsets;
-  const uint32_t* seq_caps;
-  std::vector<size_t> caps_host;
-};
 
 struct ellm_kv_cache {
   ellm_kv_desc desc;   // capacity = the largest per-sequence capacity
@@ -321,7 +302,9 @@ int ellm_attn_destroy(ellm_attn* h) {
   return ELLM_OK;
 }
 
-static void fill_args(const ellm_attn* h, ellm::AttnArgs* a) {
+}  // extern "C"
+
+void ellm::attn_fill_args(const ellm_attn* h, ellm::AttnArgs* a) {
   ellm::attn_args_from_desc(h->desc, a);
   a->ws_acc = h->ws_acc;
   a->ws_ml = h->ws_ml;
@@ -346,7 +329,7 @@ static bool takes_balanced(const ellm_attn* h, size_t batch, size_t max_position
                                      (uint32_t)max_position + 1, *wgs);
 }
 
-static int run_decode(ellm_attn* h, ellm::AttnArgs* a, uint32_t max_position, hipStream_t stream) {
+int ellm::attn_run_single_token(ellm_attn* h, ellm::AttnArgs* a, uint32_t max_position, hipStream_t stream) {
   uint32_t wgs = 0;
   if (a->positions && takes_balanced(h, a->batch, max_position, &wgs)) {
     const hipError_t e = ellm::launch_decode_balanced(*a, wgs, stream);
@@ -363,6 +346,8 @@ static int run_decode(ellm_attn* h, ellm::AttnArgs* a, uint32_t max_position, hi
   if (e != hipSuccess) return fail_hip(e, "single-token attention launch");
   return ELLM_OK;
 }
+
+extern "C" {
 
 int ellm_attn_run(ellm_attn* h, size_t position_index, size_t position_interval, size_t batch_size,
                   void* stream) {
@@ -386,11 +371,11 @@ int ellm_attn_run(ellm_attn* h, size_t position_index, size_t position_interval,
       return fail(ELLM_ERR_OUT_OF_RANGE, "positions [%zu, %zu) do not fit sequence %zu, whose capacity is %zu",
                   position_index, position_index + position_interval, i, h->caps_host[i]);
   ellm::AttnArgs a;
-  fill_args(h, &a);
+  ellm::attn_fill_args(h, &a);
   a.position_index = (uint32_t)position_index;
   a.position_interval = (uint32_t)position_interval;
   a.batch = (uint32_t)batch_size;
-  if (position_interval == 1) return run_decode(h, &a, (uint32_t)position_index, (hipStream_t)stream);
+  if (position_interval == 1) return ellm::attn_run_single_token(h, &a, (uint32_t)position_index, (hipStream_t)stream);
   hipError_t e = ellm::launch_prefill(a, (hipStream_t)stream);
   if (e != hipSuccess) return fail_hip(e, "chunk attention launch");
   return ELLM_OK;
@@ -410,12 +395,12 @@ int ellm_attn_run_ragged(ellm_attn* h, const uint32_t* positions, size_t max_pos
     return fail(ELLM_ERR_OUT_OF_RANGE, "max_position %zu is not below the sequence capacity %zu",
                 max_position, d.sequence_capacity);
   ellm::AttnArgs a;
-  fill_args(h, &a);
+  ellm::attn_fill_args(h, &a);
   a.position_index = (uint32_t)max_position;
   a.position_interval = 1;
   a.batch = (uint32_t)batch_size;
   a.positions = positions;
-  return run_decode(h, &a, (uint32_t)max_position, (hipStream_t)stream);
+  return ellm::attn_run_single_token(h, &a, (uint32_t)max_position, (hipStream_t)stream);
 }
 
 int ellm_attn_ragged_path(const ellm_attn* h, size_t max_position, size_t batch_size) {

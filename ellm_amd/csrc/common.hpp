@@ -148,6 +148,34 @@ __device__ __forceinline__ size_t seq_plane_offset(const size_t* table, size_t s
   return table ? table[seq] : (size_t)seq * stride;
 }
 
+// What the fused Q/K/V projection does to every finished query / key head row (reference:
+// matmul_finalize_rmsnorm_rope_inplace_3x128, src/kernel/x86_64/f16_512/matmul_rms_complex.rs:76-96),
+// on the eight consecutive elements a lane holds:
+//   sum of squares of the lane's eight elements, in order, with fused multiply-adds;
+//   y = x / (sqrt(mean of squares) + eps), eps added to the root (src/kernel/generic/rms_norm.rs:19);
+//   (a, b) -> (a cos - b sin, a sin + b cos) with the four (cos, sin) pairs of `rope8`.
+// The caller adds the lanes' sums of squares up to the head's 128 elements in between.
+__device__ __forceinline__ float squares8(const float (&x)[8]) {
+  float ss = 0.0f;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) ss = fmaf(x[e], x[e], ss);
+  return ss;
+}
+__device__ __forceinline__ float inverse_rms(float sum_of_squares, float eps) {
+  return 1.0f / (sqrtf(sum_of_squares / (float)kHeadDim) + eps);
+}
+template <typename T>
+__device__ __forceinline__ u32x4 scale_rotate_pack8(const float (&x)[8], float inv, u32x4 rope8) {
+  u32x4 out;
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    const float cs = Mfma<T>::to_float((uint16_t)(rope8[e] & 0xffffu)), sn = Mfma<T>::to_float((uint16_t)(rope8[e] >> 16));
+    const float y0 = x[2 * e] * inv, y1 = x[2 * e + 1] * inv;
+    out[e] = Mfma<T>::pack2(y0 * cs - y1 * sn, y0 * sn + y1 * cs);
+  }
+  return out;
+}
+
 constexpr float kLog2e = 1.4426950408889634f;
 constexpr float kLn2 = 0.6931471805599453f;
 

@@ -29,8 +29,10 @@ namespace ellm {
 using namespace dec;
 namespace {
 
-template <typename T>
-__global__ __launch_bounds__(kDecThreads, 4) void decode_split_kernel(DecodeKernelArgs p) {
+// PENDING: the launch of a fused step (ellm_matmul3_attn_run): the query rows and the new key /
+// value row of every plane come as the projection's raw sums (p.pend) and are finished here.
+template <typename T, bool PENDING>
+__global__ __launch_bounds__(kDecThreads, PENDING ? 2 : 4) void decode_split_kernel(DecodeKernelArgs p) {
   __shared__ __attribute__((aligned(16))) uint16_t smem[kDecWaves * kWaveLdsHalves];
   __shared__ uint32_t s_last;
 
@@ -60,12 +62,32 @@ __global__ __launch_bounds__(kDecThreads, 4) void decode_split_kernel(DecodeKern
   const uint32_t head0 = kvh * p.group + hgrp * kMaxHeadsPerGroup;
   const uint32_t row0 = seq * p.n_q_heads + head0;  // output row of the group's first head
   u32x4 qreg[4];
-  load_queries(p.q + (size_t)row0 * kHeadDim, t, heads_here, qreg);
-
   float m_run, l_run;
   f32x4 acc[8];
-  stream_keys<T>(p.k + plane, p.v + plane, p.kv_stride_pos, k_begin, k_end, pos, qreg, smem, t,
-                 split * 7u + blockIdx.y * 3u + seq * 5u, p.scale_log2, m_run, l_run, acc);
+  if constexpr (PENDING) {
+    NewRow fresh;
+    fresh.present = k_end == len;   // the split that holds the plane's last key
+    fresh.store = hgrp == 0;
+    const size_t col_k = (size_t)seq * p.pend.cols + (size_t)(p.n_q_heads + kvh) * kHeadDim;
+    fresh.k_raw = p.pend.raw + col_k;
+    fresh.v_raw = p.pend.raw + col_k + (size_t)p.n_kv_heads * kHeadDim;
+    fresh.parts = p.pend.parts;
+    fresh.part_stride = p.pend.part_stride;
+    fresh.rope_row = (const uint16_t*)p.pend.rope + (size_t)pos * p.pend.rope_pos_stride +
+                     (size_t)kvh * p.pend.rope_head_stride;
+    fresh.eps = p.pend.eps;
+    fresh.k_dst = const_cast<uint16_t*>(p.k) + plane + (size_t)pos * p.kv_stride_pos;
+    fresh.v_dst = const_cast<uint16_t*>(p.v) + plane + (size_t)pos * p.kv_stride_pos;
+    stream_keys<T, true>(p.k + plane, p.v + plane, p.kv_stride_pos, k_begin, k_end, pos, qreg, smem, t,
+                         split * 7u + blockIdx.y * 3u + seq * 5u, p.scale_log2, m_run, l_run, acc, &fresh,
+                         [&]() { load_queries_pending<T>(p.pend, seq, head0, pos, t, heads_here, qreg); });
+    // the finished query rows, once per group: by the workgroup that also wrote the new key
+    if (fresh.present) store_queries(const_cast<uint16_t*>(p.q) + (size_t)row0 * kHeadDim, t, heads_here, qreg);
+  } else {
+    load_queries(p.q + (size_t)row0 * kHeadDim, t, heads_here, qreg);
+    stream_keys<T>(p.k + plane, p.v + plane, p.kv_stride_pos, k_begin, k_end, pos, qreg, smem, t,
+                   split * 7u + blockIdx.y * 3u + seq * 5u, p.scale_log2, m_run, l_run, acc);
+  }
 
   auto final_row = [&](uint32_t h, uint32_t dq, const f32x4& a, float l, float m) {
     emit_final<T>(p.out, p.lse, row0 + h, dq, a, l, m);
@@ -141,13 +163,20 @@ hipError_t launch_decode(const AttnArgs& a, hipStream_t stream) {
   p.n_split = a.n_split;
   p.batch = a.batch;
   p.scale_log2 = a.scale * kLog2e;
+  p.pend = a.pending;
 
   dim3 grid(a.n_split, a.n_kv_heads * p.head_groups, a.batch);
   dim3 block(kDecThreads);
-  if (a.dtype == 0)
-    hipLaunchKernelGGL((decode_split_kernel<F16>), grid, block, 0, stream, p);
-  else
-    hipLaunchKernelGGL((decode_split_kernel<BF16>), grid, block, 0, stream, p);
+  if (a.pending.raw) {
+    if (a.dtype == 0)
+      hipLaunchKernelGGL((decode_split_kernel<F16, true>), grid, block, 0, stream, p);
+    else
+      hipLaunchKernelGGL((decode_split_kernel<BF16, true>), grid, block, 0, stream, p);
+  } else if (a.dtype == 0) {
+    hipLaunchKernelGGL((decode_split_kernel<F16, false>), grid, block, 0, stream, p);
+  } else {
+    hipLaunchKernelGGL((decode_split_kernel<BF16, false>), grid, block, 0, stream, p);
+  }
   return hipGetLastError();
 }
 

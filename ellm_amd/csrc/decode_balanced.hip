@@ -37,7 +37,8 @@ __device__ __forceinline__ uint32_t uni(uint32_t v) { return (uint32_t)__builtin
 // clusters of 16 pieces take cluster slots p + slot0 / 16 + c, which are distinct for the same
 // reason (1 + floor(n / 16) >= ceil(n / 16)).
 
-template <typename T>
+// PENDING: the launch of a fused step, as in decode.hip.
+template <typename T, bool PENDING>
 __global__ __launch_bounds__(kDecThreads, 2) void decode_balanced_kernel(DecodeKernelArgs p) {
   __shared__ __attribute__((aligned(16))) uint16_t smem[kDecWaves * kWaveLdsHalves];
   __shared__ uint32_t prefix[kMaxBatch + 1];   // units of the sequences before sequence b (per plane)
@@ -205,12 +206,31 @@ __global__ __launch_bounds__(kDecThreads, 2) void decode_balanced_kernel(DecodeK
     const uint32_t head0 = kvh * p.group + hgrp * kMaxHeadsPerGroup;
     const uint32_t row0 = seq * p.n_q_heads + head0;
     u32x4 qreg[4];
-    load_queries(p.q + (size_t)row0 * kHeadDim, t, heads_here, qreg);
-
     float m_run, l_run;
     f32x4 acc[8];
-    stream_keys<T>(p.k + plane, p.v + plane, p.kv_stride_pos, k_begin, k_end, pos, qreg, smem, t,
-                   w * 7u + pl * 3u + seq * 5u, p.scale_log2, m_run, l_run, acc);
+    if constexpr (PENDING) {
+      NewRow fresh;
+      fresh.present = k_end == pos + 1;   // the piece that holds the plane's last key
+      fresh.store = hgrp == 0;
+      const size_t col_k = (size_t)seq * p.pend.cols + (size_t)(p.n_q_heads + kvh) * kHeadDim;
+      fresh.k_raw = p.pend.raw + col_k;
+      fresh.v_raw = p.pend.raw + col_k + (size_t)p.n_kv_heads * kHeadDim;
+      fresh.parts = p.pend.parts;
+      fresh.part_stride = p.pend.part_stride;
+      fresh.rope_row = (const uint16_t*)p.pend.rope + (size_t)pos * p.pend.rope_pos_stride +
+                       (size_t)kvh * p.pend.rope_head_stride;
+      fresh.eps = p.pend.eps;
+      fresh.k_dst = const_cast<uint16_t*>(p.k) + plane + (size_t)pos * p.kv_stride_pos;
+      fresh.v_dst = const_cast<uint16_t*>(p.v) + plane + (size_t)pos * p.kv_stride_pos;
+      stream_keys<T, true>(p.k + plane, p.v + plane, p.kv_stride_pos, k_begin, k_end, pos, qreg, smem, t,
+                           w * 7u + pl * 3u + seq * 5u, p.scale_log2, m_run, l_run, acc, &fresh,
+                           [&]() { load_queries_pending<T>(p.pend, seq, head0, pos, t, heads_here, qreg); });
+      if (fresh.present) store_queries(const_cast<uint16_t*>(p.q) + (size_t)row0 * kHeadDim, t, heads_here, qreg);
+    } else {
+      load_queries(p.q + (size_t)row0 * kHeadDim, t, heads_here, qreg);
+      stream_keys<T>(p.k + plane, p.v + plane, p.kv_stride_pos, k_begin, k_end, pos, qreg, smem, t,
+                     w * 7u + pl * 3u + seq * 5u, p.scale_log2, m_run, l_run, acc);
+    }
 
     auto final_row = [&](uint32_t h, uint32_t dq, const f32x4& av, float l, float m) {
       emit_final<T>(p.out, p.lse, (size_t)(row0 + h), dq, av, l, m);
@@ -295,10 +315,18 @@ hipError_t launch_decode_balanced(const AttnArgs& a, uint32_t wgs, hipStream_t s
   const uint32_t planes = a.batch * a.n_kv_heads * p.head_groups;
   p.n_cluster_max = planes + (wgs + planes) / kMergeFan + 2;
   p.counters_per_plane = 0;
-  if (a.dtype == 0)
-    hipLaunchKernelGGL((decode_balanced_kernel<F16>), dim3(wgs), dim3(kDecThreads), 0, stream, p);
-  else
-    hipLaunchKernelGGL((decode_balanced_kernel<BF16>), dim3(wgs), dim3(kDecThreads), 0, stream, p);
+  p.pend = a.pending;
+  const dim3 grid(wgs), block(kDecThreads);
+  if (a.pending.raw) {
+    if (a.dtype == 0)
+      hipLaunchKernelGGL((decode_balanced_kernel<F16, true>), grid, block, 0, stream, p);
+    else
+      hipLaunchKernelGGL((decode_balanced_kernel<BF16, true>), grid, block, 0, stream, p);
+  } else if (a.dtype == 0) {
+    hipLaunchKernelGGL((decode_balanced_kernel<F16, false>), grid, block, 0, stream, p);
+  } else {
+    hipLaunchKernelGGL((decode_balanced_kernel<BF16, false>), grid, block, 0, stream, p);
+  }
   return hipGetLastError();
 }
 

@@ -48,6 +48,7 @@ struct DecodeKernelArgs {
   uint32_t batch;     // sequences (decode_balanced.hip)
   uint32_t wgs_one;   // workgroups that find a compute unit each (decode_balanced.hip)
   float scale_log2;   // scale * log2(e)
+  PendingRows pend;   // raw query / key / value rows of a fused step (kernels built with PENDING)
 };
 
 // Agent-scope (device-wide coherent) relaxed 8-byte load / store of a pair of floats.
@@ -105,6 +106,98 @@ __device__ __forceinline__ void load_queries(const uint16_t* q_rows, const Lane&
   }
 }
 
+// ---- fused step: the rows the projection left raw ----------------------------------------
+
+// The eight values at `src`: binary32 partial sums, one or two of them `stride` floats apart.
+__device__ __forceinline__ void sum_parts8(const float* src, uint32_t parts, uint32_t stride, float (&x)[8]) {
+  f32x4 lo = *(const f32x4*)src, hi = *(const f32x4*)(src + 4);
+  if (parts > 1) {   // (uniform)
+    lo += *(const f32x4*)(src + stride);
+    hi += *(const f32x4*)(src + stride + 4);
+  }
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    x[e] = lo[e];
+    x[4 + e] = hi[e];
+  }
+}
+
+// load_queries() for a fused step: the group's query rows come as raw sums and are normalised
+// and rotated on the way into the operand registers.  Lane (head c, group g) holds the octets
+// 4 s + g of its head; the sum of squares is added up in the order the projection's own
+// finishing step uses (octet, pairs of octets, fours, eights, all sixteen), so the rows come
+// out with the bits that step gives them.
+template <typename T>
+__device__ __forceinline__ void load_queries_pending(const PendingRows& pr, uint32_t seq, uint32_t head0,
+                                                     uint32_t pos, const Lane& t, uint32_t heads_here,
+                                                     u32x4 (&qreg)[4]) {
+  const bool live = (uint32_t)t.c < heads_here;
+  const uint32_t head = head0 + (live ? t.c : 0);
+  const float* src = pr.raw + (size_t)seq * pr.cols + (size_t)head * kHeadDim + 8 * t.g;
+  const uint16_t* rope = (const uint16_t*)pr.rope + (size_t)pos * pr.rope_pos_stride +
+                         (size_t)head * pr.rope_head_stride + 8 * t.g;
+  float x[4][8];
+  u32x4 rr[4];
+  float ss[4];
+#pragma unroll
+  for (int s = 0; s < 4; ++s) {
+    sum_parts8(src + 32 * s, pr.parts, pr.part_stride, x[s]);
+    rr[s] = load16(rope + 32 * s);
+    ss[s] = squares8(x[s]);
+  }
+#pragma unroll
+  for (int s = 0; s < 4; ++s) {
+    ss[s] += xor_shuffle(ss[s], 16);
+    ss[s] += xor_shuffle(ss[s], 32);
+  }
+  const float inv = inverse_rms((ss[0] + ss[1]) + (ss[2] + ss[3]), pr.eps);
+#pragma unroll
+  for (int s = 0; s < 4; ++s) {
+    qreg[s] = scale_rotate_pack8<T>(x[s], inv, rr[s]);
+    if (!live) qreg[s] = u32x4{0, 0, 0, 0};
+  }
+}
+// The finished query rows go back to where the projection alone would have left them.
+__device__ __forceinline__ void store_queries(uint16_t* q_rows, const Lane& t, uint32_t heads_here,
+                                              const u32x4 (&qreg)[4]) {
+  if ((uint32_t)t.c >= heads_here) return;
+#pragma unroll
+  for (int s = 0; s < 4; ++s) store16(q_rows + (size_t)t.c * kHeadDim + 32 * s + 8 * t.g, qreg[s]);
+}
+
+// The key and value row a fused step adds to a plane: where their raw sums are, and the cache
+// rows they belong in (written by the workgroup that holds the plane's last key).
+struct NewRow {
+  bool present;              // this stretch of keys ends with the plane's new key
+  bool store;                // ... and this workgroup is the one that writes it to the cache
+  const float* k_raw;        // 128 raw sums each (first part)
+  const float* v_raw;
+  uint32_t parts, part_stride;
+  const uint16_t* rope_row;  // rotary row of (position, kv head)
+  float eps;
+  uint16_t* k_dst;
+  uint16_t* v_dst;
+};
+// Every lane c of each 16-lane group ends up with elements 8 c .. 8 c + 7 of the finished rows
+// (the arithmetic of the projection's own finishing step, lane for lane).
+template <typename T>
+__device__ __forceinline__ void finish_new_row(const NewRow& n, const Lane& t, u32x4& knew, u32x4& vnew) {
+  float kx[8], vx[8];
+  sum_parts8(n.k_raw + 8 * t.c, n.parts, n.part_stride, kx);
+  sum_parts8(n.v_raw + 8 * t.c, n.parts, n.part_stride, vx);
+  const u32x4 rr = load16(n.rope_row + 8 * t.c);
+  float ss = squares8(kx);
+#pragma unroll
+  for (int m = 1; m < 16; m <<= 1) ss += __shfl_xor(ss, m, 16);
+  knew = scale_rotate_pack8<T>(kx, inverse_rms(ss, n.eps), rr);
+  vnew = u32x4{Mfma<T>::pack2(vx[0], vx[1]), Mfma<T>::pack2(vx[2], vx[3]), Mfma<T>::pack2(vx[4], vx[5]),
+               Mfma<T>::pack2(vx[6], vx[7])};
+  if (n.store && t.g == 0) {
+    store16(n.k_dst + 8 * t.c, knew);
+    store16(n.v_dst + 8 * t.c, vnew);
+  }
+}
+
 // One wave's share of keys [k_begin, k_end) of a plane: the four waves take alternating 16-key
 // chunks, each streams its chunks HBM -> registers (128-bit loads, four full 256-byte rows per
 // instruction) -> its private LDS slice -> MFMA operands, so no workgroup barrier is needed
@@ -116,17 +209,38 @@ __device__ __forceinline__ void load_queries(const uint16_t* q_rows, const Lane&
 // Chunks are visited in an order rotated by `rot_seed` (soft-max accumulation does not care
 // about order): splits start at offsets that are multiples of the split length, and walking
 // them in lockstep would keep every stream on the same few HBM channels.
-template <typename T>
+// PENDING (a fused step): when `fresh.present`, key `pos` is not in the cache yet; the stream
+// covers [k_begin, pos) and the wave with the fewest chunks finishes the new key / value row
+// from the projection's raw sums (requested before its stream starts), writes it to the cache
+// and takes it as one more chunk of its own.
+// The raw rows are fetched behind the wave's first chunk of keys (`late_queries()` fills qreg
+// from the raw query rows at that point), so that their trip to memory runs beside the first
+// chunk's and not ahead of it.
+struct NoLateQueries {
+  __device__ __forceinline__ void operator()() const {}
+};
+template <typename T, bool PENDING = false, typename LateQueries = NoLateQueries>
 __device__ __forceinline__ void stream_keys(const uint16_t* kplane, const uint16_t* vplane, size_t stride_pos,
                                             uint32_t k_begin, uint32_t k_end, uint32_t pos,
                                             const u32x4 (&qreg)[4], uint16_t* smem, const Lane& t,
                                             uint32_t rot_seed, float scale_log2, float& m_out, float& l_out,
-                                            f32x4 (&acc)[8]) {
+                                            f32x4 (&acc)[8], const NewRow* fresh = nullptr,
+                                            LateQueries late_queries = NoLateQueries()) {
   const int g = t.g, c = t.c, wave = t.wave;
   uint16_t* ks = smem + wave * kWaveLdsHalves;  // [16][kKPitch]
   uint16_t* vt = ks + kChunk * kKPitch;         // [128][kVtPitch]
 
+  const uint32_t new_pos = pos;   // (PENDING) the position of the new key
+  bool take_new = false;
+  if constexpr (PENDING) {
+    if (fresh->present) {   // the stream ends before the new key; its last valid row is pos - 1
+      k_end = pos;
+      pos = pos ? pos - 1 : 0;
+    }
+  }
   const uint32_t n_chunks = (k_end - k_begin + kChunk - 1) / kChunk;
+  u32x4 knew = {0, 0, 0, 0}, vnew = {0, 0, 0, 0};
+  if constexpr (PENDING) take_new = fresh->present && (uint32_t)wave == n_chunks % kDecWaves;   // (uniform over the wave)
   // one 16-key chunk in flight per wave (a second one measured no faster)
   u32x4 kreg[4], vreg[4];
   auto issue_loads = [&](uint32_t chunk) {
@@ -153,11 +267,8 @@ __device__ __forceinline__ void stream_keys(const uint16_t* kplane, const uint16
     if (r >= my_chunks) r -= my_chunks;
     return wave + r * kDecWaves;
   };
-  if (my_chunks) issue_loads(chunk_at(0));
-  for (uint32_t it = 0; it < my_chunks; ++it) {
-    const uint32_t chunk = chunk_at(it);
-    const uint32_t kb = k_begin + chunk * kChunk;
-    // registers -> LDS: K row-major, V transposed.
+  // registers -> LDS: K row-major, V transposed.
+  auto stage = [&]() {
 #pragma unroll
     for (int i = 0; i < 4; ++i) store16(ks + (4 * g + i) * kKPitch + 8 * c, kreg[i]);
 #pragma unroll
@@ -166,9 +277,9 @@ __device__ __forceinline__ void stream_keys(const uint16_t* kplane, const uint16
                                 vreg[3][e >> 1], (e & 1) != 0);
       *(u32x2*)(vt + (8 * c + e) * kVtPitch + 4 * g) = col;
     }
-    if (it + 1 < my_chunks) issue_loads(chunk_at(it + 1));
-    __builtin_amdgcn_wave_barrier();
-
+  };
+  // the staged chunk, keys kb .. kb + 15 of which those up to `last` count
+  auto consume = [&](uint32_t kb, uint32_t last) {
     // S^T[key][head], lane (head c, group g) register r <-> key kb + 4 g + r.
     f32x4 st = {0, 0, 0, 0};
 #pragma unroll
@@ -180,7 +291,7 @@ __device__ __forceinline__ void stream_keys(const uint16_t* kplane, const uint16
     float tmax = -INFINITY;
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
-      tt[r] = (kb + 4 * g + r <= pos) ? st[r] * scale_log2 : -INFINITY;
+      tt[r] = (kb + 4 * g + r <= last) ? st[r] * scale_log2 : -INFINITY;
       tmax = fmaxf(tmax, tt[r]);
     }
     tmax = fmaxf(tmax, xor_shuffle(tmax, 16));
@@ -205,7 +316,35 @@ __device__ __forceinline__ void stream_keys(const uint16_t* kplane, const uint16
       u32x2 a = *(const u32x2*)(vt + (16 * b + c) * kVtPitch + 4 * g);
       acc[b] = Mfma<T>::m16x16x16(a, pb, acc[b]);
     }
+  };
+
+  if (my_chunks) issue_loads(chunk_at(0));
+  if constexpr (PENDING) {
+    late_queries();
+    if (take_new) finish_new_row<T>(*fresh, t, knew, vnew);
+  }
+  for (uint32_t it = 0; it < my_chunks; ++it) {
+    const uint32_t chunk = chunk_at(it);
+    const uint32_t kb = k_begin + chunk * kChunk;
+    stage();
+    if (it + 1 < my_chunks) issue_loads(chunk_at(it + 1));
     __builtin_amdgcn_wave_barrier();
+    consume(kb, pos);
+    __builtin_amdgcn_wave_barrier();
+  }
+  if constexpr (PENDING) {
+    if (take_new) {   // a chunk whose first row is the new key; its other rows are zeros and do not count
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const bool first = g == 0 && i == 0;
+        kreg[i] = first ? knew : u32x4{0, 0, 0, 0};
+        vreg[i] = first ? vnew : u32x4{0, 0, 0, 0};
+      }
+      stage();
+      __builtin_amdgcn_wave_barrier();
+      consume(new_pos, new_pos);
+      __builtin_amdgcn_wave_barrier();
+    }
   }
 
   l_run += xor_shuffle(l_run, 16);

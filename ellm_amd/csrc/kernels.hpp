@@ -11,6 +11,20 @@ struct ellm_attn_desc;
 
 namespace ellm {
 
+// Raw rows that the Q/K/V projection of a fused single-token step left for the attention
+// kernels to finish: binary32 sums [part][sequence][column], column = head x 128 + element over
+// the query heads, then the key heads, then the value heads.  A value is the sum of its `parts`
+// (one or two) partial sums.  The attention kernels
+// normalise and rotate the query and key heads while they load them and write the finished
+// query rows, the new key row and the new value row to where the projection alone would have.
+struct PendingRows {
+  const float* raw;   // null: nothing pending (the ordinary launch)
+  uint32_t parts, part_stride, cols;   // part_stride, cols in floats
+  const void* rope;   // (cos, sin) pairs, as in ProjectArgs
+  uint32_t rope_pos_stride, rope_head_stride;
+  float eps;
+};
+
 // Everything a launch needs; filled by the C ABI after validation.
 struct AttnArgs {
   const void* q;
@@ -51,6 +65,7 @@ struct AttnArgs {
   float* prefill_part_ml;
   size_t prefill_part_rows;
   uint32_t n_cu;
+  PendingRows pending;   // single-token path only
 };
 // Partial rows the chunk path's workspace holds for an operator of this shape (0: none needed).
 size_t prefill_workspace_rows(uint32_t max_interval, uint32_t batch_capacity, uint32_t n_q_heads,
@@ -121,7 +136,12 @@ struct ProjectArgs {
   // workspace of the few-rows kernel (may be null: the tile kernel runs whatever the row count)
   float* ws;
   uint32_t* counters;
+  // raw_out: the few-rows kernel leaves the binary32 sums of every column in ws, laid out as
+  // PendingRows describes (one part), and writes nothing else (requires project_raw_takes())
+  uint32_t raw_out;
 };
+// Whether a projection of this shape can leave raw rows (the few-rows kernel takes it).
+bool project_raw_takes(uint32_t rows, uint32_t heads, uint32_t K, bool has_workspace);
 hipError_t launch_project(const ProjectArgs& a, hipStream_t stream);
 // Few-rows kernel: rows it handles at most, floats of partial sums and counters it needs.
 size_t project_workspace_floats(uint32_t heads, uint32_t K);

@@ -232,6 +232,10 @@ int project_path(uint32_t rows, uint32_t heads, uint32_t K, bool has_workspace) 
   return kPathTiles;
 }
 
+bool project_raw_takes(uint32_t rows, uint32_t heads, uint32_t K, bool has_workspace) {
+  return project_path(rows, heads, K, has_workspace) == kPathFewRows;
+}
+
 hipError_t launch_project(const ProjectArgs& a, hipStream_t stream) {
   if (a.rows == 0) return hipSuccess;
   ProjectKernelArgs p;
@@ -266,8 +270,12 @@ hipError_t launch_project(const ProjectArgs& a, hipStream_t stream) {
   p.finalize0 = a.finalize0;
   p.eps = a.eps;
   const int path = project_path(a.rows, a.heads0 + 2 * a.heads_kv, a.K, a.ws && a.counters);
+  if (a.raw_out) {
+    if (path != kPathFewRows || a.residual) return hipErrorInvalidValue;   // (project_raw_takes() said otherwise)
+    return launch_project_small(p, a.ws, a.counters, a.dtype, kModeRaw, stream);
+  }
   if (path == kPathFewRows)
-    return launch_project_small(p, a.ws, a.counters, a.dtype, a.residual != nullptr, stream);
+    return launch_project_small(p, a.ws, a.counters, a.dtype, a.residual ? kModeAdd : kModeQkv, stream);
   if (path == kPathTiles128 || path == kPathTiles256x1)
     return launch_project_mid(p, path == kPathTiles128 ? 1 : 2, a.dtype, a.residual != nullptr, stream);
   const uint32_t blocks = p.tiles_m * p.tiles_n;

@@ -8,6 +8,7 @@
 #include <vector>
 
 #include "../../include/ellm_attn.h"
+#include "handles.hpp"
 #include "kernels.hpp"
 
 namespace {
@@ -15,16 +16,6 @@ bool aligned16(const void* p) { return ((uintptr_t)p & 15u) == 0; }
 constexpr size_t kMaxK = 1u << 16;
 }  // namespace
 
-struct ellm_matmul3 {
-  ellm_matmul3_desc d;
-  int device;
-  float* ws;
-  uint32_t* counters;
-  // destination with per-sequence capacities (ellm_matmul3_create_ragged); null / empty otherwise
-  const size_t* seq_offsets;
-  const uint32_t* seq_caps;
-  std::vector<size_t> caps_host;
-};
 struct ellm_matmul_add {
   ellm_matmul_add_desc d;
   int device;
@@ -165,11 +156,12 @@ int ellm_matmul3_destroy(ellm_matmul3* h) {
   return rc;
 }
 
-static int matmul3_launch(ellm_matmul3* h, size_t position_index, size_t position_interval,
-                          size_t batch_size, const uint32_t* positions, size_t max_start,
-                          void* stream) {
+}  // extern "C"
+
+int ellm::matmul3_fill_args(const ellm_matmul3* h, size_t position_index, size_t position_interval,
+                            size_t batch_size, const uint32_t* positions, size_t max_start,
+                            ellm::ProjectArgs* out) {
   const ellm_matmul3_desc& d = h->d;
-  if (position_interval == 0 || batch_size == 0) return ELLM_OK;
   if (int st = ellm::check_current_device(h->device)) return st;
   if (position_interval > d.max_position_interval)
     return ellm::set_error(ELLM_ERR_OUT_OF_RANGE, "position_interval %zu exceeds max_position_interval %zu", position_interval, d.max_position_interval);
@@ -216,6 +208,19 @@ static int matmul3_launch(ellm_matmul3* h, size_t position_index, size_t positio
   a.dtype = d.dtype;
   a.ws = h->ws;
   a.counters = h->counters;
+  *out = a;
+  return ELLM_OK;
+}
+
+extern "C" {
+
+static int matmul3_launch(ellm_matmul3* h, size_t position_index, size_t position_interval,
+                          size_t batch_size, const uint32_t* positions, size_t max_start,
+                          void* stream) {
+  if (position_interval == 0 || batch_size == 0) return ELLM_OK;
+  ellm::ProjectArgs a{};
+  if (int st = ellm::matmul3_fill_args(h, position_index, position_interval, batch_size, positions, max_start, &a))
+    return st;
   const hipError_t e = ellm::launch_project(a, (hipStream_t)stream);
   if (e != hipSuccess) return ellm::set_error(ELLM_ERR_HIP, "projection launch: %s", hipGetErrorString(e));
   return ELLM_OK;

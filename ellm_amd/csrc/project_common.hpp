@@ -58,6 +58,8 @@ __device__ __forceinline__ uint64_t uniform64(const void* p) {
 
 constexpr int kModeQkv = 0;  // heads normalised + rotated (or passed through), K/V to token coordinates
 constexpr int kModeAdd = 1;  // plain product plus a residual of the output's layout
+constexpr int kModeRaw = 2;  // the binary32 sums of every column to the workspace, [row][column]: a fused
+                             // single-token step, whose attention kernel finishes the rows (few-rows kernel only)
 
 // Streaming kernel for a few rows (project_small.hip).  It would take up to 128 rows, but from
 // about 64 on one 128-token tile per head (project_mid.hip) is faster: measured for the
@@ -66,8 +68,9 @@ constexpr uint32_t kSmallRowsMax = 64;
 hipError_t small_prepare();
 bool small_kernel_takes(uint32_t rows, uint32_t K);
 size_t small_workspace_floats(uint32_t heads, uint32_t K);
+// mode: kModeQkv, kModeAdd or kModeRaw
 hipError_t launch_project_small(const ProjectKernelArgs& p, float* ws, uint32_t* counters, int dtype,
-                                bool add, hipStream_t stream);
+                                int mode, hipStream_t stream);
 
 // Tile kernel with 128-token x one-head tiles (project_mid.hip), for row counts at which
 // the 256 x 256 tiles are fewer than the compute units.

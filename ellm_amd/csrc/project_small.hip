@@ -103,7 +103,12 @@ __global__ __launch_bounds__((NTB == 2 || NB == 2) ? 512 : 1024) void project_sm
       f32x4 v = {0.0f, 0.0f, 0.0f, 0.0f};
       for (int w = 0; w < n_waves; ++w)
         v += *(const f32x4*)(sums + (w * kPassRows + tid / kQuads) * kGroupCols + 4 * c4);
-      if (finalize) {
+      if constexpr (MODE == kModeRaw) {
+        // plain stores: the kernel that reads them is the next launch on the stream
+        const uint32_t cols = (p.heads0 + 2 * p.heads_kv) * kHeadDim;
+        if (R < p.rows && R % p.batch_pitch < p.batch)
+          *(f32x4*)(ws + (size_t)R * cols + hh * kHeadDim + kGroupCols * cg + 4 * c4) = v;
+      } else if (finalize) {
         float* to = ws + (((size_t)hh * kGroupsPerHead + cg) * rows_cap + R) * kGroupCols + 4 * c4;
 #pragma unroll
         for (int e = 0; e < 4; ++e) store_coherent(to + e, v[e]);
@@ -247,27 +252,17 @@ __global__ __launch_bounds__((NTB == 2 || NB == 2) ? 512 : 1024) void project_sm
     const uint32_t pos = t + (p.positions ? (live ? min(p.positions[b], p.max_start) : 0u) : p.position_index);
     u32x4 rr = {one_zero, one_zero, one_zero, one_zero};
     if (live) rr = load16(p.rope + (size_t)pos * p.rope_pos_stride + (size_t)hs * p.rope_head_stride + 8 * c8);
-    float o[8] = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-    float ss = 0.0f;
-#pragma unroll
-    for (int e = 0; e < 8; ++e) ss = fmaf(o[e], o[e], ss);
+    const float o[8] = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+    float ss = squares8(o);
 #pragma unroll
     for (int m = 1; m < 16; m <<= 1) ss += __shfl_xor(ss, m, 16);
-    const float inv = 1.0f / (sqrtf(ss / (float)kHeadDim) + p.eps);
-#pragma unroll
-    for (int e = 0; e < 4; ++e) {
-      const float cs = M::to_float((uint16_t)(rr[e] & 0xffffu)), sn = M::to_float((uint16_t)(rr[e] >> 16));
-      const float y0 = o[2 * e] * inv, y1 = o[2 * e + 1] * inv;
-      o[2 * e] = y0 * cs - y1 * sn;
-      o[2 * e + 1] = y0 * sn + y1 * cs;
-    }
+    const u32x4 packed = scale_rotate_pack8<S>(o, inverse_rms(ss, p.eps), rr);
     if (live) {
       size_t off;
       if (seg == 0)
         off = (size_t)R * p.ld0 + hs * kHeadDim + 8 * c8;
       else
         off = kv_row_offset(p, b, hs, pos) + 8 * c8;
-      const u32x4 packed = {M::pack2(o[0], o[1]), M::pack2(o[2], o[3]), M::pack2(o[4], o[5]), M::pack2(o[6], o[7])};
       store16(dst + off, packed);
     }
   }
@@ -336,6 +331,8 @@ hipError_t small_prepare() {
   if (e == hipSuccess) e = prepare_mode<BF16, kModeQkv>();
   if (e == hipSuccess) e = prepare_mode<F16, kModeAdd>();
   if (e == hipSuccess) e = prepare_mode<BF16, kModeAdd>();
+  if (e == hipSuccess) e = prepare_mode<F16, kModeRaw>();
+  if (e == hipSuccess) e = prepare_mode<BF16, kModeRaw>();
   return e;
 }
 
@@ -352,15 +349,19 @@ bool small_kernel_takes(uint32_t rows, uint32_t K) {
 // (rows rounded up to a pass); one counter per head.
 size_t small_workspace_floats(uint32_t heads, uint32_t K) {
   (void)K;
-  return (size_t)heads * (kSmallRowsMax + 32) * kHeadDim;
+  // (also holds the raw rows of a fused single-token step: up to two partial sums of kSmallRowsMax rows)
+  return (size_t)heads * (2 * kSmallRowsMax + 32) * kHeadDim;
 }
 
 hipError_t launch_project_small(const ProjectKernelArgs& p, float* ws, uint32_t* counters, int dtype,
-                                bool add, hipStream_t stream) {
+                                int mode, hipStream_t stream) {
   const uint32_t heads = p.heads0 + 2 * p.heads_kv;
-  if (add)
+  if (mode == kModeAdd)
     return dtype == 0 ? launch_blocks<F16, kModeAdd>(p, ws, counters, heads, stream)
                       : launch_blocks<BF16, kModeAdd>(p, ws, counters, heads, stream);
+  if (mode == kModeRaw)
+    return dtype == 0 ? launch_blocks<F16, kModeRaw>(p, ws, counters, heads, stream)
+                      : launch_blocks<BF16, kModeRaw>(p, ws, counters, heads, stream);
   return dtype == 0 ? launch_blocks<F16, kModeQkv>(p, ws, counters, heads, stream)
                     : launch_blocks<BF16, kModeQkv>(p, ws, counters, heads, stream);
 }

@@ -79,6 +79,26 @@ class MatMul3:
         check(self._lib.ellm_matmul3_run_ragged(self._handle, _positions_ptr(positions, batch_size),
                                                 int(max_position), batch_size, _stream_ptr(stream)))
 
+    def run_with_attention(self, attention, position_index, batch_size, positions=None, stream=None):
+        """This projection and `attention` (an ellm_amd.Attention over the same q / k / v) for one
+        new token per sequence as one call (ellm_matmul3_attn_run / _run_ragged): what run followed
+        by attention.run(position, 1, batch) leaves, with the head rows finished by the attention
+        launch.  positions: per-sequence device positions, position_index then their upper bound."""
+        if positions is None:
+            check(self._lib.ellm_matmul3_attn_run(self._handle, attention._handle, int(position_index),
+                                                  batch_size, _stream_ptr(stream)))
+        else:
+            check(self._lib.ellm_matmul3_attn_run_ragged(self._handle, attention._handle,
+                                                         _positions_ptr(positions, batch_size),
+                                                         int(position_index), batch_size, _stream_ptr(stream)))
+
+    def attention_path(self, attention, batch_size):
+        """1: run_with_attention runs fused for this batch size; 0: as the two ordinary calls."""
+        rc = self._lib.ellm_matmul3_attn_path(self._handle, attention._handle, batch_size)
+        if rc < 0:
+            check(-rc)
+        return rc
+
     def close(self):
         if self._handle:
             check(self._lib.ellm_matmul3_destroy(self._handle))

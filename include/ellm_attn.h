@@ -459,6 +459,32 @@ int ellm_matmul3_destroy(ellm_matmul3* handle);
 int ellm_matmul3_reset(ellm_matmul3* handle, void* stream);
 
 /*
+ * A single-token step's MatMul3::run followed by Attention::run (position_interval 1) as one
+ * call: the two consecutive operators of a layer in the reference's queue
+ * (src/qwen3_moe/attention.rs:126-140 then :169-174; run one after the other by
+ * src/serving/start.rs:69-73).  After the call q_state, k_state / v_state (the cache rows at
+ * the sequences' positions) and the attention output hold what ellm_matmul3_run[_ragged]
+ * followed by ellm_attn_run[_ragged] leaves there, to the same tolerances; in between
+ * nothing is promised (the projection's launch leaves raw binary32 sums in its handle's
+ * workspace and the attention launch normalises and rotates the query and key rows while it
+ * loads them, which spares the projection an exchange between its workgroups).  Two
+ * launches on `stream`, no allocation, no synchronisation: may be recorded into a graph.
+ * The handles must describe the same step: proj's q_state / k_state / v_state are attn's
+ * q / k / v, same dtype, head counts, batch_size, kv_strides, sequence_capacity and (for caches
+ * with per-sequence capacities) the same sequence table; else ELLM_ERR_INVALID_ARGUMENT.
+ * Shapes the fused form does not take (more than 64 sequences, hidden_size not a multiple of
+ * 256 or below 1024) run the two ordinary calls: same results.  ellm_matmul3_attn_path tells
+ * which (1 fused, 0 two ordinary calls, negative: a status).  Neither handle may have
+ * another call in flight.
+ */
+int ellm_matmul3_attn_run(ellm_matmul3* proj, ellm_attn* attn, size_t position_index,
+                          size_t batch_size, void* stream);
+/* The same with one position per sequence (device uint32, clamped to max_position). */
+int ellm_matmul3_attn_run_ragged(ellm_matmul3* proj, ellm_attn* attn, const uint32_t* positions,
+                                 size_t max_position, size_t batch_size, void* stream);
+int ellm_matmul3_attn_path(const ellm_matmul3* proj, const ellm_attn* attn, size_t batch_size);
+
+/*
  * Output projection with residual: replaces MatMulAdd::new / run
  * (src/compiler/mul/matmul_add.rs:45-75, 128-232; built by Tensor::matmul_add,
  * src/ptensor/tensor.rs:402-437; used by src/qwen3_moe/attention.rs:176-196 on
