@@ -65,6 +65,8 @@ __global__ __launch_bounds__(kDecThreads, PENDING ? 2 : 4) void decode_split_ker
   float m_run, l_run;
   f32x4 acc[8];
   if constexpr (PENDING) {
+    PendingQueries queries;   // requested first: the stream's own loads follow
+    queries.fetch(p.pend, seq, head0, pos, t, heads_here);
     NewRow fresh;
     fresh.present = k_end == len;   // the split that holds the plane's last key
     fresh.store = hgrp == 0;
@@ -80,7 +82,7 @@ __global__ __launch_bounds__(kDecThreads, PENDING ? 2 : 4) void decode_split_ker
     fresh.v_dst = const_cast<uint16_t*>(p.v) + plane + (size_t)pos * p.kv_stride_pos;
     stream_keys<T, true>(p.k + plane, p.v + plane, p.kv_stride_pos, k_begin, k_end, pos, qreg, smem, t,
                          split * 7u + blockIdx.y * 3u + seq * 5u, p.scale_log2, m_run, l_run, acc, &fresh,
-                         [&]() { load_queries_pending<T>(p.pend, seq, head0, pos, t, heads_here, qreg); });
+                         &queries, heads_here);
     // the finished query rows, once per group: by the workgroup that also wrote the new key
     if (fresh.present) store_queries(const_cast<uint16_t*>(p.q) + (size_t)row0 * kHeadDim, t, heads_here, qreg);
   } else {

@@ -108,55 +108,72 @@ __device__ __forceinline__ void load_queries(const uint16_t* q_rows, const Lane&
 
 // ---- fused step: the rows the projection left raw ----------------------------------------
 
-// The eight values at `src`: binary32 partial sums, one or two of them `stride` floats apart.
-__device__ __forceinline__ void sum_parts8(const float* src, uint32_t parts, uint32_t stride, float (&x)[8]) {
-  f32x4 lo = *(const f32x4*)src, hi = *(const f32x4*)(src + 4);
-  if (parts > 1) {   // (uniform)
-    lo += *(const f32x4*)(src + stride);
-    hi += *(const f32x4*)(src + stride + 4);
+// Eight consecutive raw values: binary32 partial sums, one or two of them `stride` floats apart.
+// Fetched first (two or four 16-byte loads, nothing waits) and added up later, so that the
+// caller can put other loads in flight between the two.
+struct Raw8 {
+  f32x4 lo[2], hi[2];
+  __device__ __forceinline__ void fetch(const float* src, uint32_t parts, uint32_t stride) {
+    lo[0] = *(const f32x4*)src;
+    hi[0] = *(const f32x4*)(src + 4);
+    lo[1] = hi[1] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+    if (parts > 1) {   // (uniform)
+      lo[1] = *(const f32x4*)(src + stride);
+      hi[1] = *(const f32x4*)(src + stride + 4);
+    }
   }
+  __device__ __forceinline__ void sum(float (&x)[8]) const {
+    const f32x4 l = lo[0] + lo[1], h = hi[0] + hi[1];
 #pragma unroll
-  for (int e = 0; e < 4; ++e) {
-    x[e] = lo[e];
-    x[4 + e] = hi[e];
+    for (int e = 0; e < 4; ++e) {
+      x[e] = l[e];
+      x[4 + e] = h[e];
+    }
   }
-}
+};
 
 // load_queries() for a fused step: the group's query rows come as raw sums and are normalised
 // and rotated on the way into the operand registers.  Lane (head c, group g) holds the octets
 // 4 s + g of its head; the sum of squares is added up in the order the projection's own
 // finishing step uses (octet, pairs of octets, fours, eights, all sixteen), so the rows come
 // out with the bits that step gives them.
-template <typename T>
-__device__ __forceinline__ void load_queries_pending(const PendingRows& pr, uint32_t seq, uint32_t head0,
-                                                     uint32_t pos, const Lane& t, uint32_t heads_here,
-                                                     u32x4 (&qreg)[4]) {
-  const bool live = (uint32_t)t.c < heads_here;
-  const uint32_t head = head0 + (live ? t.c : 0);
-  const float* src = pr.raw + (size_t)seq * pr.cols + (size_t)head * kHeadDim + 8 * t.g;
-  const uint16_t* rope = (const uint16_t*)pr.rope + (size_t)pos * pr.rope_pos_stride +
-                         (size_t)head * pr.rope_head_stride + 8 * t.g;
-  float x[4][8];
-  u32x4 rr[4];
-  float ss[4];
+struct PendingQueries {
+  Raw8 raw[4];
+  u32x4 rope[4];
+  __device__ __forceinline__ void fetch(const PendingRows& pr, uint32_t seq, uint32_t head0, uint32_t pos,
+                                        const Lane& t, uint32_t heads_here) {
+    const uint32_t head = head0 + ((uint32_t)t.c < heads_here ? t.c : 0);
+    const float* src = pr.raw + (size_t)seq * pr.cols + (size_t)head * kHeadDim + 8 * t.g;
+    const uint16_t* row = (const uint16_t*)pr.rope + (size_t)pos * pr.rope_pos_stride +
+                          (size_t)head * pr.rope_head_stride + 8 * t.g;
 #pragma unroll
-  for (int s = 0; s < 4; ++s) {
-    sum_parts8(src + 32 * s, pr.parts, pr.part_stride, x[s]);
-    rr[s] = load16(rope + 32 * s);
-    ss[s] = squares8(x[s]);
+    for (int s = 0; s < 4; ++s) {
+      raw[s].fetch(src + 32 * s, pr.parts, pr.part_stride);
+      rope[s] = load16(row + 32 * s);
+    }
   }
+  template <typename T>
+  __device__ __forceinline__ void finish(float eps, const Lane& t, uint32_t heads_here, u32x4 (&qreg)[4]) const {
+    float x[4][8], ss[4];
 #pragma unroll
-  for (int s = 0; s < 4; ++s) {
-    ss[s] += xor_shuffle(ss[s], 16);
-    ss[s] += xor_shuffle(ss[s], 32);
-  }
-  const float inv = inverse_rms((ss[0] + ss[1]) + (ss[2] + ss[3]), pr.eps);
+    for (int s = 0; s < 4; ++s) {
+      raw[s].sum(x[s]);
+      ss[s] = squares8(x[s]);
+    }
 #pragma unroll
-  for (int s = 0; s < 4; ++s) {
-    qreg[s] = scale_rotate_pack8<T>(x[s], inv, rr[s]);
-    if (!live) qreg[s] = u32x4{0, 0, 0, 0};
+    for (int s = 0; s < 4; ++s) {
+      ss[s] += xor_shuffle(ss[s], 16);
+      ss[s] += xor_shuffle(ss[s], 32);
+    }
+    const float inv = inverse_rms((ss[0] + ss[1]) + (ss[2] + ss[3]), eps);
+    const bool live = (uint32_t)t.c < heads_here;
+#pragma unroll
+    for (int s = 0; s < 4; ++s) {
+      qreg[s] = scale_rotate_pack8<T>(x[s], inv, rope[s]);
+      if (!live) qreg[s] = u32x4{0, 0, 0, 0};
+    }
   }
-}
+};
 // The finished query rows go back to where the projection alone would have left them.
 __device__ __forceinline__ void store_queries(uint16_t* q_rows, const Lane& t, uint32_t heads_here,
                                               const u32x4 (&qreg)[4]) {
@@ -180,23 +197,31 @@ struct NewRow {
 };
 // Every lane c of each 16-lane group ends up with elements 8 c .. 8 c + 7 of the finished rows
 // (the arithmetic of the projection's own finishing step, lane for lane).
-template <typename T>
-__device__ __forceinline__ void finish_new_row(const NewRow& n, const Lane& t, u32x4& knew, u32x4& vnew) {
-  float kx[8], vx[8];
-  sum_parts8(n.k_raw + 8 * t.c, n.parts, n.part_stride, kx);
-  sum_parts8(n.v_raw + 8 * t.c, n.parts, n.part_stride, vx);
-  const u32x4 rr = load16(n.rope_row + 8 * t.c);
-  float ss = squares8(kx);
-#pragma unroll
-  for (int m = 1; m < 16; m <<= 1) ss += __shfl_xor(ss, m, 16);
-  knew = scale_rotate_pack8<T>(kx, inverse_rms(ss, n.eps), rr);
-  vnew = u32x4{Mfma<T>::pack2(vx[0], vx[1]), Mfma<T>::pack2(vx[2], vx[3]), Mfma<T>::pack2(vx[4], vx[5]),
-               Mfma<T>::pack2(vx[6], vx[7])};
-  if (n.store && t.g == 0) {
-    store16(n.k_dst + 8 * t.c, knew);
-    store16(n.v_dst + 8 * t.c, vnew);
+struct NewRowLoads {
+  Raw8 k, v;
+  u32x4 rope;
+  __device__ __forceinline__ void fetch(const NewRow& n, const Lane& t) {
+    k.fetch(n.k_raw + 8 * t.c, n.parts, n.part_stride);
+    v.fetch(n.v_raw + 8 * t.c, n.parts, n.part_stride);
+    rope = load16(n.rope_row + 8 * t.c);
   }
-}
+  template <typename T>
+  __device__ __forceinline__ void finish(const NewRow& n, const Lane& t, u32x4& knew, u32x4& vnew) const {
+    float kx[8], vx[8];
+    k.sum(kx);
+    v.sum(vx);
+    float ss = squares8(kx);
+#pragma unroll
+    for (int m = 1; m < 16; m <<= 1) ss += __shfl_xor(ss, m, 16);
+    knew = scale_rotate_pack8<T>(kx, inverse_rms(ss, n.eps), rope);
+    vnew = u32x4{Mfma<T>::pack2(vx[0], vx[1]), Mfma<T>::pack2(vx[2], vx[3]), Mfma<T>::pack2(vx[4], vx[5]),
+                 Mfma<T>::pack2(vx[6], vx[7])};
+    if (n.store && t.g == 0) {
+      store16(n.k_dst + 8 * t.c, knew);
+      store16(n.v_dst + 8 * t.c, vnew);
+    }
+  }
+};
 
 // One wave's share of keys [k_begin, k_end) of a plane: the four waves take alternating 16-key
 // chunks, each streams its chunks HBM -> registers (128-bit loads, four full 256-byte rows per
@@ -213,19 +238,16 @@ __device__ __forceinline__ void finish_new_row(const NewRow& n, const Lane& t, u
 // covers [k_begin, pos) and the wave with the fewest chunks finishes the new key / value row
 // from the projection's raw sums (requested before its stream starts), writes it to the cache
 // and takes it as one more chunk of its own.
-// The raw rows are fetched behind the wave's first chunk of keys (`late_queries()` fills qreg
-// from the raw query rows at that point), so that their trip to memory runs beside the first
-// chunk's and not ahead of it.
-struct NoLateQueries {
-  __device__ __forceinline__ void operator()() const {}
-};
-template <typename T, bool PENDING = false, typename LateQueries = NoLateQueries>
+// The raw rows are requested ahead of the wave's first chunk of keys and finished behind its
+// request (`queries` holds the requested raw query rows; qreg is filled here), so that both
+// trips to memory run side by side.
+template <typename T, bool PENDING = false>
 __device__ __forceinline__ void stream_keys(const uint16_t* kplane, const uint16_t* vplane, size_t stride_pos,
                                             uint32_t k_begin, uint32_t k_end, uint32_t pos,
-                                            const u32x4 (&qreg)[4], uint16_t* smem, const Lane& t,
+                                            u32x4 (&qreg)[4], uint16_t* smem, const Lane& t,
                                             uint32_t rot_seed, float scale_log2, float& m_out, float& l_out,
                                             f32x4 (&acc)[8], const NewRow* fresh = nullptr,
-                                            LateQueries late_queries = NoLateQueries()) {
+                                            const PendingQueries* queries = nullptr, uint32_t heads_here = 0) {
   const int g = t.g, c = t.c, wave = t.wave;
   uint16_t* ks = smem + wave * kWaveLdsHalves;  // [16][kKPitch]
   uint16_t* vt = ks + kChunk * kKPitch;         // [128][kVtPitch]
@@ -318,10 +340,14 @@ __device__ __forceinline__ void stream_keys(const uint16_t* kplane, const uint16
     }
   };
 
+  NewRowLoads fresh_loads;
+  if constexpr (PENDING) {
+    if (take_new) fresh_loads.fetch(*fresh, t);
+  }
   if (my_chunks) issue_loads(chunk_at(0));
   if constexpr (PENDING) {
-    late_queries();
-    if (take_new) finish_new_row<T>(*fresh, t, knew, vnew);
+    queries->template finish<T>(fresh->eps, t, heads_here, qreg);
+    if (take_new) fresh_loads.template finish<T>(*fresh, t, knew, vnew);
   }
   for (uint32_t it = 0; it < my_chunks; ++it) {
     const uint32_t chunk = chunk_at(it);

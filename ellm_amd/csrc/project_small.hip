@@ -39,7 +39,9 @@ __device__ __forceinline__ void wait_vm_done() { __builtin_amdgcn_s_waitcnt(0x0F
 
 typedef __attribute__((address_space(3))) u32x4 LdsVec4;
 
-// NTB: 16-token blocks per pass (1 or 2); NB: 16-column MFMA blocks per workgroup (1 or 2).
+// NTB: 16-token blocks per pass (1 or 2); NB: 16-column MFMA blocks per workgroup (1 or 2), or 0: half
+// a block, 8 columns (the other 8 rows of the MFMA's weight operand are zero), for outputs so narrow
+// that 16-column workgroups would leave compute units without one (kModeAdd and kModeRaw only).
 // blockDim.x = 64 * waves, waves = min(16, K / 256).  `passes` passes of 16 NTB token rows
 // each reuse the weight operands, which stay in registers; more than one pass needs
 // waves == K / 256 (one round of K per wave).
@@ -51,7 +53,10 @@ template <typename S, int MODE, int NTB, int NB, bool VIA_LDS>
 __global__ __launch_bounds__((NTB == 2 || NB == 2) ? 512 : 1024) void project_small_kernel(ProjectKernelArgs p, float* ws,
                                                              uint32_t* counters, uint32_t passes) {
   using M = Mfma<S>;
-  constexpr int kColBlocks = NB, kGroupCols = 16 * NB, kGroupsPerHead = kHeadDim / kGroupCols;
+  static_assert(NB != 0 || MODE != kModeQkv, "the heads' finishing step reads whole 16-column blocks");
+  constexpr int kColBlocks = NB ? NB : 1, kGroupCols = NB ? 16 * NB : 8, kGroupsPerHead = kHeadDim / kGroupCols;
+  constexpr bool kHalf = NB == 0;
+  constexpr bool kEarlyResidual = MODE == kModeAdd && kHalf;
   constexpr int kPassRows = 16 * NTB;
   extern __shared__ __attribute__((aligned(16))) float sums[];  // [wave][NTB][16 tokens][kGroupCols]
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, n_waves = blockDim.x >> 6;
@@ -64,7 +69,7 @@ __global__ __launch_bounds__((NTB == 2 || NB == 2) ? 512 : 1024) void project_sm
   const bool finalize = MODE == kModeQkv && ((seg == 1) || (seg == 0 && p.finalize0));
   uint16_t* const dst = (seg == 0) ? p.out0 : (seg == 1 ? p.k_out : p.v_out);
 
-  const uint16_t* wrow = p.w[seg] + ((size_t)hs * kHeadDim + kGroupCols * cg + i16) * K + 8 * q4;
+  const uint16_t* wrow = p.w[seg] + ((size_t)hs * kHeadDim + kGroupCols * cg + (kHalf ? (i16 & 7) : i16)) * K + 8 * q4;
   const size_t wblock = (size_t)16 * K;  // elements between the rows of consecutive column blocks
   const __amdgpu_buffer_rsrc_t x_rsrc =
       __builtin_amdgcn_make_buffer_rsrc((void*)uniform64(p.x), 0, p.rows * K * 2, kBufFlags);
@@ -83,7 +88,8 @@ __global__ __launch_bounds__((NTB == 2 || NB == 2) ? 512 : 1024) void project_sm
     for (int nb = 0; nb < kColBlocks; ++nb)
 #pragma unroll
       for (int s = 0; s < kStepsPerRound; ++s)
-        w[nb][s] = __builtin_nontemporal_load((const u32x4*)(wrow + nb * wblock + k0 + 32 * s));
+        w[nb][s] = (kHalf && i16 >= 8) ? u32x4{0, 0, 0, 0}
+                                       : __builtin_nontemporal_load((const u32x4*)(wrow + nb * wblock + k0 + 32 * s));
   };
 
   constexpr int kQuads = kGroupCols / 4;
@@ -91,12 +97,23 @@ __global__ __launch_bounds__((NTB == 2 || NB == 2) ? 512 : 1024) void project_sm
   // of the pass, four columns of the group) add them up and either finish the row or leave it
   // for the head's last workgroup.
   auto finish_pass = [&](uint32_t pass, f32x4 (&acc)[kColBlocks][NTB]) {
+    // the residual's piece is requested before the sums meet, not behind them (where the
+    // registers are there for it: the 16-wave forms run at 128 a lane)
+    u32x2 rs = {0u, 0u};
+    if constexpr (kEarlyResidual) {
+      if (tid < 16 * kQuads * NTB) {
+        const uint32_t R = pass * kPassRows + tid / kQuads;
+        if (R < p.rows && R % p.batch_pitch < p.batch)
+          rs = *(const u32x2*)(p.residual + (size_t)R * p.ld0 + hs * kHeadDim + kGroupCols * cg + 4 * (tid % kQuads));
+      }
+    }
     // lane (token i16, columns 16 nb + 4 q4 .. + 3)
 #pragma unroll
     for (int nb = 0; nb < kColBlocks; ++nb)
 #pragma unroll
       for (int tb = 0; tb < NTB; ++tb)
-        *(f32x4*)(sums + ((wave * NTB + tb) * 16 + i16) * kGroupCols + 16 * nb + 4 * q4) = acc[nb][tb];
+        if (!kHalf || q4 < 2)
+          *(f32x4*)(sums + ((wave * NTB + tb) * 16 + i16) * kGroupCols + 16 * nb + 4 * q4) = acc[nb][tb];
     __syncthreads();
     if (tid < 16 * kQuads * NTB) {
       const uint32_t R = pass * kPassRows + tid / kQuads, c4 = tid % kQuads;
@@ -123,7 +140,7 @@ __global__ __launch_bounds__((NTB == 2 || NB == 2) ? 512 : 1024) void project_sm
             off = kv_row_offset(p, b, hs, pos) + kGroupCols * cg + 4 * c4;
           }
           if (MODE == kModeAdd) {
-            const u32x2 rs = *(const u32x2*)(p.residual + off);
+            if constexpr (!kEarlyResidual) rs = *(const u32x2*)(p.residual + off);
             v[0] += M::to_float((uint16_t)(rs[0] & 0xffffu));
             v[1] += M::to_float((uint16_t)(rs[0] >> 16));
             v[2] += M::to_float((uint16_t)(rs[1] & 0xffffu));
@@ -142,7 +159,7 @@ __global__ __launch_bounds__((NTB == 2 || NB == 2) ? 512 : 1024) void project_sm
       const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) float*)sums;
       const uint8_t* wg_rows = (const uint8_t*)(p.w[seg] + ((size_t)hs * kHeadDim + kGroupCols * cg) * K);
       const uint32_t row_bytes = 2 * K, pitch = row_bytes + 16;  // + 16: the 16 rows of an operand read tile the banks
-      constexpr int kPieces = 8 * NB;                            // 1 KB pieces per wave
+      constexpr int kPieces = kGroupCols / 2;                    // 1 KB pieces per wave (waves x 256 = K)
       u32x4 stg[kPieces];
 #pragma unroll
       for (int u = 0; u < kPieces; ++u)
@@ -160,14 +177,16 @@ __global__ __launch_bounds__((NTB == 2 || NB == 2) ? 512 : 1024) void project_sm
       for (int nb = 0; nb < kColBlocks; ++nb)
 #pragma unroll
         for (int s = 0; s < kStepsPerRound; ++s)
-          wreg[nb][s] = *(const LdsVec4*)(lds0 + (16 * nb + i16) * pitch + (k_first + 32 * s + 8 * q4) * 2);
+          wreg[nb][s] = (kHalf && i16 >= 8)
+                            ? u32x4{0, 0, 0, 0}
+                            : (u32x4)*(const LdsVec4*)(lds0 + (16 * nb + i16) * pitch + (k_first + 32 * s + 8 * q4) * 2);
       __syncthreads();  // the sums reuse the rows' LDS
     }
     // the weight operands stay in registers; the token rows of the next pass are requested
     // before those of this one are used, where the registers are there for them (a second set
     // of token rows in the widest forms would not fit, and a kernel that spills, by however
     // little, pays several microseconds a launch for its scratch memory to be set up)
-    constexpr bool kAhead = NTB == 1 && !(MODE == kModeQkv && NB == 1);
+    constexpr bool kAhead = NTB == 1 && !(MODE == kModeQkv && NB == 1) && !kEarlyResidual;
     for (uint32_t pass = 0; pass < passes; ++pass) {
       u32x4 xnext[kAhead ? NTB : 1][kAhead ? kStepsPerRound : 1];
       const bool more = pass + 1 < passes;  // (uniform)
@@ -276,10 +295,11 @@ constexpr uint32_t kLdsBudget = 150 * 1024;
 template <typename S, int MODE, int NTB, int NB>
 hipError_t launch_one(const ProjectKernelArgs& p, float* ws, uint32_t* counters, uint32_t heads, uint32_t waves,
                       hipStream_t stream) {
-  const dim3 grid(heads * (kHeadDim / (16 * NB))), block(64 * waves);
+  constexpr uint32_t kCols = NB ? 16 * NB : 8;
+  const dim3 grid(heads * (kHeadDim / kCols)), block(64 * waves);
   const uint32_t passes = (p.rows + 16 * NTB - 1) / (16 * NTB);
-  const uint32_t sums_bytes = waves * NTB * 64 * 16 * NB;
-  const uint32_t rows_bytes = 16 * NB * (2 * p.K + 16);
+  const uint32_t sums_bytes = waves * NTB * 64 * kCols;
+  const uint32_t rows_bytes = kCols * (2 * p.K + 16);
   if (waves * kRoundK == p.K && rows_bytes <= kLdsBudget) {
     const uint32_t lds = rows_bytes > sums_bytes ? rows_bytes : sums_bytes;
     hipLaunchKernelGGL((project_small_kernel<S, MODE, NTB, NB, true>), grid, block, lds, stream, p, ws, counters,
@@ -302,6 +322,13 @@ hipError_t launch_blocks(const ProjectKernelArgs& p, float* ws, uint32_t* counte
                     (waves * kRoundK != p.K || 32 * (2 * p.K + 16) <= kLdsBudget);
   // two token blocks a pass want 512 threads for the finishing step and 256 registers a lane
   const bool two_blocks = p.rows > 16 && waves == 8;
+  // 16-column workgroups fewer than three quarters of a 256-unit part: 8 columns each (the output
+  // projection 4096 -> 2048: 256 workgroups instead of 128; 7.6 -> us at one row)
+  if constexpr (MODE != kModeQkv) {
+    if (heads * (kHeadDim / 16) <= 192 && waves * kRoundK == p.K)
+      return two_blocks ? launch_one<S, MODE, 2, 0>(p, ws, counters, heads, waves, stream)
+                        : launch_one<S, MODE, 1, 0>(p, ws, counters, heads, waves, stream);
+  }
   if (!two_blocks)
     return wide ? launch_one<S, MODE, 1, 2>(p, ws, counters, heads, waves, stream)
                 : launch_one<S, MODE, 1, 1>(p, ws, counters, heads, waves, stream);
@@ -322,6 +349,14 @@ static hipError_t prepare_mode() {
   for (const void* k : kernels) {
     const hipError_t e = hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBudget);
     if (e != hipSuccess) return e;
+  }
+  if constexpr (MODE != kModeQkv) {
+    const void* narrow[] = {(const void*)project_small_kernel<S, MODE, 1, 0, true>,
+                            (const void*)project_small_kernel<S, MODE, 2, 0, true>};
+    for (const void* k : narrow) {
+      const hipError_t e = hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBudget);
+      if (e != hipSuccess) return e;
+    }
   }
   return hipSuccess;
 }
