@@ -97,10 +97,14 @@ int ellm::validate_attn_desc(const ellm_attn_desc* d) {
                 d->kv_strides[2]);
   if (d->sequence_capacity == 0 || d->sequence_capacity > 0x7fffffffu)
     return fail(ELLM_ERR_INVALID_ARGUMENT, "sequence_capacity %zu out of range", d->sequence_capacity);
-  if (d->sequence_capacity * d->kv_strides[2] > 0x7fffffffu)
+  // offsets inside a plane are 64-bit; a tile of 64 rows is addressed with 32-bit byte offsets
+  if (d->kv_strides[2] > ((size_t)1 << 24))
     return fail(ELLM_ERR_UNSUPPORTED,
-                "a K/V plane spans %zu elements; offsets inside a plane are 32-bit (max 2^31 - 1)",
-                d->sequence_capacity * d->kv_strides[2]);
+                "kv_strides[2] = %zu elements: rows of a K/V plane may be at most 2^24 elements apart",
+                d->kv_strides[2]);
+  size_t span = 0;
+  if (__builtin_mul_overflow(d->sequence_capacity, d->kv_strides[2], &span) || span > ((size_t)1 << 46))
+    return fail(ELLM_ERR_UNSUPPORTED, "a K/V plane spans more than 2^46 elements");
   if (d->max_position_interval == 0 || d->max_position_interval > d->sequence_capacity)
     return fail(ELLM_ERR_INVALID_ARGUMENT,
                 "max_position_interval %zu must be in 1..sequence_capacity", d->max_position_interval);

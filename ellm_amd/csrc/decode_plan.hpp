@@ -39,19 +39,28 @@ inline DecodePlan decode_plan(uint32_t max_len, uint32_t batch, uint32_t n_kv_he
   // on 2 x 256): the plan with the shorter estimated time is taken, time = keys per split x
   // workgroups on the busiest unit (x 1.03 when units are shared).  Splits are rounded down in
   // number: a few workgroups beyond a whole round make some units host one more, and those
-  // finish that much later (20 x 8192: 67 us with 560 workgroups, 57 us with 480).  Never
-  // shorter than four 64-key steps.
+  // finish that much later (20 x 8192: 67 us with 560 workgroups, 57 us with 480).
   const uint64_t planes = (uint64_t)batch * n_kv_heads;
   // both merge levels fold at most 16 partials: at most 16 * 16 splits per plane
   const uint32_t floor_len =
       ((max_len + kPlanMergeFan * kPlanMergeFan - 1) / (kPlanMergeFan * kPlanMergeFan) + kDecodeStepKeys - 1) /
       kDecodeStepKeys * kDecodeStepKeys;
+  // Never shorter than four 64-key steps, except where even such splits leave at least half of
+  // the units without a workgroup (one sequence of a few hundred keys, a handful of a thousand):
+  // there a wave's chunks, fetched one after the other, are a chain of trips to memory, and one
+  // 64-key step per workgroup with one fold of at most 16 partials is the shorter chain
+  // (1 x 512 keys: 9.4 -> 6.7 us, 4 x 1024: 10.0 -> 8.5, 1 x 2048: 8.4; folds of at most 8 or 4
+  // partials, i.e. longer splits, measured the same or slower).
+  const bool tiny = planes * ((max_len + 4 * kDecodeStepKeys - 1) / (4 * kDecodeStepKeys)) * 2 <= n_cu;
+  const uint32_t one_fold_len = ((max_len + kPlanMergeFan - 1) / kPlanMergeFan + kDecodeStepKeys - 1) /
+                                kDecodeStepKeys * kDecodeStepKeys;
+  const uint32_t min_len = tiny ? one_fold_len : 4 * kDecodeStepKeys;
   auto plan_for = [&](uint32_t per_cu, uint64_t* cost) {
     const uint32_t target = n_cu * per_cu;
     const uint32_t want = target / planes > 0 ? (uint32_t)(target / planes) : 1;
     uint32_t split_len = (max_len + want - 1) / want;
     split_len = (split_len + kDecodeStepKeys - 1) / kDecodeStepKeys * kDecodeStepKeys;
-    if (split_len < 4 * kDecodeStepKeys) split_len = 4 * kDecodeStepKeys;
+    if (split_len < min_len) split_len = min_len;
     if (split_len < floor_len) split_len = floor_len;
     DecodePlan plan;
     plan.split_len = split_len;

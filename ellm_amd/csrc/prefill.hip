@@ -81,6 +81,21 @@ __device__ __forceinline__ uint64_t uniform64(const void* p) {  // the compiler 
   const uint32_t hi = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)((uint64_t)p >> 32));
   return ((uint64_t)hi << 32) | (uint64_t)lo;
 }
+// Bytes a buffer descriptor may cover from byte `off` of a plane whose last visible byte ends at
+// `valid`: what is left, capped at the 32 bits the descriptor's size field has (a tile or chunk
+// reaches at most 64 rows beyond `off`, far less than that).  Both offsets are 64-bit: a plane
+// of the reference's own [position][sequence][kv_head][128] state spans more than 2^32 bytes at
+// 33 sequences x 131072 positions.  Scalar arithmetic (the arguments are wave-uniform).
+__device__ __forceinline__ uint32_t bytes_left(uint64_t valid, uint64_t off) {
+  const uint64_t left = valid > off ? valid - off : 0;
+  const uint32_t capped = left > 0xffffffffull ? 0xffffffffu : (uint32_t)left;
+  return (uint32_t)__builtin_amdgcn_readfirstlane((int)capped);
+}
+__device__ __forceinline__ uint64_t uniform_u64(uint64_t v) {
+  const uint32_t lo = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)v);
+  const uint32_t hi = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(v >> 32));
+  return ((uint64_t)hi << 32) | (uint64_t)lo;
+}
 typedef __attribute__((address_space(3))) uint16_t LdsHalf;
 typedef __attribute__((address_space(3))) u32x4 LdsU32x4;
 typedef __attribute__((address_space(3))) u32x2 LdsU32x2;
@@ -173,8 +188,8 @@ __global__ __launch_bounds__(kPpThreads, 2) void prefill_pingpong_kernel(Prefill
   const uint32_t plane_lo = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(uint64_t)plane);
   const uint32_t plane_hi = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)((uint64_t)plane >> 32));
   const uint64_t plane_u = ((uint64_t)plane_hi << 32) | (uint64_t)plane_lo;
-  const uint32_t tile_bytes = kBK * stride_pos * 2;
-  const uint32_t valid_bytes = (kmax * stride_pos + kHeadDim) * 2;  // API bound: a plane spans < 2^32 bytes
+  const uint32_t tile_bytes = kBK * stride_pos * 2;   // (API bound: 64 rows span < 2^32 bytes)
+  const uint64_t valid_bytes = uniform_u64(((uint64_t)kmax * stride_pos + kHeadDim) * 2);
   uint32_t piece_off[4];
 #pragma unroll
   for (int i = 0; i < 4; ++i) piece_off[i] = ((ld_r + 16 * i) * stride_pos + 8 * ld_c) * 2;
@@ -190,9 +205,8 @@ __global__ __launch_bounds__(kPpThreads, 2) void prefill_pingpong_kernel(Prefill
   const uint32_t vs_store = lds0 + 2 * (2 * kKsHalves + ld_r * kVsPitch + 8 * ld_c);
   u32x4 stg[4];
   auto load_piece = [&](uint32_t kt, int i) {  // kt (relative to kt0) must be wave-uniform to the compiler
-    const uint32_t off = (kt0 + kt) * tile_bytes;
-    // (written as a scalar min and subtract: a saturating subtract would be a vector instruction)
-    const uint32_t left = valid_bytes - __builtin_amdgcn_readfirstlane(min(valid_bytes, off));
+    const uint64_t off = (uint64_t)(kt0 + kt) * tile_bytes;
+    const uint32_t left = bytes_left(valid_bytes, off);
     const __amdgpu_buffer_rsrc_t rsrc =
         __builtin_amdgcn_make_buffer_rsrc((void*)(plane_u + off), 0, left, kBufferFlags);
     stg[i] = __builtin_amdgcn_raw_buffer_load_b128(rsrc, piece_off[i], 0, 0);
@@ -522,14 +536,14 @@ __global__ __launch_bounds__(WAVES * kWave, WAVES == 4 ? 2 : 1) void chunk_strea
   const int ld_c = tid & 15, ld_r = (tid >> 4) & (kPieceRows - 1);
   const uint64_t kplane_u = uniform64(kplane), vplane_u = uniform64(vplane);
   const uint32_t chunk_bytes = kCK * stride_pos * 2;
-  const uint32_t valid_bytes = (kmax * stride_pos + kHeadDim) * 2;
+  const uint64_t valid_bytes = uniform_u64(((uint64_t)kmax * stride_pos + kHeadDim) * 2);
   const uint32_t piece_off0 = (ld_r * stride_pos + 8 * ld_c) * 2;
   const uint32_t piece_step = kPieceRows * stride_pos * 2;
   u32x4 stg[DEPTH][2 * kPieces];
   auto load_chunk = [&](uint32_t ck, u32x4 (&st)[2 * kPieces]) {  // ck relative to this split's first chunk; wave-uniform
     if (!stager) return;
-    const uint32_t off = k0 * stride_pos * 2 + ck * chunk_bytes;
-    const uint32_t left = valid_bytes - __builtin_amdgcn_readfirstlane(min(valid_bytes, off));
+    const uint64_t off = (uint64_t)k0 * stride_pos * 2 + (uint64_t)ck * chunk_bytes;
+    const uint32_t left = bytes_left(valid_bytes, off);
     const __amdgpu_buffer_rsrc_t kr = __builtin_amdgcn_make_buffer_rsrc((void*)(kplane_u + off), 0, left, kBufferFlags);
     const __amdgpu_buffer_rsrc_t vr = __builtin_amdgcn_make_buffer_rsrc((void*)(vplane_u + off), 0, left, kBufferFlags);
 #pragma unroll

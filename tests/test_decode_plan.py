@@ -53,11 +53,14 @@ def test_plans_are_well_formed_and_fit_the_workspace(rows):
     assert len(rows) > 50000
     for n_cu, hq, hkv, cap, batch, length, split_len, n_split, fits in rows:
         case = (n_cu, hq, hkv, cap, batch, length, split_len, n_split)
-        assert split_len % 64 == 0 and split_len >= 256, case
+        planes = batch * hkv
+        tiny = planes * -(-length // 256) * 2 <= n_cu      # even 256-key splits would leave half of the units idle
+        assert split_len % 64 == 0 and split_len >= (64 if tiny else 256), case
+        if tiny and split_len < 256:
+            assert n_split <= 16, case                                               # one fold
         assert n_split == -(-length // split_len) and 1 <= n_split <= 256, case     # two fold levels of 16
         assert (n_split - 1) * split_len < length, case                             # no split without keys
         assert fits == 1, case                       # the handle's workspace holds every plan it can be asked for
-        planes = batch * hkv
         if n_split > 1 and split_len > 256 and split_len * 256 > length + 64 * 256:
             # (not at one of the two floors) never more than two workgroups per compute unit
             assert planes * n_split <= 2 * n_cu, case
@@ -72,7 +75,9 @@ def test_one_workgroup_per_unit_where_the_planes_divide_the_units(rows):
     assert by[(256, 32, 4, 20, 8192)] == (2752, 3)         # 80 planes x 3 = 240 on 256 beat 480 on 2 x 256
     assert by[(256, 32, 4, 12, 8192)] == (1664, 5)         # 48 planes x 5 = 240
     assert by[(256, 32, 4, 98, 8192)] == (8192, 1)         # more planes than units: no split
-    assert by[(256, 32, 4, 1, 255)] == (256, 1)
+    assert by[(256, 32, 4, 1, 255)] == (64, 4)            # a tiny call: one 64-key step per workgroup
+    assert by[(256, 32, 4, 4, 1000)] == (64, 16)          # 16 planes x 16 = 256 workgroups, one fold
+    assert by[(256, 32, 4, 16, 1000)] == (256, 4)         # 64 planes: not tiny any more
 
 
 STATIC_PROBE = r"""
