@@ -398,3 +398,131 @@ def test_config4_one_layer_at_its_real_shape_ragged_cache():
     for op in (proj_pf, proj_dec, att_pf, att_dec):
         op.close()
     cache.close()
+
+
+def test_config4_all_48_layers_first_middle_and_last_checked():
+    """The mixed step of configs[4] as bench.py runs it (`mixed48`): 48 layers, each with its own
+    random-init projection weights and its own K/V in one cache object with per-sequence capacities
+    (223.6 GB resident), a 16384-token prefill of sequence 0 and one new token of 32 sequences with
+    cache lengths U{1024..131072} (seed 7), projections writing K/V into the caches.  All 192 launches
+    run in the benchmark's order on one stream; the outputs of layers 0, 23 and 47 are kept as they
+    leave their layer and checked against the oracle on what the device holds for that layer: sampled
+    prefill rows, every head of four of the 32 single-token sequences, and the projection's own rows
+    of those within one unit in the last place."""
+    import torch
+
+    import ellm_amd
+
+    dtype, hq, hkv, hidden, s_pf, n_dec, layers = orc.F16, 32, 4, 2048, 16384, 32, 48
+    td = torch.float16
+    sc = 1.0 / np.sqrt(D)
+    lengths = np.random.default_rng(7).integers(1024, 131072 + 1, size=n_dec)
+    caps = [s_pf] + [int((n + 63) // 64 * 64) for n in lengths]
+    need = 2 * layers * hkv * sum(caps) * D * 2
+    torch.cuda.empty_cache()
+    free, _ = torch.cuda.mem_get_info()
+    if free < need + 8 * 2 ** 30:
+        pytest.skip(f"needs {need / 2 ** 30:.0f} GiB of device memory for the 48 caches, {free / 2 ** 30:.0f} free")
+    cache = ellm_amd.KVCache.ragged(layers, caps, hkv, ellm_amd.DTYPE_F16)
+    total = sum(caps)
+    offs = np.concatenate([[0], np.cumsum(caps)[:-1]])
+    jj = np.arange(D // 2, dtype=np.float64)
+    ang = np.arange(max(caps), dtype=np.float64)[:, None] * (1.0e6 ** (-2.0 * jj / D))[None, :]
+    rope_h = np.empty((max(caps), D), dtype=np.float32)
+    rope_h[:, 0::2], rope_h[:, 1::2] = np.cos(ang), np.sin(ang)
+    rope_h = orc.to_storage(rope_h, dtype)
+    rope = to_dev(rope_h, dtype)
+    x_pf = _device_normal((s_pf, 1, hidden), 310, dtype)
+    x_dec = _device_normal((1, n_dec, hidden), 300, dtype)
+    q_pf = torch.zeros((s_pf, 1, hq, D), dtype=td, device="cuda")
+    q_dec = torch.zeros((1, n_dec, hq, D), dtype=td, device="cuda")
+    out_pf, out_dec = torch.zeros_like(q_pf), torch.zeros_like(q_dec)
+    lse_pf = torch.zeros((s_pf, 1, hq), dtype=torch.float32, device="cuda")
+    lse_dec = torch.zeros((1, n_dec, hq), dtype=torch.float32, device="cuda")
+    pos = (lengths - 1).astype(np.int32)
+    dpos = torch.from_numpy(pos).cuda()
+    max_pos = int(pos.max())
+    ops, weights = [], []
+    for layer in range(layers):
+        kt, vt = cache.layer_flat_tensors(layer, td)
+        kt.normal_()              # the sequences' caches already hold their tokens
+        vt.normal_()
+        v0, v1 = cache.layer_ragged(layer, 0), cache.layer_ragged(layer, 1)
+        w = [(_device_normal((h * D, hidden), 700 + 3 * layer + i, dtype).float() * hidden ** -0.5).to(td)
+             for i, h in enumerate((hq, hkv, hkv))]
+        weights.append(w)
+        ops.append((ellm_amd.MatMul3(x_pf, w[0], q_pf, w[1], kt, w[2], vt, rope, D, 1, hq, hkv, v0.strides, 0, seq_table=v0),
+                    ellm_amd.Attention(q_pf, kt, vt, out_pf, 1, hq, hkv, D, v0.strides, sc, lse=lse_pf,
+                                       max_position_interval=s_pf, seq_table=v0),
+                    ellm_amd.MatMul3(x_dec, w[0], q_dec, w[1], kt, w[2], vt, rope, D, n_dec, hq, hkv, v1.strides, 0,
+                                     seq_table=v1),
+                    ellm_amd.Attention(q_dec, kt, vt, out_dec, n_dec, hq, hkv, D, v1.strides, sc, lse=lse_dec,
+                                       max_position_interval=1, seq_table=v1)))
+    checked = (0, layers // 2 - 1, layers - 1)
+    kept = {}
+    torch.cuda.synchronize()
+    for layer, (qkv_pre, att_pre, qkv_dec, att_dec) in enumerate(ops):      # the benchmark's order
+        qkv_pre.run(0, s_pf, 1)
+        att_pre.run(0, s_pf, 1)
+        qkv_dec.run_ragged(dpos, max_pos, n_dec)
+        att_dec.run_ragged(dpos, max_pos, n_dec)
+        if layer in checked:      # the activations are layer-shared scratch: keep this layer's
+            kept[layer] = tuple(t.clone() for t in (q_pf, out_pf, lse_pf, q_dec, out_dec, lse_dec))
+    torch.cuda.synchronize()
+
+    rng = np.random.default_rng(241)
+    xh_dec = _host(x_dec, dtype)
+    xh_pf = _host(x_pf, dtype)
+    picks = sorted({int(np.argmin(lengths)), int(np.argmax(lengths)), 5, 20})
+    all_heads = np.array([[0, 0, h] for h in range(hq)], dtype=np.uint32)
+
+    def ulps(got, want):
+        got, want = orc.from_storage(got, dtype), orc.from_storage(want, dtype)
+        return float((np.abs(got - want) / 2.0 ** (np.floor(np.log2(np.maximum(np.abs(want), 0.125))) - 10)).max())
+
+    for layer in checked:
+        kt, vt = cache.layer_flat_tensors(layer, td)
+        wh = [_host(x, dtype) for x in weights[layer]]
+        g_q_pf, g_out_pf, g_lse_pf, g_q_dec, g_out_dec, g_lse_dec = kept[layer]
+        # prefill side: the plane of sequence 0 and sampled (token, head) rows
+        k0, v0h = _host(kt[:, :s_pf], dtype), _host(vt[:, :s_pf], dtype)          # [hkv, 16384, 128]
+        ref = orc.Operator(_host(g_q_pf, dtype), k0, v0h, np.zeros((1,), np.float16), None, 1, hq, hkv, D,
+                           [0, s_pf * D, D, 1], sc, dtype)
+        toks = np.concatenate([[0, 63, s_pf - 1], rng.integers(0, s_pf, 9)])
+        rows = np.stack([toks, np.zeros_like(toks), rng.integers(0, hq, toks.size)], 1).astype(np.uint32)
+        _check_rows(ref, rows, 0, g_out_pf, g_lse_pf, dtype)
+        # ... and a window of its projection
+        t0 = int(rng.integers(0, s_pf - 16))
+        oq = np.zeros((16, 1, hq, D), dtype=np.float16)
+        ok = np.zeros((1, hkv, s_pf, D), dtype=np.float16)
+        ov = np.zeros_like(ok)
+        assert orc.matmul3(np.ascontiguousarray(xh_pf[t0:t0 + 16]), wh[0], wh[1], wh[2], oq, ok, ov, rope_h,
+                           [hkv * s_pf * D, s_pf * D, D, 1], s_pf, t0, 16, dtype) == 0
+        worst = max(ulps(_host(g_q_pf, dtype)[t0:t0 + 16], oq), ulps(k0[:, t0:t0 + 16], ok[0, :, t0:t0 + 16]),
+                    ulps(v0h[:, t0:t0 + 16], ov[0, :, t0:t0 + 16]))
+        assert worst <= 1.0, (layer, "prefill projection", worst)
+        # single-token side: every head of four sequences, and their projection rows
+        got_dec, got_lse = to_host(g_out_dec, dtype), g_lse_dec.cpu().numpy()
+        qh_dec = _host(g_q_dec, dtype)
+        for i in picks:
+            o, cap_i = int(offs[1 + i]), caps[1 + i]
+            ki, vi = _host(kt[:, o:o + cap_i], dtype), _host(vt[:, o:o + cap_i], dtype)
+            ref = orc.Operator(np.ascontiguousarray(qh_dec[:, i:i + 1]), ki, vi, np.zeros((1,), np.float16), None, 1,
+                               hq, hkv, D, [0, cap_i * D, D, 1], sc, dtype)
+            want, want_lse, _ = ref.run_rows(int(pos[i]), all_heads, 8)
+            res = compare(got_dec[0, i], orc.from_storage(want, dtype), dtype)
+            assert res["ok"], (layer, i, int(lengths[i]), res)
+            assert np.abs(got_lse[0, i] - want_lse).max() <= LSE_TOL, (layer, i)
+            oq = np.zeros((1, 1, hq, D), dtype=np.float16)
+            ok = np.zeros((1, hkv, cap_i, D), dtype=np.float16)
+            ov = np.zeros_like(ok)
+            assert orc.matmul3(np.ascontiguousarray(xh_dec[:, i:i + 1]), wh[0], wh[1], wh[2], oq, ok, ov, rope_h,
+                               [hkv * cap_i * D, cap_i * D, D, 1], cap_i, int(pos[i]), 1, dtype) == 0
+            worst = max(ulps(qh_dec[:, i:i + 1], oq), ulps(ki[:, pos[i]], ok[0, :, pos[i]]),
+                        ulps(vi[:, pos[i]], ov[0, :, pos[i]]))
+            assert worst <= 1.0, (layer, i, "single-token projection", worst)
+        print(f"layer {layer}: prefill rows, 4 x 32 single-token rows and their projection rows match the oracle", flush=True)
+    for group in ops:
+        for op in group:
+            op.close()
+    cache.close()
