@@ -17,28 +17,35 @@ namespace {
 
 constexpr int kMidKc = 64;                        // K elements per chunk: one 128-byte line per row
 constexpr int kMidRowPitch = kMidKc * 2;          // unpadded; pieces permuted as in project.hip
-constexpr int kMidThreads = 256;
-// MB = 32-token blocks per wave: the tile is 128 MB tokens x one head.
-template <int MB>
+// MB = 32-token blocks per wave, WAVES = 4 or 8 waves: the tile is 32 MB WAVES tokens x one head.
+// Forms in use: 4 waves x 1 block (128 tokens) and 8 waves x 1 block (256 tokens, two waves per SIMD
+// with 180 registers each).  4 waves x 2 blocks (256 tokens, one wave per SIMD with 330 registers: the
+// same MFMAs per chunk, 40 % fewer operand reads, but nothing to issue from while the wave waits for
+// its operands or at the chunk's barrier) still compiles and measured 7 % slower.
+template <int MB, int WAVES>
 struct MidShape {
-  static constexpr int kTokens = 128 * MB;
+  static_assert((WAVES == 4 && (MB == 1 || MB == 2)) || (WAVES == 8 && MB == 1), "forms of the tile");
+  static constexpr int kThreads = 64 * WAVES;
+  static constexpr int kTokens = 32 * MB * WAVES;
   static constexpr int kStageBytes = (kTokens + kHeadDim) * kMidRowPitch;  // X rows then W rows: 32 or 48 KB
-  static constexpr int kStages = MB == 1 ? 4 : 3;   // chunk c in stage c % kStages
+  static constexpr int kStages = kTokens == 128 ? 4 : 3;   // chunk c in stage c % kStages
   static constexpr int kLdsBytes = kStages * kStageBytes;
-  static constexpr int kLoads = 4 * MB + 4;         // 1 KB wave loads per chunk and wave
+  static constexpr int kRowsPerLoad = 8 * WAVES;    // rows one load of every wave moves (1 KB = 8 rows a wave)
+  static constexpr int kXLoads = kTokens / kRowsPerLoad, kWLoads = kHeadDim / kRowsPerLoad;
+  static constexpr int kLoads = kXLoads + kWLoads;  // 1 KB wave loads per chunk and wave
   static constexpr int kAhead = kStages - 1;        // chunks requested ahead of the one being multiplied
   // loads a wave still has outstanding when its pieces of the next chunk must have landed: the
   // chunks requested after that one (the literal in the kernel's s_waitcnt)
   static constexpr int kMayBePending = (kAhead - 1) * kLoads;
-  static_assert(kMayBePending == (MB == 1 ? 16 : 12), "s_waitcnt vmcnt literals in project_mid_kernel");
-  static_assert(4 * kEpWaveBytes <= kLdsBytes, "the epilogue reuses the stages");
+  static_assert(kMayBePending == (WAVES == 8 ? 6 : (MB == 1 ? 16 : 12)), "s_waitcnt vmcnt literals in project_mid_kernel");
+  static_assert(WAVES * kEpWaveBytes <= kLdsBytes, "the epilogue reuses the stages");
   static_assert(kLdsBytes <= 160 * 1024, "LDS of a compute unit");
 };
 
-template <typename S, int MODE, int MB>
-__global__ __launch_bounds__(kMidThreads) void project_mid_kernel(ProjectKernelArgs p) {
+template <typename S, int MODE, int MB, int WAVES>
+__global__ __launch_bounds__(64 * WAVES) void project_mid_kernel(ProjectKernelArgs p) {
   using M = Mfma<S>;
-  using Shape = MidShape<MB>;
+  using Shape = MidShape<MB, WAVES>;
   constexpr int kStageBytes = Shape::kStageBytes, kStages = Shape::kStages, kLoads = Shape::kLoads;
   extern __shared__ __attribute__((aligned(16))) uint8_t mid_smem[];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -75,15 +82,16 @@ __global__ __launch_bounds__(kMidThreads) void project_mid_kernel(ProjectKernelA
   const u32x4 w_rsrc = make_rsrc(uniform64(wbase) + (uint64_t)hs * kHeadDim * K * 2, kHeadDim * K * 2);
 
   // staging: lane l of a wave instruction delivers its 16 bytes to M0 + 16 l, so a wave fills
-  // 1 KB = eight whole rows of a stage per instruction; thread -> row tid / 8 (+ 32 i: the
-  // X rows for i < 4 MB, then the 128 W rows), LDS piece tid % 8.  The permutation of the pieces
+  // 1 KB = eight whole rows of a stage per instruction; thread -> row tid / 8 (+ 8 WAVES i: the
+  // X rows for i < kXLoads, then the 128 W rows), LDS piece tid % 8.  The permutation of the pieces
   // within a row (piece p of row r sits at p ^ ((r >> 1) & 7)) is applied on the memory side:
   // which piece of the line a lane asks for.  Eight lanes still fetch one whole 128-byte line.
   // Rows past the end of the activations read zeros.
   const uint32_t st_row = tid >> 3, st_piece = (tid & 7) ^ ((tid >> 4) & 7);
-  uint32_t src_off[4 * MB];
+  constexpr int kXLoads = Shape::kXLoads;
+  uint32_t src_off[kXLoads];
 #pragma unroll
-  for (int i = 0; i < 4 * MB; ++i) src_off[i] = (st_row + 32 * i) * K * 2 + st_piece * 16;
+  for (int i = 0; i < kXLoads; ++i) src_off[i] = (st_row + Shape::kRowsPerLoad * i) * K * 2 + st_piece * 16;
   const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t*)mid_smem;
   const uint32_t st_wave = lds0 + (uint32_t)__builtin_amdgcn_readfirstlane(wave) * 1024;
   // Written as asm: the compiler's own form of this load makes it wait for every outstanding
@@ -98,9 +106,9 @@ __global__ __launch_bounds__(kMidThreads) void project_mid_kernel(ProjectKernelA
   // access, zeros into a stage nobody reads, and every iteration issues the same eight loads.
   const u32x4 none_rsrc = make_rsrc(uniform64(p.x), 0);
   auto load_piece = [&](uint32_t chunk, int i) {
-    const uint32_t to = st_wave + (chunk % kStages) * kStageBytes + 4096 * i;
+    const uint32_t to = st_wave + (chunk % kStages) * kStageBytes + 1024 * WAVES * i;
     const bool real = chunk < n_chunks;
-    load_lds(real ? (i < 4 * MB ? x_rsrc : w_rsrc) : none_rsrc, src_off[i < 4 * MB ? i : i - 4 * MB],
+    load_lds(real ? (i < kXLoads ? x_rsrc : w_rsrc) : none_rsrc, src_off[i < kXLoads ? i : i - kXLoads],
              chunk * (kMidKc * 2), to);
   };
 
@@ -136,8 +144,10 @@ __global__ __launch_bounds__(kMidThreads) void project_mid_kernel(ProjectKernelA
   // (requested behind the first chunks, used after the loop: destinations, positions and the
   // first rows of the rotary table or the residual)
   const HeadRows<MB> head = prepare_head<S, MODE, MB>(p, tn, row0 + 32 * MB * wave, lane);
-  if constexpr (MB == 1)
-    asm volatile("s_waitcnt vmcnt(16)" ::: "memory");   // Shape::kMayBePending
+  if constexpr (WAVES == 8)
+    asm volatile("s_waitcnt vmcnt(6)" ::: "memory");    // Shape::kMayBePending
+  else if constexpr (MB == 1)
+    asm volatile("s_waitcnt vmcnt(16)" ::: "memory");
   else
     asm volatile("s_waitcnt vmcnt(12)" ::: "memory");
   __syncthreads();
@@ -178,7 +188,9 @@ __global__ __launch_bounds__(kMidThreads) void project_mid_kernel(ProjectKernelA
       if constexpr (n == 3 * kPerStep - 1) {
         // this wave's pieces of chunk c + 1 are in LDS, and its reads of this chunk's stage
         // have returned
-        if constexpr (MB == 1)
+        if constexpr (WAVES == 8)
+          asm volatile("s_waitcnt vmcnt(6) lgkmcnt(0)" ::: "memory");
+        else if constexpr (MB == 1)
           asm volatile("s_waitcnt vmcnt(16) lgkmcnt(0)" ::: "memory");
         else
           asm volatile("s_waitcnt vmcnt(12) lgkmcnt(0)" ::: "memory");
@@ -192,44 +204,50 @@ __global__ __launch_bounds__(kMidThreads) void project_mid_kernel(ProjectKernelA
   finish_head<S, MODE, MB>(p, acc, head, lds0 + wave * kEpWaveBytes, lane);
 }
 
-template <int MB>
+template <int MB, int WAVES>
 hipError_t prepare_shape() {
-  const void* kernels[] = {(const void*)project_mid_kernel<F16, kModeQkv, MB>,
-                           (const void*)project_mid_kernel<BF16, kModeQkv, MB>,
-                           (const void*)project_mid_kernel<F16, kModeAdd, MB>,
-                           (const void*)project_mid_kernel<BF16, kModeAdd, MB>};
+  const void* kernels[] = {(const void*)project_mid_kernel<F16, kModeQkv, MB, WAVES>,
+                           (const void*)project_mid_kernel<BF16, kModeQkv, MB, WAVES>,
+                           (const void*)project_mid_kernel<F16, kModeAdd, MB, WAVES>,
+                           (const void*)project_mid_kernel<BF16, kModeAdd, MB, WAVES>};
   for (const void* k : kernels) {
     const hipError_t e =
-        hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, MidShape<MB>::kLdsBytes);
+        hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, MidShape<MB, WAVES>::kLdsBytes);
     if (e != hipSuccess) return e;
   }
   return hipSuccess;
 }
 
-template <int MB>
+template <int MB, int WAVES>
 hipError_t launch_shape(ProjectKernelArgs p, int dtype, bool add, hipStream_t stream) {
-  p.tiles_m = (p.rows + MidShape<MB>::kTokens - 1) / MidShape<MB>::kTokens;
+  using Shape = MidShape<MB, WAVES>;
+  p.tiles_m = (p.rows + Shape::kTokens - 1) / Shape::kTokens;
   p.tiles_n = p.heads0 + 2 * p.heads_kv;
   const uint32_t blocks = p.tiles_m * p.tiles_n;
   auto go = [&](auto kernel) {
-    hipLaunchKernelGGL(kernel, dim3(blocks), dim3(kMidThreads), MidShape<MB>::kLdsBytes, stream, p);
+    hipLaunchKernelGGL(kernel, dim3(blocks), dim3(Shape::kThreads), Shape::kLdsBytes, stream, p);
     return hipGetLastError();
   };
   if (add)
-    return dtype == 0 ? go(project_mid_kernel<F16, kModeAdd, MB>) : go(project_mid_kernel<BF16, kModeAdd, MB>);
-  return dtype == 0 ? go(project_mid_kernel<F16, kModeQkv, MB>) : go(project_mid_kernel<BF16, kModeQkv, MB>);
+    return dtype == 0 ? go(project_mid_kernel<F16, kModeAdd, MB, WAVES>) : go(project_mid_kernel<BF16, kModeAdd, MB, WAVES>);
+  return dtype == 0 ? go(project_mid_kernel<F16, kModeQkv, MB, WAVES>) : go(project_mid_kernel<BF16, kModeQkv, MB, WAVES>);
 }
 
 }  // namespace
 
 hipError_t mid_prepare() {
-  const hipError_t e = prepare_shape<1>();
-  return e != hipSuccess ? e : prepare_shape<2>();
+  const hipError_t e = prepare_shape<1, 4>();
+  return e != hipSuccess ? e : prepare_shape<1, 8>();
 }
 
+// The 256-token tile runs as eight waves of one token block each: measured against four waves of two
+// blocks at 1536 rows x 2048 -> 5120, 36.9 against 39.5 us (either way a compute unit takes in
+// (256 + 128) x 128 bytes of operands per chunk at the 55-60 GB/s one unit streams from L2, which is
+// what sets the chunk time of 0.8 us; the second wave per SIMD only hides the stalls around it).
 hipError_t launch_project_mid(ProjectKernelArgs p, uint32_t token_blocks, int dtype, bool add,
                               hipStream_t stream) {
-  return token_blocks == 2 ? launch_shape<2>(p, dtype, add, stream) : launch_shape<1>(p, dtype, add, stream);
+  if (token_blocks != 2) return launch_shape<1, 4>(p, dtype, add, stream);
+  return launch_shape<1, 8>(p, dtype, add, stream);
 }
 
 }  // namespace proj
