@@ -1321,7 +1321,12 @@ def main():
             targets[f"layerstep_{lb}x{ll}"] = {
                 "ms": round(dev_ms, 4), "us_per_layer": round(dev_ms * 1e3 / 48, 2),
                 "three_calls_us_per_layer": round(ls["graph_dev_ms"] * 1e3 / 48, 2),
+                "fused_us_per_layer": round(ls["fused_dev_ms"] * 1e3 / 48, 2),
                 "frac": round(nbytes / (dev_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)}
+
+    cpu = None
+    if not args.skip_cpu and dec is not None:
+        cpu = cpu_baseline_decode(16, 8192)
 
     also += last_entries
     if dec is None:  # partial run for profiling
