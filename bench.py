@@ -39,7 +39,9 @@ TRAFFIC_BYTES = {
     "prefill": (1363516 + 319881) * 1024,
     "kvwrite": (73808 + 65536) * 1024,
     "qkv": (1130126 + 327680) * 1024,          # fetched past the L2s (mostly from the last-level cache) + written
-    "stepproj": (21383 + 1318) * 1024,
+    "stepproj": (2 * 10695 + 1318) * 1024,
+    # 48 layers of the fused step, 16 x 8192: raw Q/K/V sums + attention finishing them + output projection
+    "layerstep_16x8192": 48 * (2 * (10534 + 131938 + 8990) + 320 + 2378 + 128) * 1024,
 }
 MFMA_F16_PEAK_TFLOPS = 2500.0  # MI355X dense fp16/bf16 MFMA, published
 D = 128
@@ -1315,7 +1317,7 @@ def main():
                 "roofline": {"bound": "hbm", "achieved": round(nbytes / (dev_ms * 1e-3) / 1e9, 1),
                              "peak": HBM_PEAK_GBS, "unit": "GB/s",
                              "frac": round(nbytes / (dev_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
-                             "traffic": None},
+                             "traffic": TRAFFIC_BYTES.get(f"layerstep_{lb}x{ll}")},
                 "cpu_baseline": ls_cpu,
             })
             targets[f"layerstep_{lb}x{ll}"] = {

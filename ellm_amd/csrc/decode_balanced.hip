@@ -26,7 +26,7 @@ namespace {
 
 constexpr uint32_t kUnitKeys = kDecodeStepKeys;   // 64: one step of the four waves
 constexpr uint32_t kMaxBatch = 1024;              // lengths are scanned in LDS
-constexpr uint32_t kMaxPieces = kMergeFan * kMergeFan;  // two fold levels of 16
+static_assert(kBalancedFan == (uint32_t)kMergeFan, "decode_shares.hpp numbers the slots for this fan");
 
 // (the compiler cannot see that a value every lane computes alike is wave-uniform)
 __device__ __forceinline__ uint32_t uni(uint32_t v) { return (uint32_t)__builtin_amdgcn_readfirstlane((int)v); }
@@ -116,39 +116,25 @@ __global__ __launch_bounds__(kDecThreads, 2) void decode_balanced_kernel(DecodeK
   const uint32_t PL = p.n_kv_heads * p.head_groups;   // planes per sequence
   const uint32_t U = PL * total_units;
   // workgroups that take part: at most one per unit, and few enough that no plane is cut
-  // into more pieces than two fold levels take (a plane of u units has at most u / q + 2
-  // pieces, q = U / W units being the smaller share)
-  const uint32_t q_min = (umax_all + kMaxPieces - 3) / (kMaxPieces - 2);
+  // into more pieces than two fold levels take.
   // Planes of equal length (to the unit): a whole number of workgroups per plane, so that the
   // shares below end where the planes end and no workgroup starts a second piece (24 sequences
   // x 8192 keys: 96 planes, 480 workgroups of 5 pieces a plane instead of 512 shares of 5.33).
   // Else a multiple of eight, for the XCD order below.
-  const uint32_t planes_all = PL * B;
-  auto takers = [&](uint32_t limit) {
-    uint32_t n = min(min(limit, U), U / q_min);
-    if (umax_all == umin_all && planes_all <= n)
-      n -= n % planes_all;
-    else if (n >= 8)
-      n &= ~7u;
-    return n;
-  };
   // One workgroup per compute unit streams as fast as two that share one, leaves half the
   // partial rows to fold and ends more evenly (32 sequences of 1k-128k keys: 658 against 679 us);
   // two per unit are better where the rounding above would leave units idle (96 equal planes:
   // 192 of 256) and where a workgroup walks several short planes one after the other, each with
   // its own start-up that a second workgroup on the unit hides (400 planes of 100-4096 keys).
-  uint32_t W = takers(gridDim.x);
-  if (p.wgs_one < gridDim.x && planes_all <= p.wgs_one) {
-    const uint32_t one_each = takers(p.wgs_one);
-    if (100u * one_each >= 47u * W) W = one_each;
-  }
+  // (decode_shares.hpp: balanced_workgroups, also walked by the CPU tests)
+  const uint32_t planes_all = PL * B;
+  const uint32_t W = balanced_workgroups(gridDim.x, p.wgs_one, U, umax_all, umin_all, planes_all);
   // Workgroups are dealt to the eight XCDs by their id modulo 8.  Each XCD takes one contiguous
   // eighth of the shares, so that no two of them walk the same stretch of memory side by side
   // (with shares numbered like the workgroups and as many pieces per plane as XCDs, every XCD
   // would read the same stretch of every plane).
-  uint32_t w = blockIdx.x;
-  if (w >= W) return;
-  if ((W & 7u) == 0) w = (w & 7u) * (W >> 3) + (w >> 3);
+  if (blockIdx.x >= W) return;
+  const uint32_t w = balanced_share_of(blockIdx.x, W);
   // share g begins at floor(g U / W) (decode_shares.hpp): equal to the unit, and for equal planes
   // with W a multiple of their number a plane's end is a share's end
   const Shares shares(W, U);
@@ -196,7 +182,7 @@ __global__ __launch_bounds__(kDecThreads, 2) void decode_balanced_kernel(DecodeK
     const uint32_t last_w = stop == E ? w : holder(E - 1);
     const uint32_t n_pieces = last_w - first_w + 1, piece = w - first_w;
     const uint32_t plane_id = seq * PL + pl;
-    const uint32_t slot0 = first_w + plane_id;
+    const uint32_t slot0 = balanced_slot0(first_w, plane_id);
 
     const uint32_t k_begin = a * kUnitKeys;
     const uint32_t k_end = min(pos + 1, a_end * kUnitKeys);
@@ -248,7 +234,7 @@ __global__ __launch_bounds__(kDecThreads, 2) void decode_balanced_kernel(DecodeK
       const uint32_t n_clusters = (n_pieces + kMergeFan - 1) / kMergeFan;
       const uint32_t cluster = piece / kMergeFan;
       const uint32_t in_cluster = min((uint32_t)kMergeFan, n_pieces - cluster * kMergeFan);
-      const uint32_t cslot0 = plane_id + slot0 / kMergeFan;
+      const uint32_t cslot0 = balanced_cluster_slot0(slot0, plane_id);
       if (arrive(p.counters + cslot0 + cluster, in_cluster, &s_last, t.tid)) {
         if (n_clusters == 1) {
           fold(smem, t, heads_here, p.ws_acc, p.ws_ml, slot0 * G, 1, G, n_pieces, final_row);
@@ -281,7 +267,7 @@ bool decode_balanced_takes(const DecodeWorkspace& w, uint32_t batch, uint32_t n_
   const uint64_t units = planes * ((max_len + kUnitKeys - 1) / kUnitKeys);
   if (units < 8ull * wgs || units + wgs >= (1ull << 31) || wgs >= (1u << 16)) return false;
   const uint64_t G = group < (uint32_t)kMaxHeadsPerGroup ? group : (uint32_t)kMaxHeadsPerGroup;
-  const uint64_t slots = wgs + planes, cslots = planes + slots / kMergeFan + 2;
+  const uint64_t slots = balanced_slots(wgs, (uint32_t)planes), cslots = balanced_cluster_slots(wgs, (uint32_t)planes);
   return slots * G <= w.rows && cslots * G <= w.rows2 && cslots + planes <= w.counters;
 }
 
@@ -315,7 +301,7 @@ hipError_t launch_decode_balanced(const AttnArgs& a, uint32_t wgs, hipStream_t s
   p.scale_log2 = a.scale * kLog2e;
   // cluster slots (the kernel's cslot0 + cluster stays below this): the planes' own counters follow
   const uint32_t planes = a.batch * a.n_kv_heads * p.head_groups;
-  p.n_cluster_max = planes + (wgs + planes) / kMergeFan + 2;
+  p.n_cluster_max = balanced_cluster_slots(wgs, planes);
   p.counters_per_plane = 0;
   p.pend = a.pending;
   const dim3 grid(wgs), block(kDecThreads);
