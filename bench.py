@@ -1114,12 +1114,24 @@ def main():
         lc_dec = bench_decode(24, 8192, args.steps, min(args.warmup, 5), copies=3)
         lc = {t: bench_prefill(t, args.steps, min(args.warmup, 5), p0=8192, batch=24, copies=3) for t in (2, 8, 16, 24, 33, 48, 64)}
         kv_bytes = 2 * 24 * 4 * 8192 * D * 2
+        # the same launches on K = V = 0 (same instruction stream, operands that toggle nothing) with the
+        # board's power and engine clock beside them: what the operand values cost under the power cap
+        lc_pw = {}
+        for t in (16, 64):
+            real = bench_prefill(t, 5, 2, p0=8192, batch=24, copies=3, power_seconds=0.6)
+            zero = bench_prefill(t, 5, 2, p0=8192, batch=24, copies=3, zero_kv=True, power_seconds=0.6)
+            lc_pw[str(t)] = {"us": round(real["kernel_ms"] * 1e3, 1), "zero_kv_us": round(zero["kernel_ms"] * 1e3, 1),
+                             "watts": (real["power"] or {}).get("watts"), "engine_mhz": (real["power"] or {}).get("engine_mhz"),
+                             "zero_kv_watts": (zero["power"] or {}).get("watts"),
+                             "zero_kv_engine_mhz": (zero["power"] or {}).get("engine_mhz"),
+                             "cap_watts": (real["power"] or {}).get("cap_watts")}
         also.append({
             "workload": "last chunk: 2-64 tokens x 24 seq on 8192-token caches, 32q/4kv, fp16; value = 16 tokens",
             "metric": "chunk attention us per call", "unit": "us",
             "value": round(lc[16]["ms_per_step"] * 1e3, 1),
             "us_by_tokens": {str(t): round(r["ms_per_step"] * 1e3, 1) for t, r in lc.items()},
             "single_token_us": round(lc_dec["ms_per_step"] * 1e3, 1),
+            "board_power_by_tokens": lc_pw,
             "kv_gbs_by_tokens": {str(t): round(kv_bytes / (r["ms_per_step"] * 1e-3) / 1e9, 1) for t, r in lc.items()},
             "steps": args.steps,
             "roofline": {"bound": "hbm", "achieved": round(kv_bytes / (lc[16]["kernel_ms"] * 1e-3) / 1e9, 1),
@@ -1128,7 +1140,9 @@ def main():
                          "traffic": TRAFFIC_BYTES["lastchunk"]},
         })
         targets["lastchunk_24x8192"] = {"us_by_tokens": {str(t): round(r["kernel_ms"] * 1e3, 1) for t, r in lc.items()},
-                                        "single_token_us": round(lc_dec["kernel_ms"] * 1e3, 1)}
+                                        "single_token_us": round(lc_dec["kernel_ms"] * 1e3, 1),
+                                        "zero_kv_us": {t: v["zero_kv_us"] for t, v in lc_pw.items()},
+                                        "engine_mhz": {t: v["engine_mhz"] for t, v in lc_pw.items()}}
 
     if args.only in ("", "mixed"):
         # one layer of the mixed-step configuration: a 16384-token prefill and a single-token step over 32

@@ -62,6 +62,10 @@ PREFILL = [
     ("stream_g16_20tok_twelve_waves_below_capacity", 3, 2, 16, 1, 900, 700, 20),
     ("stream_g3_50tok_eight_waves_odd_group", 2, 2, 6, 2, 800, 600, 50),
     ("pingpong_49tok_b24", 24, 24, 32, 4, 1200, 1001, 49),           # 392 rows a plane: the tile kernel
+    # up to the reference's full chunk (sequence_chunk_size = 64, src/serving/start copy.rs:30) x 24 sequences
+    ("chunk_56tok_b24_off_tile_edge", 24, 24, 32, 4, 1200, 1001, 56),
+    ("chunk_63tok_b24_across_tile_edge", 24, 24, 32, 4, 1200, 1087, 63),
+    ("chunk_64tok_b24_on_tile_edge", 24, 24, 32, 4, 1216, 1088, 64),
     ("stream_batch_below_capacity_9tok", 5, 3, 8, 2, 900, 700, 9),    # 36 rows: a part-filled second wave
     ("stream_g16_8tok_full_workgroup", 1, 1, 16, 1, 3000, 2900, 8),   # 128 rows exactly
     ("stream_first_split_only_for_early_rows", 2, 2, 8, 2, 700, 500, 5),
