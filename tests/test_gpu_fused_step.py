@@ -252,3 +252,135 @@ def test_fused_step_refuses_handles_of_different_steps():
     finally:
         a.close()
         b.close()
+
+
+def _two_calls_and_fused(make_ops, reset, snapshot, positions, batch):
+    """Runs the step as the two ordinary calls and as the fused call on freshly reset buffers;
+    returns both snapshots."""
+    import torch
+
+    qkv, attn = make_ops()
+    try:
+        assert qkv.attention_path(attn, batch) == 1
+        dpos = _positions_dev(positions)
+        bound = int(max(positions))
+        reset()
+        qkv.run_ragged(dpos, bound, batch)
+        attn.run_ragged(dpos, bound, batch)
+        plain = snapshot()
+        reset()
+        qkv.run_with_attention(attn, bound, batch, positions=dpos)
+        fused = snapshot()
+        torch.cuda.synchronize()
+    finally:
+        qkv.close()
+        attn.close()
+    return plain, fused
+
+
+def _assert_fused_equals_plain(plain, fused, dtype, batch):
+    for what, a, b in zip(("q", "k", "v"), plain[:3], fused[:3]):
+        live = (slice(None), slice(0, batch)) if what == "q" else slice(None)
+        assert np.array_equal(a[live], b[live]), what
+    f = lambda a: orc.from_storage(a, dtype)
+    r = compare(f(fused[3])[:, :batch], f(plain[3])[:, :batch], dtype)
+    assert r["ok"], r
+    assert np.abs(fused[4][:, :batch] - plain[4][:, :batch]).max() <= LSE_TOL
+
+
+@pytest.mark.parametrize("dtype", [orc.F16, orc.BF16], ids=["f16", "bf16"])
+def test_fused_step_on_a_cache_with_per_sequence_capacities(dtype):
+    """Both handles over one layer of an ellm_kv_create_ragged cache (the same sequence table):
+    the new rows land where the two ordinary calls put them, bit for bit, the last row of the
+    shortest plane included; the ordinary calls on this cache are checked against the uniform
+    cache and the oracle in test_gpu_ragged_cache.py."""
+    import torch
+
+    import ellm_amd
+
+    caps = [320, 64, 1000, 129]
+    hq, hkv, hidden, b = 8, 2, 1024, 4
+    tdt = torch_dtype(dtype)
+    cache = ellm_amd.KVCache.ragged(1, caps, hkv, ellm_amd.DTYPE_F16 if dtype == orc.F16 else ellm_amd.DTYPE_BF16)
+    view = cache.layer_ragged(0)
+    kt, vt = cache.layer_flat_tensors(0, tdt)
+    k0 = to_dev(rand_storage(tuple(kt.shape), 3, dtype), dtype)
+    v0 = to_dev(rand_storage(tuple(vt.shape), 4, dtype), dtype)
+    w = [to_dev(rand_storage((h * D, hidden), 20 + i, dtype, scale=hidden ** -0.5), dtype) for i, h in enumerate((hq, hkv, hkv))]
+    rope = to_dev(_rope_table(max(caps), dtype), dtype)
+    x = to_dev(rand_storage((1, b, hidden), 30, dtype), dtype)
+    q = torch.zeros((1, b, hq, D), dtype=tdt, device="cuda")
+    att = torch.zeros_like(q)
+    lse = torch.zeros((1, b, hq), dtype=torch.float32, device="cuda")
+
+    def make_ops():
+        return (ellm_amd.MatMul3(x, w[0], q, w[1], kt, w[2], vt, rope, D, b, hq, hkv, view.strides, 0, seq_table=view),
+                ellm_amd.Attention(q, kt, vt, att, b, hq, hkv, D, view.strides, 1.0 / np.sqrt(D), lse=lse,
+                                   max_position_interval=1, seq_table=view))
+
+    def reset():
+        kt.copy_(k0.view(kt.shape))
+        vt.copy_(v0.view(vt.shape))
+        for t in (q, att, lse):
+            t.fill_(float("nan"))
+
+    def snapshot():
+        torch.cuda.synchronize()
+        return [t.view(torch.int16).cpu().numpy().view(np.uint16).copy() for t in (q, kt, vt, att)] + [lse.cpu().numpy().copy()]
+
+    try:
+        for positions in ([319, 63, 999, 128], [0, 17, 512, 64]):
+            print("positions", positions, flush=True)
+            plain, fused = _two_calls_and_fused(make_ops, reset, snapshot, positions, b)
+            _assert_fused_equals_plain(plain, fused, dtype, b)
+            assert not np.isnan(orc.from_storage(fused[3], dtype)).any()
+    finally:
+        cache.close()
+
+
+def test_fused_step_on_the_reference_state_layout():
+    """K/V as the reference's own [position][sequence][kv_head][128] state
+    (src/qwen3_moe/attention.rs:149-166), kv_strides = [Hkv*D, D, B*Hkv*D, 1]: the fused call
+    against the two ordinary calls, whose results on this layout test_gpu_parity.py and
+    test_gpu_projection.py check against the oracle."""
+    import torch
+
+    import ellm_amd
+
+    dtype = orc.F16
+    b, hq, hkv, cap, hidden = 3, 8, 2, 600, 1024
+    strides = [hkv * D, D, b * hkv * D, 1]
+    k0 = to_dev(rand_storage((cap, b, hkv, D), 5, dtype), dtype)
+    v0 = to_dev(rand_storage((cap, b, hkv, D), 6, dtype), dtype)
+    kt, vt = torch.zeros_like(k0), torch.zeros_like(v0)
+    w = [to_dev(rand_storage((h * D, hidden), 40 + i, dtype, scale=hidden ** -0.5), dtype) for i, h in enumerate((hq, hkv, hkv))]
+    rope = to_dev(_rope_table(cap, dtype), dtype)
+    x = to_dev(rand_storage((1, b, hidden), 50, dtype), dtype)
+    q = torch.zeros((1, b, hq, D), dtype=torch.float16, device="cuda")
+    att = torch.zeros_like(q)
+    lse = torch.zeros((1, b, hq), dtype=torch.float32, device="cuda")
+
+    def make_ops():
+        return (ellm_amd.MatMul3(x, w[0], q, w[1], kt, w[2], vt, rope, D, b, hq, hkv, strides, cap),
+                ellm_amd.Attention(q, kt, vt, att, b, hq, hkv, D, strides, 1.0 / np.sqrt(D), lse=lse,
+                                   sequence_capacity=cap, max_position_interval=1))
+
+    def reset():
+        kt.copy_(k0)
+        vt.copy_(v0)
+        for t in (q, att, lse):
+            t.fill_(float("nan"))
+
+    def snapshot():
+        torch.cuda.synchronize()
+        return [t.view(torch.int16).cpu().numpy().view(np.uint16).copy() for t in (q, kt, vt, att)] + [lse.cpu().numpy().copy()]
+
+    positions = [599, 0, 300]
+    plain, fused = _two_calls_and_fused(make_ops, reset, snapshot, positions, b)
+    _assert_fused_equals_plain(plain, fused, dtype, b)
+    # only the rows at the sequences' positions changed, and they did change
+    kb, k0b = fused[1], k0.view(torch.int16).cpu().numpy().view(np.uint16)
+    mask = np.ones((cap, b, hkv), dtype=bool)
+    for s, p in enumerate(positions):
+        mask[p, s, :] = False
+    assert np.array_equal(kb[mask], k0b[mask]) and not np.array_equal(kb[~mask], k0b[~mask])
