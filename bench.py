@@ -327,10 +327,19 @@ def bench_kv_write(n_tokens, steps, warmup, hkv=4, seqs=1):
     rows = n_tokens * seqs * hkv
     alg_bytes = rows * D * 2 * 4 + cap * D * 2          # K, V read and written; the table read once
     kern_ms = sum(per) / len(per)
+    # yardsticks on the same buffers: the library's plain write (ellm_kv_append: the same rows copied,
+    # nothing computed) and the runtime's own device-to-device copy of the same bytes
+    per_plain, _ = _time_steps(lambda i: cache.append(i % copies, 0, ks[i % copies], vs[i % copies]), steps, warmup)
+    dst = [torch.empty((2,) + tuple(ks[0].shape), dtype=torch.float16, device="cuda") for _ in range(copies)]
+    src = [torch.stack((ks[c], vs[c])) for c in range(copies)]
+    per_copy, _ = _time_steps(lambda i: dst[i % copies].copy_(src[i % copies]), steps, warmup)
+    copy_bytes = rows * D * 2 * 4
     cache.close()
     return {"alg_bytes": alg_bytes, "ms_per_step": step_ms, "kernel_ms": kern_ms,
             "gbs": alg_bytes / (step_ms * 1e-3) / 1e9,
-            "kernel_gbs": alg_bytes / (kern_ms * 1e-3) / 1e9}
+            "kernel_gbs": alg_bytes / (kern_ms * 1e-3) / 1e9,
+            "plain_append_gbs": copy_bytes / (sum(per_plain) / len(per_plain) * 1e-3) / 1e9,
+            "device_copy_gbs": copy_bytes / (sum(per_copy) / len(per_copy) * 1e-3) / 1e9}
 
 
 def bench_mixed_step(layers, prefill_tokens, batch, lo, hi, steps, warmup, hidden=2048, hq=32, hkv=4, seed=7):
@@ -1210,6 +1219,9 @@ def main():
             "workload": "cache write, key RMS norm + rotation: 32768 tokens x 4 kv heads, fp16",
             "metric": "kv write HBM GB/s", "value": round(kw["gbs"], 1), "unit": "GB/s",
             "ms_per_step": round(kw["ms_per_step"], 5), "steps": args.steps,
+            # the same rows through ellm_kv_append (copied, nothing computed) and the same bytes through
+            # the runtime's device-to-device copy, timed in this run
+            "plain_append_gbs": round(kw["plain_append_gbs"], 1), "device_copy_gbs": round(kw["device_copy_gbs"], 1),
             "roofline": {"bound": "hbm", "achieved": round(kw["kernel_gbs"], 1),
                          "peak": HBM_PEAK_GBS, "unit": "GB/s",
                          "frac": round(kw["kernel_gbs"] / HBM_PEAK_GBS, 4),

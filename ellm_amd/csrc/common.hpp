@@ -100,6 +100,9 @@ __device__ __forceinline__ float fast_log2(float x) { return __builtin_amdgcn_lo
 
 __device__ __forceinline__ u32x4 load16(const void* p) { return *(const u32x4*)p; }
 __device__ __forceinline__ void store16(void* p, u32x4 v) { *(u32x4*)p = v; }
+// The same for bytes that are touched once (streamed rows): marked so that the caches do not keep them.
+__device__ __forceinline__ u32x4 load16_once(const void* p) { return __builtin_nontemporal_load((const u32x4*)p); }
+__device__ __forceinline__ void store16_once(void* p, u32x4 v) { __builtin_nontemporal_store(v, (u32x4*)p); }
 
 // Exchange with the lane whose index differs in the given bit (16 or 32).
 __device__ __forceinline__ float xor_shuffle(float v, int mask) { return __shfl_xor(v, mask, 64); }

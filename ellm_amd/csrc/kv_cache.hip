@@ -26,8 +26,8 @@ __global__ __launch_bounds__(256) void kv_append_kernel(
     const size_t src = (((size_t)t * src_batch_pitch + b) * n_kv_heads + h) * kHeadDim + 8 * c;
     const size_t dst = seq_plane_offset(layout.seq_offsets, layout.stride_seq, b) +
                        (size_t)h * layout.stride_head + (size_t)(position_index + t) * kHeadDim + 8 * c;
-    store16(k_dst + dst, load16(k_src + src));
-    store16(v_dst + dst, load16(v_src + src));
+    store16_once(k_dst + dst, load16_once(k_src + src));
+    store16_once(v_dst + dst, load16_once(v_src + src));
   }
 }
 
@@ -42,9 +42,14 @@ __global__ __launch_bounds__(256) void kv_append_kernel(
 // one rounding per operation, in the order of the reference's scalar code: the
 // sum of squares runs through the 128 elements from first to last (the sixteen
 // lanes take turns, each adding its eight squares to the running sum it is
-// handed), so the result is the same bits a sequential CPU loop produces.  The
-// extra instructions (about 150 a row) stay well under what the HBM transfer of
-// the row allows.
+// handed), so the result is the same bits a sequential CPU loop produces.
+// The value lane - 1 of the same 16-lane row holds; 0 in the row's first lane (a data-parallel
+// move inside the vector ALU, no trip through the LDS crossbar).
+__device__ __forceinline__ float from_left_neighbour(float v) {
+  constexpr int kRowShr1 = 0x111;
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), kRowShr1, 0xf, 0xf, true));
+}
+
 template <typename T>
 __global__ __launch_bounds__(256) void kv_append_norm_rope_kernel(
     uint16_t* __restrict__ k_dst, uint16_t* __restrict__ v_dst, const uint16_t* __restrict__ k_src,
@@ -74,8 +79,8 @@ __global__ __launch_bounds__(256) void kv_append_norm_rope_kernel(
     const uint32_t pos_dst = layout.seq_caps ? min(pos, layout.seq_caps[b] - 1) : pos;
     const size_t dst = seq_plane_offset(layout.seq_offsets, layout.stride_seq, b) +
                        (size_t)h * layout.stride_head + (size_t)pos_dst * kHeadDim + 8 * c;
-    const u32x4 kraw = load16(k_src + src);
-    const u32x4 vraw = load16(v_src + src);
+    const u32x4 kraw = load16_once(k_src + src);
+    const u32x4 vraw = load16_once(v_src + src);
     const u32x4 rraw = load16(rope + (size_t)pos * kHeadDim + 8 * c);
     float x[8], sq[8];
 #pragma unroll
@@ -85,14 +90,18 @@ __global__ __launch_bounds__(256) void kv_append_norm_rope_kernel(
     }
 #pragma unroll
     for (int e = 0; e < 8; ++e) sq[e] = x[e] * x[e];
-    float sum = 0.0f;  // sum of squares of all elements before this lane's
+    // Turn by turn every lane adds its eight squares to what its left neighbour held after the
+    // turn before (a row shift inside the 16-lane row, zero into lane 0): lane c's value is final
+    // from turn c on, so after sixteen turns lane 15 holds the sum over all 128 elements, added
+    // first to last.
+    float mine = 0.0f;
 #pragma unroll
     for (int l = 0; l < 16; ++l) {
-      float mine = sum;
+      mine = from_left_neighbour(mine);
 #pragma unroll
       for (int e = 0; e < 8; ++e) mine = mine + sq[e];
-      sum = __shfl(mine, l, 16);  // lane l's total moves on to everybody
     }
+    const float sum = __shfl(mine, 15, 16);
     const float variance = sum / (float)kHeadDim;
     const float rrms = 1.0f / (sqrtf(variance) + eps);
     u32x4 out;
@@ -106,8 +115,8 @@ __global__ __launch_bounds__(256) void kv_append_norm_rope_kernel(
       out[e] = T::pack2(re, im);
     }
     if (live) {
-      store16(k_dst + dst, out);
-      store16(v_dst + dst, vraw);
+      store16_once(k_dst + dst, out);
+      store16_once(v_dst + dst, vraw);
     }
   }
 }
