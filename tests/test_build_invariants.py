@@ -35,7 +35,8 @@ def test_one_head_tile_kernels_leave_m0_to_the_inline_asm(tmp_path):
     assert not any("movrel" in l or "s_set_gpr_idx" in l for l in code)
 
 
-@pytest.mark.parametrize("name", ["project_mid.hip", "project_small.hip", "prefill.hip", "decode.hip", "decode_balanced.hip"])
+@pytest.mark.parametrize("name", ["project.hip", "project_mid.hip", "project_small.hip", "prefill.hip", "decode.hip",
+                                  "decode_balanced.hip", "kv_cache.hip"])
 def test_hot_kernels_do_not_spill(name, tmp_path):
     text = _listing(name, tmp_path)
     sizes = [int(x) for x in re.findall(r"\.private_segment_fixed_size:\s*(\d+)", text)]
@@ -57,14 +58,12 @@ def _loops(lines):
     return out
 
 
-@pytest.mark.parametrize("name,limit,in_loop", [("project.hip", 64, 0)])
-def test_projection_kernels_keep_scratch_out_of_their_matrix_loops(name, limit, in_loop, tmp_path):
-    """The 256 x 256 tile kernel runs at 512 registers a lane and parks a few epilogue values
-    (destination rows, computed once per tile after the K loop) in scratch.  That is harmless
-    only while it stays a few dozen bytes and the K loop never touches scratch."""
+@pytest.mark.parametrize("name,in_loop", [("project.hip", 0)])
+def test_projection_kernels_keep_scratch_out_of_their_matrix_loops(name, in_loop, tmp_path):
+    """The 256 x 256 tile kernel runs at 512 registers a lane: whatever the register allocator
+    does with the epilogue's values, the K loop never touches scratch (the kernel has none
+    today: test_hot_kernels_do_not_spill)."""
     text = _listing(name, tmp_path)
-    sizes = [int(x) for x in re.findall(r"\.private_segment_fixed_size:\s*(\d+)", text)]
-    assert sizes and max(sizes) <= limit, sizes
     lines = [l.split(";")[0] for l in text.splitlines()]
     for first, last in _loops(lines):
         body = lines[first:last + 1]
