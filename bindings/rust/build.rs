@@ -27,7 +27,7 @@ fn main() {
     // so that binaries find the library without LD_LIBRARY_PATH
     println!("cargo:rustc-link-arg=-Wl,-rpath,{}", lib_dir.display());
     for f in [
-        "api.hip", "noalloc.hip", "decode.hip", "decode_balanced.hip", "prefill.hip", "kv_cache.hip",
+        "api.hip", "attn_general.hip", "noalloc.hip", "decode.hip", "decode_balanced.hip", "prefill.hip", "kv_cache.hip",
         "project.hip", "project_mid.hip", "project_small.hip", "project_api.hip", "step.hip", "handles.hpp", "common.hpp",
         "kernels.hpp", "decode_common.hpp", "decode_plan.hpp", "decode_shares.hpp", "chunk_plan.hpp", "project_common.hpp",
         "project_epilogue.hpp", "Makefile",

@@ -38,6 +38,8 @@ pub const ELLM_ERR_NO_DEVICE: c_int = 5;
 
 pub const ELLM_DTYPE_F16: c_int = 0;
 pub const ELLM_DTYPE_BF16: c_int = 1;
+/// Attention only (`ellm_attn_create`): binary32 storage, the plain kernel.
+pub const ELLM_DTYPE_F32: c_int = 2;
 
 // ---- descriptors (field for field as in include/ellm_attn.h) ------------------------------
 

@@ -10,6 +10,7 @@ from ._lib import (  # noqa: F401
     ABI_SYMBOLS,
     DTYPE_BF16,
     DTYPE_F16,
+    DTYPE_F32,
     EllmError,
     LibraryMissing,
     lib_path,

@@ -4,6 +4,7 @@ import os
 
 DTYPE_F16 = 0
 DTYPE_BF16 = 1
+DTYPE_F32 = 2   # attention only
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 

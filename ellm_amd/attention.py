@@ -16,13 +16,15 @@ from . import _lib
 from ._lib import AttnDesc, KvDesc, KvRaggedDesc, KvSeqTable, check, load_library
 
 
-def _dtype_code(t):
+def _dtype_code(t, allow_f32=False):
     import torch
 
     if t.dtype == torch.float16:
         return _lib.DTYPE_F16
     if t.dtype == torch.bfloat16:
         return _lib.DTYPE_BF16
+    if allow_f32 and t.dtype == torch.float32:
+        return _lib.DTYPE_F32
     raise TypeError(f"unsupported storage type {t.dtype}")
 
 
@@ -63,6 +65,8 @@ class Attention:
 
     q, out: [max_position_interval, batch_capacity, attention_head_num, head_size]
     k, v:   any 4-d view [sequence, kv_head, position, head_size] (strides are passed on)
+    float16 / bfloat16 tensors with head_size 128 run the MFMA kernels; other head sizes up to
+    256 and float32 tensors run the library's plain kernel (same arguments and results).
     """
 
     def __init__(self, q, k, v, out, batch_size, attention_head_num, kv_head_num, head_size,
@@ -96,7 +100,7 @@ class Attention:
         for i in range(4):
             d.kv_strides[i] = int(kv_strides[i])
         d.inverse_sqrt_head = float(inverse_sqrt_head)
-        d.dtype = _dtype_code(q)
+        d.dtype = _dtype_code(q, allow_f32=True)
         d.sequence_capacity = cap
         d.max_position_interval = interval
         self.desc = d

@@ -69,17 +69,20 @@ int ellm::set_error(int status, const char* fmt, ...) {
   return status;
 }
 
+bool ellm::attn_is_general(const ellm_attn_desc& d) { return d.head_size != 128 || d.dtype == ELLM_DTYPE_F32; }
+
 int ellm::validate_attn_desc(const ellm_attn_desc* d) {
   if (!d) return fail(ELLM_ERR_INVALID_ARGUMENT, "null descriptor");
   if (!d->q || !d->k || !d->v || !d->out)
     return fail(ELLM_ERR_INVALID_ARGUMENT, "q, k, v and out must be non-null device pointers");
   if (!aligned16(d->q) || !aligned16(d->k) || !aligned16(d->v) || !aligned16(d->out))
     return fail(ELLM_ERR_INVALID_ARGUMENT, "q, k, v and out must be 16-byte aligned");
-  if (d->dtype != ELLM_DTYPE_F16 && d->dtype != ELLM_DTYPE_BF16)
-    return fail(ELLM_ERR_INVALID_ARGUMENT, "dtype %d is neither ELLM_DTYPE_F16 nor ELLM_DTYPE_BF16",
+  if (d->dtype != ELLM_DTYPE_F16 && d->dtype != ELLM_DTYPE_BF16 && d->dtype != ELLM_DTYPE_F32)
+    return fail(ELLM_ERR_INVALID_ARGUMENT, "dtype %d is none of ELLM_DTYPE_F16, ELLM_DTYPE_BF16, ELLM_DTYPE_F32",
                 d->dtype);
-  if (d->head_size != 128)
-    return fail(ELLM_ERR_UNSUPPORTED, "head_size %zu: only 128 is supported", d->head_size);
+  if (d->head_size == 0 || d->head_size > 256)
+    return fail(ELLM_ERR_UNSUPPORTED, "head_size %zu: 1 to 256 are supported", d->head_size);
+  const bool general = ellm::attn_is_general(*d);
   if (d->batch_size == 0 || d->attention_head_num == 0 || d->kv_head_num == 0)
     return fail(ELLM_ERR_INVALID_ARGUMENT, "batch_size, attention_head_num, kv_head_num must be > 0");
   if (d->attention_head_num % d->kv_head_num != 0)
@@ -88,10 +91,10 @@ int ellm::validate_attn_desc(const ellm_attn_desc* d) {
   if (d->kv_strides[3] != 1)
     return fail(ELLM_ERR_INVALID_ARGUMENT, "kv_strides[3] must be 1 (head dimension contiguous)");
   for (int i = 0; i < 3; ++i)
-    if (d->kv_strides[i] == 0 || d->kv_strides[i] % 8 != 0)
+    if (d->kv_strides[i] == 0 || (!general && d->kv_strides[i] % 8 != 0))
       return fail(ELLM_ERR_INVALID_ARGUMENT,
-                  "kv_strides[%d] = %zu must be a non-zero multiple of 8 elements", i,
-                  d->kv_strides[i]);
+                  "kv_strides[%d] = %zu must be a non-zero multiple of 8 elements (non-zero for head sizes "
+                  "other than 128 and for binary32)", i, d->kv_strides[i]);
   if (d->kv_strides[2] < d->head_size)
     return fail(ELLM_ERR_INVALID_ARGUMENT, "kv_strides[2] = %zu is smaller than head_size",
                 d->kv_strides[2]);
@@ -262,6 +265,13 @@ static int attn_create(const ellm_attn_desc* d, const ellm_kv_seq_table* table, 
   h->counters = nullptr;
   h->part_rows = ellm::prefill_workspace_rows((uint32_t)d->max_position_interval, (uint32_t)d->batch_size,
                                               (uint32_t)d->attention_head_num, (uint32_t)n_cu);
+  h->general = ellm::attn_is_general(*d);
+  if (h->general) {   // the kernel for other head sizes and binary32 keeps nothing between workgroups
+    h->ws = ellm::DecodeWorkspace{0, 0, 0};
+    h->part_rows = 0;
+    *out_handle = h;
+    return ELLM_OK;
+  }
   hipError_t e = hipMalloc((void**)&h->ws_acc, h->ws.rows * 128 * sizeof(float));
   if (e == hipSuccess) e = hipMalloc((void**)&h->ws_ml, h->ws.rows * 2 * sizeof(float));
   if (e == hipSuccess) e = hipMalloc((void**)&h->ws2_acc, h->ws.rows2 * 128 * sizeof(float));
@@ -293,6 +303,7 @@ int ellm_attn_create_ragged(const ellm_attn_desc* d, const ellm_kv_seq_table* ta
 int ellm_attn_reset(ellm_attn* h, void* stream) {
   if (!h) return fail(ELLM_ERR_INVALID_ARGUMENT, "null handle");
   if (int st = ellm::check_current_device(h->device)) return st;
+  if (h->general) return ELLM_OK;   // no counters
   const hipError_t e = ellm::launch_fill_u32(h->counters, h->ws.counters, 0u, (hipStream_t)stream);
   if (e != hipSuccess) return fail_hip(e, "counter reset launch");
   return ELLM_OK;
@@ -334,6 +345,11 @@ static bool takes_balanced(const ellm_attn* h, size_t batch, size_t max_position
 }
 
 int ellm::attn_run_single_token(ellm_attn* h, ellm::AttnArgs* a, uint32_t max_position, hipStream_t stream) {
+  if (h->general) {
+    const hipError_t e = ellm::launch_attn_general(*a, (uint32_t)h->desc.head_size, stream);
+    if (e != hipSuccess) return fail_hip(e, "attention launch (general head size)");
+    return ELLM_OK;
+  }
   uint32_t wgs = 0;
   if (a->positions && takes_balanced(h, a->batch, max_position, &wgs)) {
     const hipError_t e = ellm::launch_decode_balanced(*a, wgs, stream);
@@ -380,7 +396,8 @@ int ellm_attn_run(ellm_attn* h, size_t position_index, size_t position_interval,
   a.position_interval = (uint32_t)position_interval;
   a.batch = (uint32_t)batch_size;
   if (position_interval == 1) return ellm::attn_run_single_token(h, &a, (uint32_t)position_index, (hipStream_t)stream);
-  hipError_t e = ellm::launch_prefill(a, (hipStream_t)stream);
+  hipError_t e = h->general ? ellm::launch_attn_general(a, (uint32_t)d.head_size, (hipStream_t)stream)
+                            : ellm::launch_prefill(a, (hipStream_t)stream);
   if (e != hipSuccess) return fail_hip(e, "chunk attention launch");
   return ELLM_OK;
 }
@@ -412,6 +429,7 @@ int ellm_attn_ragged_path(const ellm_attn* h, size_t max_position, size_t batch_
   if (batch_size == 0 || batch_size > h->desc.batch_size || max_position >= h->desc.sequence_capacity)
     return -fail(ELLM_ERR_OUT_OF_RANGE, "batch_size %zu / max_position %zu outside the handle's %zu / %zu",
                  batch_size, max_position, h->desc.batch_size, h->desc.sequence_capacity);
+  if (h->general) return 0;
   uint32_t wgs = 0;
   return takes_balanced(h, batch_size, max_position, &wgs) ? 1 : 0;
 }

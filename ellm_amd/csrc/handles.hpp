@@ -27,6 +27,8 @@ struct ellm_attn {
   const size_t* seq_offsets;
   const uint32_t* seq_caps;
   std::vector<size_t> caps_host;
+  // a head size other than 128 or binary32 storage: every call goes to attn_general.hip
+  bool general;
 };
 
 struct ellm_matmul3 {

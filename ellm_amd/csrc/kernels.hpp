@@ -40,7 +40,7 @@ struct AttnArgs {
   size_t kv_stride_head;  // elements
   size_t kv_stride_pos;   // elements
   float scale;
-  int dtype;              // 0 = binary16, 1 = bfloat16
+  int dtype;              // 0 = binary16, 1 = bfloat16, 2 = binary32 (attn_general.hip only)
   uint32_t capacity;      // positions per K/V plane
   // per run
   uint32_t position_index;
@@ -78,6 +78,8 @@ bool decode_balanced_takes(const DecodeWorkspace& w, uint32_t batch, uint32_t n_
                            uint32_t max_len, uint32_t wgs);
 hipError_t launch_decode_balanced(const AttnArgs& a, uint32_t wgs, hipStream_t stream);
 hipError_t launch_prefill(const AttnArgs& a, hipStream_t stream);
+// Any head size up to 256 and binary32 storage (dtype 2): chunk and single-token calls alike.
+hipError_t launch_attn_general(const AttnArgs& a, uint32_t head_size, hipStream_t stream);
 
 // Where the rows of a cache layer live: plane of (sequence, head) at
 // seq_plane_offset(seq_offsets, stride_seq, sequence) + head x stride_head, rows 128 apart;
@@ -161,6 +163,9 @@ int check_current_device(int device);
 // The checks ellm_attn_create applies to a description (status + message recorded), and the
 // shape part of AttnArgs taken from a checked description (workspace pointers left null).
 int validate_attn_desc(const ellm_attn_desc* d);
+// A description the MFMA kernels do not take (head size other than 128, or binary32 storage):
+// its calls go to launch_attn_general.
+bool attn_is_general(const ellm_attn_desc& d);
 void attn_args_from_desc(const ellm_attn_desc& d, AttnArgs* a);
 
 // Looks up, once per device, the address of the current device's copy of the static scratch

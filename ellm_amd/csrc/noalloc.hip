@@ -99,6 +99,9 @@ extern "C" {
 int ellm_attn_run_noalloc(const ellm_attn_desc* desc, const uint32_t* positions, size_t position,
                           size_t batch_size, void* stream) {
   if (int st = ellm::validate_attn_desc(desc)) return st;
+  if (ellm::attn_is_general(*desc))
+    return ellm::set_error(ELLM_ERR_UNSUPPORTED, "head_size %zu / dtype %d: this entry point takes 128-wide 16-bit heads only",
+                           desc->head_size, desc->dtype);
   if (batch_size == 0) return ELLM_OK;
   if (batch_size > desc->batch_size)
     return ellm::set_error(ELLM_ERR_OUT_OF_RANGE, "batch_size %zu exceeds the capacity %zu", batch_size,

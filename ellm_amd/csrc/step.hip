@@ -25,6 +25,7 @@ const char* mismatch(const ellm_matmul3* m, const ellm_attn* a) {
   const ellm_matmul3_desc& p = m->d;
   const ellm_attn_desc& d = a->desc;
   if (m->device != a->device) return "the handles were created on different devices";
+  if (a->general) return "the attention operator has a head size other than 128 or binary32 storage";
   if (p.q_state != d.q) return "the projection's q_state is not the attention operator's q";
   if (p.k_state != d.k || p.v_state != d.v) return "the projection's k_state / v_state are not the attention operator's k / v";
   if (p.dtype != d.dtype) return "the handles differ in dtype";

@@ -39,7 +39,7 @@ extern "C" {
 typedef enum ellm_status {
   ELLM_OK = 0,
   ELLM_ERR_INVALID_ARGUMENT = 1, /* null pointer, zero size, bad dtype, strides, ... */
-  ELLM_ERR_UNSUPPORTED = 2,      /* head_size != 128, group size not supported, ...   */
+  ELLM_ERR_UNSUPPORTED = 2,      /* head_size beyond 256, != 128 for projections and caches, ... */
   ELLM_ERR_OUT_OF_RANGE = 3,     /* position / batch / slot beyond the stated capacity */
   ELLM_ERR_HIP = 4,              /* a HIP runtime call (or a host allocation) failed      */
   ELLM_ERR_NO_DEVICE = 5         /* no gfx950 device visible                           */
@@ -47,7 +47,8 @@ typedef enum ellm_status {
 
 typedef enum ellm_dtype {
   ELLM_DTYPE_F16 = 0,
-  ELLM_DTYPE_BF16 = 1
+  ELLM_DTYPE_BF16 = 1,
+  ELLM_DTYPE_F32 = 2  /* attention only (ellm_attn_create / _create_ragged), see ellm_attn_desc */
 } ellm_dtype;
 
 /* Message for the last non-OK status returned on the calling thread. */
@@ -82,6 +83,14 @@ int ellm_device_count(void);
  *   dtype, sequence_capacity (positions per K/V plane; run() rejects positions
  *            at or beyond it), max_position_interval (largest position_interval
  *            run() will be given; sizes q/out).
+ *
+ * head_size 128 with 16-bit storage (every model configuration the reference ships) runs the
+ * MFMA kernels.  Any other head_size from 1 to 256, and ELLM_DTYPE_F32 storage (the type of
+ * the reference's generic leaf and of its operator test, src/kernel/generic/
+ * flash_attention.rs:60-89, src/compiler/mul/attention.rs:262-330), run a plain kernel with the
+ * same arguments, masks and results (binary32 arithmetic throughout), written to be right and
+ * not for a roofline; there kv_strides[0..2] need not be multiples of 8.
+ * ellm_attn_run_noalloc and ellm_matmul3_attn_run take 128-wide 16-bit heads only.
  */
 typedef struct ellm_attn_desc {
   const void* q;

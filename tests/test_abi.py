@@ -82,7 +82,10 @@ def _desc(**over):
     (dict(out=None), INVALID),
     (dict(k=0x1008), INVALID),                       # not 16-byte aligned
     (dict(dtype=7), INVALID),
-    (dict(head_size=64), UNSUPPORTED),               # like the AVX-512 kernel: 128 only
+    (dict(head_size=0), UNSUPPORTED),
+    (dict(head_size=257), UNSUPPORTED),              # the plain kernel's lanes hold four elements each
+    (dict(head_size=64, kv_strides=(2 * 64 * 64, 64 * 64, 32, 1)), INVALID),   # rows closer than a head
+    (dict(dtype=3), INVALID),
     (dict(attention_head_num=7), INVALID),           # not a multiple of kv_head_num
     (dict(kv_head_num=0), INVALID),
     (dict(kv_strides=(2 * 64 * 128, 64 * 128, 128, 2)), INVALID),
