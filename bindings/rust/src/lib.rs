@@ -253,6 +253,33 @@ extern "C" {
         max_position: usize,
         stream: Stream,
     ) -> c_int;
+    pub fn ellm_kv_append_attn_run(
+        cache: *mut ellm_kv_cache,
+        layer: usize,
+        attn: *mut ellm_attn,
+        position_index: usize,
+        batch_size: usize,
+        k_src: *const c_void,
+        v_src: *const c_void,
+        rope: *const c_void,
+        rope_positions: usize,
+        eps: f32,
+        stream: Stream,
+    ) -> c_int;
+    pub fn ellm_kv_append_attn_run_ragged(
+        cache: *mut ellm_kv_cache,
+        layer: usize,
+        attn: *mut ellm_attn,
+        positions: *const u32,
+        max_position: usize,
+        batch_size: usize,
+        k_src: *const c_void,
+        v_src: *const c_void,
+        rope: *const c_void,
+        rope_positions: usize,
+        eps: f32,
+        stream: Stream,
+    ) -> c_int;
 
     pub fn ellm_schedule_calls(
         prompt_begin: usize,

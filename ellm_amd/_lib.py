@@ -144,6 +144,9 @@ ABI_SYMBOLS = {
     "ellm_kv_append": (ctypes.c_int, [_vp, _sz, _sz, _sz, _sz, _vp, _vp, _sz, _vp]),
     "ellm_kv_append_norm_rope": (ctypes.c_int, [_vp, _sz, _sz, _sz, _sz, _vp, _vp, _sz, _vp, _sz,
                                                 ctypes.c_float, _vp, _sz, _vp]),
+    "ellm_kv_append_attn_run": (ctypes.c_int, [_vp, _sz, _vp, _sz, _sz, _vp, _vp, _vp, _sz, ctypes.c_float, _vp]),
+    "ellm_kv_append_attn_run_ragged": (ctypes.c_int, [_vp, _sz, _vp, _vp, _sz, _sz, _vp, _vp, _vp, _sz,
+                                                      ctypes.c_float, _vp]),
     "ellm_schedule_calls": (ctypes.c_int, [_sz, _sz, _sz, _sz, _vp, _sz, ctypes.POINTER(_sz)]),
     "ellm_graph_begin": (ctypes.c_int, [_vp]),
     "ellm_graph_end": (ctypes.c_int, [_vp, _pvp]),

@@ -277,6 +277,30 @@ class KVCache:
             ctypes.c_void_p(_device_buffer("rope", rope, rope.shape[0] * 128, k_src.dtype)),
             rope.shape[0], ctypes.c_float(eps), pos_ptr, int(max_position), _stream_ptr(stream)))
 
+    def append_norm_rope_with_attention(self, layer, attention, position_index, k_src, v_src, rope, eps=1e-6,
+                                        batch_size=None, positions=None, max_position=0, stream=None):
+        """append_norm_rope() of one new token per sequence and `attention`'s single-token run over
+        the cache including it, as one launch (ellm_kv_append_attn_run / _run_ragged).  `attention`
+        must have been created over this layer of this cache; k_src, v_src: [1, batch, kv_heads, 128]."""
+        if k_src.shape[0] != 1:
+            raise ValueError("one new token per sequence")
+        pitch = k_src.shape[1]
+        if batch_size is None:
+            batch_size = pitch
+        if batch_size > pitch:
+            raise ValueError(f"batch_size {batch_size} exceeds the {pitch} rows of k_src")
+        need = pitch * self.desc.kv_head_num * self.desc.head_size
+        ks = ctypes.c_void_p(_device_buffer("k_src", k_src, need))
+        vs = ctypes.c_void_p(_device_buffer("v_src", v_src, need, k_src.dtype))
+        rp = ctypes.c_void_p(_device_buffer("rope", rope, rope.shape[0] * 128, k_src.dtype))
+        if positions is None:
+            check(self._lib.ellm_kv_append_attn_run(self._handle, layer, attention._handle, position_index, batch_size,
+                                                    ks, vs, rp, rope.shape[0], ctypes.c_float(eps), _stream_ptr(stream)))
+        else:
+            check(self._lib.ellm_kv_append_attn_run_ragged(
+                self._handle, layer, attention._handle, _positions_ptr(positions, batch_size), int(max_position),
+                batch_size, ks, vs, rp, rope.shape[0], ctypes.c_float(eps), _stream_ptr(stream)))
+
     def close(self):
         if self._handle:
             check(self._lib.ellm_kv_destroy(self._handle))

@@ -663,6 +663,82 @@ int ellm_kv_append_norm_rope(ellm_kv_cache* c, size_t layer, size_t position_ind
   return ELLM_OK;
 }
 
+// Why an attention operator cannot take a layer of a cache as the destination of its own new rows
+// (null: it can).
+static const char* append_mismatch(const ellm_kv_cache* c, size_t layer, const ellm_attn* a) {
+  const ellm_attn_desc& d = a->desc;
+  if (a->general) return "the attention operator has a head size other than 128 or binary32 storage";
+  if (c->device != a->device) return "the cache and the operator were created on different devices";
+  if (d.dtype != c->desc.dtype) return "the cache and the operator differ in dtype";
+  if (d.kv_head_num != c->desc.kv_head_num) return "the cache and the operator differ in kv_head_num";
+  const void* k = (const char*)c->k + layer * c->layer_elems * 2;
+  const void* v = (const char*)c->v + layer * c->layer_elems * 2;
+  if (d.k != k || d.v != v) return "the operator's k / v are not this layer of the cache";
+  if (d.kv_strides[1] != c->stride_head || d.kv_strides[2] != 128 || d.kv_strides[3] != 1)
+    return "the operator's kv_strides are not the cache's";
+  if (c->ragged) {
+    if (a->seq_offsets != c->seq_offsets_dev || a->seq_caps != c->seq_caps_dev)
+      return "the operator was not created with this cache's sequence table (from its first sequence)";
+  } else if (a->seq_offsets || d.kv_strides[0] != c->stride_seq) {
+    return "the operator's kv_strides are not the cache's";
+  }
+  return nullptr;
+}
+
+static int kv_append_attn(ellm_kv_cache* c, size_t layer, ellm_attn* a, const void* k_src, const void* v_src,
+                          const void* rope, size_t rope_positions, float eps, size_t position_index,
+                          const uint32_t* positions, size_t max_position, size_t batch_size, void* stream) {
+  if (!c || !a) return fail(ELLM_ERR_INVALID_ARGUMENT, "null cache or attention handle");
+  if (batch_size == 0) return ELLM_OK;
+  if (!k_src || !v_src || !rope) return fail(ELLM_ERR_INVALID_ARGUMENT, "null source or rotary table");
+  if (int st = ellm::check_current_device(c->device)) return st;
+  if (!aligned16(k_src) || !aligned16(v_src) || !aligned16(rope))
+    return fail(ELLM_ERR_INVALID_ARGUMENT, "sources and rotary table must be 16-byte aligned");
+  if (!(eps >= 0.0f)) return fail(ELLM_ERR_INVALID_ARGUMENT, "eps must be >= 0");
+  if (layer >= c->desc.layers) return fail(ELLM_ERR_OUT_OF_RANGE, "layer %zu of %zu", layer, c->desc.layers);
+  if (const char* why = append_mismatch(c, layer, a)) return fail(ELLM_ERR_INVALID_ARGUMENT, "%s", why);
+  if (batch_size > c->desc.sequences || batch_size > a->desc.batch_size)
+    return fail(ELLM_ERR_OUT_OF_RANGE, "batch_size %zu exceeds the cache's %zu sequences or the operator's %zu",
+                batch_size, c->desc.sequences, a->desc.batch_size);
+  // the range checks of ellm_kv_append_norm_rope (one token) and of ellm_attn_run / _run_ragged
+  const size_t first = positions ? max_position : position_index;
+  const size_t room = positions ? c->max_cap(batch_size) : c->min_cap(batch_size);
+  if (first >= room) return fail(ELLM_ERR_OUT_OF_RANGE, "position %zu does not fit the capacity %zu", first, room);
+  if (first >= rope_positions)
+    return fail(ELLM_ERR_OUT_OF_RANGE, "position %zu is beyond the %zu rows of the rotary table", first, rope_positions);
+  if (first >= a->desc.sequence_capacity)
+    return fail(ELLM_ERR_OUT_OF_RANGE, "position %zu is not below the operator's sequence capacity %zu", first,
+                a->desc.sequence_capacity);
+  ellm::AttnArgs args;
+  ellm::attn_fill_args(a, &args);
+  args.position_index = (uint32_t)first;
+  args.position_interval = 1;
+  args.batch = (uint32_t)batch_size;
+  args.positions = positions;
+  args.pending.k_rows = k_src;
+  args.pending.v_rows = v_src;
+  args.pending.rope = rope;
+  args.pending.rope_pos_stride = 128;
+  args.pending.rope_head_stride = 0;
+  args.pending.eps = eps;
+  return ellm::attn_run_single_token(a, &args, (uint32_t)first, (hipStream_t)stream);
+}
+
+int ellm_kv_append_attn_run(ellm_kv_cache* cache, size_t layer, ellm_attn* attn, size_t position_index,
+                            size_t batch_size, const void* k_src, const void* v_src, const void* rope,
+                            size_t rope_positions, float eps, void* stream) {
+  return kv_append_attn(cache, layer, attn, k_src, v_src, rope, rope_positions, eps, position_index, nullptr, 0,
+                        batch_size, stream);
+}
+
+int ellm_kv_append_attn_run_ragged(ellm_kv_cache* cache, size_t layer, ellm_attn* attn, const uint32_t* positions,
+                                   size_t max_position, size_t batch_size, const void* k_src, const void* v_src,
+                                   const void* rope, size_t rope_positions, float eps, void* stream) {
+  if (!positions) return fail(ELLM_ERR_INVALID_ARGUMENT, "positions must be a device array");
+  return kv_append_attn(cache, layer, attn, k_src, v_src, rope, rope_positions, eps, 0, positions, max_position,
+                        batch_size, stream);
+}
+
 int ellm_schedule_calls(size_t prompt_begin, size_t prompt_end, size_t chunk, size_t generation_end,
                         ellm_call* calls, size_t capacity, size_t* n_calls) {
   if (!n_calls) return fail(ELLM_ERR_INVALID_ARGUMENT, "null n_calls");

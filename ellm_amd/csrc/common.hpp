@@ -39,6 +39,7 @@ struct Mfma;
 
 template <>
 struct Mfma<F16> {
+  typedef F16 storage;
   static __device__ __forceinline__ f32x16 m32x32x16(u32x4 a, u32x4 b, f32x16 c) {
     return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a),
                                                   __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
@@ -68,6 +69,7 @@ struct Mfma<F16> {
 
 template <>
 struct Mfma<BF16> {
+  typedef BF16 storage;
   static __device__ __forceinline__ f32x16 m32x32x16(u32x4 a, u32x4 b, f32x16 c) {
     return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a),
                                                    __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
@@ -175,6 +177,58 @@ __device__ __forceinline__ u32x4 scale_rotate_pack8(const float (&x)[8], float i
     const float cs = Mfma<T>::to_float((uint16_t)(rope8[e] & 0xffffu)), sn = Mfma<T>::to_float((uint16_t)(rope8[e] >> 16));
     const float y0 = x[2 * e] * inv, y1 = x[2 * e + 1] * inv;
     out[e] = Mfma<T>::pack2(y0 * cs - y1 * sn, y0 * sn + y1 * cs);
+  }
+  return out;
+}
+
+// The value lane - 1 of the same 16-lane row holds; 0 in the row's first lane (a data-parallel
+// move inside the vector ALU, no trip through the LDS crossbar).
+__device__ __forceinline__ float from_left_neighbour(float v) {
+  constexpr int kRowShr1 = 0x111;
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), kRowShr1, 0xf, 0xf, true));
+}
+
+// One 128-wide key row as a stored 16-bit row, normalised and rotated the way the cache write
+// does it (kv_append_norm_rope_kernel; the reference's scalar order, generic forms
+// src/kernel/generic/rms_norm.rs:6-26 and complex_mul.rs:3-20):
+//   y = x / (sqrt(mean(x^2)) + eps);  (e, f) = (a c - b d, a d + b c) for the interleaved pairs
+//   (a, b) of y and (c, d) = (cos, sin) of the rotary row.
+// Sixteen lanes own the row (lane c of the 16-lane row: elements 8 c .. 8 c + 7 in kraw, the
+// same elements of the rotary row in rraw).  Binary32 with one rounding per operation and no
+// contraction; the sum of squares runs through the 128 elements first to last: turn by turn
+// every lane adds its eight squares to what its left neighbour held after the turn before, so
+// lane c's value is final from turn c on and lane 15 ends with the whole sum, the same bits a
+// sequential CPU loop produces.  Every lane of the wave must call this (row shifts, one shuffle).
+template <typename T>
+__device__ __forceinline__ u32x4 norm_rope_row16(u32x4 kraw, u32x4 rraw, float eps) {
+#pragma clang fp contract(off)
+  float x[8], sq[8];
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    x[2 * e] = Mfma<T>::to_float((uint16_t)(kraw[e] & 0xffffu));
+    x[2 * e + 1] = Mfma<T>::to_float((uint16_t)(kraw[e] >> 16));
+  }
+#pragma unroll
+  for (int e = 0; e < 8; ++e) sq[e] = x[e] * x[e];
+  float mine = 0.0f;
+#pragma unroll
+  for (int l = 0; l < 16; ++l) {
+    mine = from_left_neighbour(mine);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) mine = mine + sq[e];
+  }
+  const float sum = __shfl(mine, 15, 16);
+  const float variance = sum / (float)kHeadDim;
+  const float rrms = 1.0f / (sqrtf(variance) + eps);
+  u32x4 out;
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    const float a = x[2 * e] * rrms, bb = x[2 * e + 1] * rrms;
+    const float cs = Mfma<T>::to_float((uint16_t)(rraw[e] & 0xffffu));
+    const float sn = Mfma<T>::to_float((uint16_t)(rraw[e] >> 16));
+    const float re = a * cs - bb * sn;
+    const float im = a * sn + bb * cs;
+    out[e] = Mfma<T>::pack2(re, im);
   }
   return out;
 }

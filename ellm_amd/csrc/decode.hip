@@ -29,9 +29,10 @@ namespace ellm {
 using namespace dec;
 namespace {
 
-// PENDING: the launch of a fused step (ellm_matmul3_attn_run): the query rows and the new key /
-// value row of every plane come as the projection's raw sums (p.pend) and are finished here.
-template <typename T, bool PENDING>
+// PENDING = kPendSums: the launch of a fused step (ellm_matmul3_attn_run): the query rows and the
+// new key / value row of every plane come as the projection's raw sums (p.pend) and are finished
+// here.  kPendRows (ellm_kv_append_attn_run): the new key / value rows come as stored 16-bit rows.
+template <typename T, int PENDING>
 __global__ __launch_bounds__(kDecThreads, PENDING ? 2 : 4) void decode_split_kernel(DecodeKernelArgs p) {
   __shared__ __attribute__((aligned(16))) uint16_t smem[kDecWaves * kWaveLdsHalves];
   __shared__ uint32_t s_last;
@@ -66,25 +67,20 @@ __global__ __launch_bounds__(kDecThreads, PENDING ? 2 : 4) void decode_split_ker
   f32x4 acc[8];
   if constexpr (PENDING) {
     PendingQueries queries;   // requested first: the stream's own loads follow
-    queries.fetch(p.pend, seq, head0, pos, t, heads_here);
-    NewRow fresh;
-    fresh.present = k_end == len;   // the split that holds the plane's last key
-    fresh.store = hgrp == 0;
-    const size_t col_k = (size_t)seq * p.pend.cols + (size_t)(p.n_q_heads + kvh) * kHeadDim;
-    fresh.k_raw = p.pend.raw + col_k;
-    fresh.v_raw = p.pend.raw + col_k + (size_t)p.n_kv_heads * kHeadDim;
-    fresh.parts = p.pend.parts;
-    fresh.part_stride = p.pend.part_stride;
-    fresh.rope_row = (const uint16_t*)p.pend.rope + (size_t)pos * p.pend.rope_pos_stride +
-                     (size_t)kvh * p.pend.rope_head_stride;
-    fresh.eps = p.pend.eps;
-    fresh.k_dst = const_cast<uint16_t*>(p.k) + plane + (size_t)pos * p.kv_stride_pos;
-    fresh.v_dst = const_cast<uint16_t*>(p.v) + plane + (size_t)pos * p.kv_stride_pos;
-    stream_keys<T, true>(p.k + plane, p.v + plane, p.kv_stride_pos, k_begin, k_end, pos, qreg, smem, t,
-                         split * 7u + blockIdx.y * 3u + seq * 5u, p.scale_log2, m_run, l_run, acc, &fresh,
-                         &queries, heads_here);
+    if constexpr (PENDING == kPendSums) queries.fetch(p.pend, seq, head0, pos, t, heads_here);
+    // the split that holds the plane's last key takes the new row; one workgroup of a group writes it
+    const NewRow fresh = new_row_of<PENDING>(p.pend, seq, kvh, pos, p.n_q_heads, p.n_kv_heads,
+                                             const_cast<uint16_t*>(p.k) + plane + (size_t)pos * p.kv_stride_pos,
+                                             const_cast<uint16_t*>(p.v) + plane + (size_t)pos * p.kv_stride_pos,
+                                             k_end == len, hgrp == 0);
+    if constexpr (PENDING == kPendRows) load_queries(p.q + (size_t)row0 * kHeadDim, t, heads_here, qreg);
+    stream_keys<T, PENDING>(p.k + plane, p.v + plane, p.kv_stride_pos, k_begin, k_end, pos, qreg, smem, t,
+                            split * 7u + blockIdx.y * 3u + seq * 5u, p.scale_log2, m_run, l_run, acc, &fresh,
+                            PENDING == kPendSums ? &queries : nullptr, heads_here);
     // the finished query rows, once per group: by the workgroup that also wrote the new key
-    if (fresh.present) store_queries(const_cast<uint16_t*>(p.q) + (size_t)row0 * kHeadDim, t, heads_here, qreg);
+    if constexpr (PENDING == kPendSums) {
+      if (fresh.present) store_queries(const_cast<uint16_t*>(p.q) + (size_t)row0 * kHeadDim, t, heads_here, qreg);
+    }
   } else {
     load_queries(p.q + (size_t)row0 * kHeadDim, t, heads_here, qreg);
     stream_keys<T>(p.k + plane, p.v + plane, p.kv_stride_pos, k_begin, k_end, pos, qreg, smem, t,
@@ -171,13 +167,18 @@ hipError_t launch_decode(const AttnArgs& a, hipStream_t stream) {
   dim3 block(kDecThreads);
   if (a.pending.raw) {
     if (a.dtype == 0)
-      hipLaunchKernelGGL((decode_split_kernel<F16, true>), grid, block, 0, stream, p);
+      hipLaunchKernelGGL((decode_split_kernel<F16, kPendSums>), grid, block, 0, stream, p);
     else
-      hipLaunchKernelGGL((decode_split_kernel<BF16, true>), grid, block, 0, stream, p);
+      hipLaunchKernelGGL((decode_split_kernel<BF16, kPendSums>), grid, block, 0, stream, p);
+  } else if (a.pending.k_rows) {
+    if (a.dtype == 0)
+      hipLaunchKernelGGL((decode_split_kernel<F16, kPendRows>), grid, block, 0, stream, p);
+    else
+      hipLaunchKernelGGL((decode_split_kernel<BF16, kPendRows>), grid, block, 0, stream, p);
   } else if (a.dtype == 0) {
-    hipLaunchKernelGGL((decode_split_kernel<F16, false>), grid, block, 0, stream, p);
+    hipLaunchKernelGGL((decode_split_kernel<F16, kPendNone>), grid, block, 0, stream, p);
   } else {
-    hipLaunchKernelGGL((decode_split_kernel<BF16, false>), grid, block, 0, stream, p);
+    hipLaunchKernelGGL((decode_split_kernel<BF16, kPendNone>), grid, block, 0, stream, p);
   }
   return hipGetLastError();
 }

@@ -38,7 +38,7 @@ __device__ __forceinline__ uint32_t uni(uint32_t v) { return (uint32_t)__builtin
 // reason (1 + floor(n / 16) >= ceil(n / 16)).
 
 // PENDING: the launch of a fused step, as in decode.hip.
-template <typename T, bool PENDING>
+template <typename T, int PENDING>
 __global__ __launch_bounds__(kDecThreads, 2) void decode_balanced_kernel(DecodeKernelArgs p) {
   __shared__ __attribute__((aligned(16))) uint16_t smem[kDecWaves * kWaveLdsHalves];
   __shared__ uint32_t prefix[kMaxBatch + 1];   // units of the sequences before sequence b (per plane)
@@ -196,24 +196,19 @@ __global__ __launch_bounds__(kDecThreads, 2) void decode_balanced_kernel(DecodeK
     f32x4 acc[8];
     if constexpr (PENDING) {
       PendingQueries queries;   // requested first: the stream's own loads follow
-      queries.fetch(p.pend, seq, head0, pos, t, heads_here);
-      NewRow fresh;
-      fresh.present = k_end == pos + 1;   // the piece that holds the plane's last key
-      fresh.store = hgrp == 0;
-      const size_t col_k = (size_t)seq * p.pend.cols + (size_t)(p.n_q_heads + kvh) * kHeadDim;
-      fresh.k_raw = p.pend.raw + col_k;
-      fresh.v_raw = p.pend.raw + col_k + (size_t)p.n_kv_heads * kHeadDim;
-      fresh.parts = p.pend.parts;
-      fresh.part_stride = p.pend.part_stride;
-      fresh.rope_row = (const uint16_t*)p.pend.rope + (size_t)pos * p.pend.rope_pos_stride +
-                       (size_t)kvh * p.pend.rope_head_stride;
-      fresh.eps = p.pend.eps;
-      fresh.k_dst = const_cast<uint16_t*>(p.k) + plane + (size_t)pos * p.kv_stride_pos;
-      fresh.v_dst = const_cast<uint16_t*>(p.v) + plane + (size_t)pos * p.kv_stride_pos;
-      stream_keys<T, true>(p.k + plane, p.v + plane, p.kv_stride_pos, k_begin, k_end, pos, qreg, smem, t,
-                           w * 7u + pl * 3u + seq * 5u, p.scale_log2, m_run, l_run, acc, &fresh,
-                           &queries, heads_here);
-      if (fresh.present) store_queries(const_cast<uint16_t*>(p.q) + (size_t)row0 * kHeadDim, t, heads_here, qreg);
+      if constexpr (PENDING == kPendSums) queries.fetch(p.pend, seq, head0, pos, t, heads_here);
+      // the piece that holds the plane's last key takes the new row; one workgroup of a group writes it
+      const NewRow fresh = new_row_of<PENDING>(p.pend, seq, kvh, pos, p.n_q_heads, p.n_kv_heads,
+                                               const_cast<uint16_t*>(p.k) + plane + (size_t)pos * p.kv_stride_pos,
+                                               const_cast<uint16_t*>(p.v) + plane + (size_t)pos * p.kv_stride_pos,
+                                               k_end == pos + 1, hgrp == 0);
+      if constexpr (PENDING == kPendRows) load_queries(p.q + (size_t)row0 * kHeadDim, t, heads_here, qreg);
+      stream_keys<T, PENDING>(p.k + plane, p.v + plane, p.kv_stride_pos, k_begin, k_end, pos, qreg, smem, t,
+                              w * 7u + pl * 3u + seq * 5u, p.scale_log2, m_run, l_run, acc, &fresh,
+                              PENDING == kPendSums ? &queries : nullptr, heads_here);
+      if constexpr (PENDING == kPendSums) {
+        if (fresh.present) store_queries(const_cast<uint16_t*>(p.q) + (size_t)row0 * kHeadDim, t, heads_here, qreg);
+      }
     } else {
       load_queries(p.q + (size_t)row0 * kHeadDim, t, heads_here, qreg);
       stream_keys<T>(p.k + plane, p.v + plane, p.kv_stride_pos, k_begin, k_end, pos, qreg, smem, t,
@@ -307,13 +302,18 @@ hipError_t launch_decode_balanced(const AttnArgs& a, uint32_t wgs, hipStream_t s
   const dim3 grid(wgs), block(kDecThreads);
   if (a.pending.raw) {
     if (a.dtype == 0)
-      hipLaunchKernelGGL((decode_balanced_kernel<F16, true>), grid, block, 0, stream, p);
+      hipLaunchKernelGGL((decode_balanced_kernel<F16, kPendSums>), grid, block, 0, stream, p);
     else
-      hipLaunchKernelGGL((decode_balanced_kernel<BF16, true>), grid, block, 0, stream, p);
+      hipLaunchKernelGGL((decode_balanced_kernel<BF16, kPendSums>), grid, block, 0, stream, p);
+  } else if (a.pending.k_rows) {
+    if (a.dtype == 0)
+      hipLaunchKernelGGL((decode_balanced_kernel<F16, kPendRows>), grid, block, 0, stream, p);
+    else
+      hipLaunchKernelGGL((decode_balanced_kernel<BF16, kPendRows>), grid, block, 0, stream, p);
   } else if (a.dtype == 0) {
-    hipLaunchKernelGGL((decode_balanced_kernel<F16, false>), grid, block, 0, stream, p);
+    hipLaunchKernelGGL((decode_balanced_kernel<F16, kPendNone>), grid, block, 0, stream, p);
   } else {
-    hipLaunchKernelGGL((decode_balanced_kernel<BF16, false>), grid, block, 0, stream, p);
+    hipLaunchKernelGGL((decode_balanced_kernel<BF16, kPendNone>), grid, block, 0, stream, p);
   }
   return hipGetLastError();
 }

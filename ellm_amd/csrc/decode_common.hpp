@@ -187,17 +187,55 @@ __device__ __forceinline__ void store_queries(uint16_t* q_rows, const Lane& t, u
 struct NewRow {
   bool present;              // this stretch of keys ends with the plane's new key
   bool store;                // ... and this workgroup is the one that writes it to the cache
-  const float* k_raw;        // 128 raw sums each (first part)
+  const float* k_raw;        // kPendSums: 128 raw sums each (first part)
   const float* v_raw;
   uint32_t parts, part_stride;
+  const uint16_t* k_row16;   // kPendRows: the 128-element source rows
+  const uint16_t* v_row16;
   const uint16_t* rope_row;  // rotary row of (position, kv head)
   float eps;
   uint16_t* k_dst;
   uint16_t* v_dst;
 };
+// What a launch finds pending (template argument of the kernels and of stream_keys).
+constexpr int kPendNone = 0;   // the ordinary launch
+constexpr int kPendSums = 1;   // a fused projection step: raw binary32 sums of the query, key and value rows
+constexpr int kPendRows = 2;   // a fused cache write: stored 16-bit key / value rows, queries final
+
+// The new row of plane (sequence, kv head) at position pos, as the launch's PendingRows describe it.
+template <int MODE>
+__device__ __forceinline__ NewRow new_row_of(const PendingRows& pr, uint32_t seq, uint32_t kvh, uint32_t pos,
+                                             uint32_t n_q_heads, uint32_t n_kv_heads, uint16_t* k_dst, uint16_t* v_dst,
+                                             bool present, bool store) {
+  NewRow n;
+  n.present = present;
+  n.store = store;
+  n.k_raw = n.v_raw = nullptr;
+  n.parts = n.part_stride = 0;
+  n.k_row16 = n.v_row16 = nullptr;
+  if constexpr (MODE == kPendSums) {
+    const size_t col_k = (size_t)seq * pr.cols + (size_t)(n_q_heads + kvh) * kHeadDim;
+    n.k_raw = pr.raw + col_k;
+    n.v_raw = pr.raw + col_k + (size_t)n_kv_heads * kHeadDim;
+    n.parts = pr.parts;
+    n.part_stride = pr.part_stride;
+  } else {
+    const size_t row = ((size_t)seq * n_kv_heads + kvh) * kHeadDim;
+    n.k_row16 = (const uint16_t*)pr.k_rows + row;
+    n.v_row16 = (const uint16_t*)pr.v_rows + row;
+  }
+  n.rope_row = (const uint16_t*)pr.rope + (size_t)pos * pr.rope_pos_stride + (size_t)kvh * pr.rope_head_stride;
+  n.eps = pr.eps;
+  n.k_dst = k_dst;
+  n.v_dst = v_dst;
+  return n;
+}
 // Every lane c of each 16-lane group ends up with elements 8 c .. 8 c + 7 of the finished rows
 // (the arithmetic of the projection's own finishing step, lane for lane).
-struct NewRowLoads {
+template <int MODE>
+struct NewRowLoads;
+template <>
+struct NewRowLoads<kPendSums> {
   Raw8 k, v;
   u32x4 rope;
   __device__ __forceinline__ void fetch(const NewRow& n, const Lane& t) {
@@ -222,6 +260,32 @@ struct NewRowLoads {
     }
   }
 };
+// Stored 16-bit rows: the cache write's own arithmetic (norm_rope_row16), so the row that lands in
+// the cache carries the bits ellm_kv_append_norm_rope would have written.
+template <>
+struct NewRowLoads<kPendRows> {
+  u32x4 k, v, rope;
+  __device__ __forceinline__ void fetch(const NewRow& n, const Lane& t) {
+    k = load16(n.k_row16 + 8 * t.c);
+    v = load16(n.v_row16 + 8 * t.c);
+    rope = load16(n.rope_row + 8 * t.c);
+  }
+  template <typename T>
+  __device__ __forceinline__ void finish(const NewRow& n, const Lane& t, u32x4& knew, u32x4& vnew) const {
+    knew = norm_rope_row16<T>(k, rope, n.eps);
+    vnew = v;
+    if (n.store && t.g == 0) {
+      store16(n.k_dst + 8 * t.c, knew);
+      store16(n.v_dst + 8 * t.c, vnew);
+    }
+  }
+};
+template <>
+struct NewRowLoads<kPendNone> {
+  __device__ __forceinline__ void fetch(const NewRow&, const Lane&) {}
+  template <typename T>
+  __device__ __forceinline__ void finish(const NewRow&, const Lane&, u32x4&, u32x4&) const {}
+};
 
 // One wave's share of keys [k_begin, k_end) of a plane: the four waves take alternating 16-key
 // chunks, each streams its chunks HBM -> registers (128-bit loads, four full 256-byte rows per
@@ -240,8 +304,9 @@ struct NewRowLoads {
 // and takes it as one more chunk of its own.
 // The raw rows are requested ahead of the wave's first chunk of keys and finished behind its
 // request (`queries` holds the requested raw query rows; qreg is filled here), so that both
-// trips to memory run side by side.
-template <typename T, bool PENDING = false>
+// trips to memory run side by side.  With kPendRows (a fused cache write) the new rows come as
+// stored 16-bit rows, the query rows are final (qreg filled by the caller, `queries` null).
+template <typename T, int PENDING = kPendNone>
 __device__ __forceinline__ void stream_keys(const uint16_t* kplane, const uint16_t* vplane, size_t stride_pos,
                                             uint32_t k_begin, uint32_t k_end, uint32_t pos,
                                             u32x4 (&qreg)[4], uint16_t* smem, const Lane& t,
@@ -340,14 +405,14 @@ __device__ __forceinline__ void stream_keys(const uint16_t* kplane, const uint16
     }
   };
 
-  NewRowLoads fresh_loads;
+  NewRowLoads<PENDING> fresh_loads;
   if constexpr (PENDING) {
     if (take_new) fresh_loads.fetch(*fresh, t);
   }
   if (my_chunks) issue_loads(chunk_at(0));
+  if constexpr (PENDING == kPendSums) queries->template finish<T>(fresh->eps, t, heads_here, qreg);
   if constexpr (PENDING) {
-    queries->template finish<T>(fresh->eps, t, heads_here, qreg);
-    if (take_new) fresh_loads.template finish<T>(*fresh, t, knew, vnew);
+    if (take_new) fresh_loads.template finish<T>(*fresh, t, knew, vnew);   // (the whole wave: uniform)
   }
   for (uint32_t it = 0; it < my_chunks; ++it) {
     const uint32_t chunk = chunk_at(it);

@@ -18,11 +18,18 @@ namespace ellm {
 // normalise and rotate the query and key heads while they load them and write the finished
 // query rows, the new key row and the new value row to where the projection alone would have.
 struct PendingRows {
-  const float* raw;   // null: nothing pending (the ordinary launch)
+  const float* raw;   // null: no raw sums pending
   uint32_t parts, part_stride, cols;   // part_stride, cols in floats
   const void* rope;   // (cos, sin) pairs, as in ProjectArgs
   uint32_t rope_pos_stride, rope_head_stride;
   float eps;
+  // The other form (ellm_kv_append_attn_run; raw is null then): the query rows are final and
+  // only the new key / value rows are pending, as stored 16-bit rows [sequence][kv_head][128]
+  // that the cache write (kv_append_norm_rope_kernel) would normalise, rotate and copy: the
+  // attention launch does that with the same arithmetic, bit for bit.  null: nothing of that
+  // kind pending.
+  const void* k_rows;
+  const void* v_rows;
 };
 
 // Everything a launch needs; filled by the C ABI after validation.

@@ -38,18 +38,9 @@ __global__ __launch_bounds__(256) void kv_append_kernel(
 //   y = x / (sqrt(mean(x^2)) + eps);  (e, f) = (a c - b d, a d + b c) for the
 //   interleaved pairs (a, b) of y and (c, d) = (cos, sin) of the rotary row of
 //   the token's position.
-// Sixteen lanes own one row (8 elements each).  All arithmetic is binary32 with
-// one rounding per operation, in the order of the reference's scalar code: the
-// sum of squares runs through the 128 elements from first to last (the sixteen
-// lanes take turns, each adding its eight squares to the running sum it is
-// handed), so the result is the same bits a sequential CPU loop produces.
-// The value lane - 1 of the same 16-lane row holds; 0 in the row's first lane (a data-parallel
-// move inside the vector ALU, no trip through the LDS crossbar).
-__device__ __forceinline__ float from_left_neighbour(float v) {
-  constexpr int kRowShr1 = 0x111;
-  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), kRowShr1, 0xf, 0xf, true));
-}
-
+// Sixteen lanes own one row (8 elements each); the arithmetic is norm_rope_row16 (common.hpp):
+// binary32, one rounding per operation, the reference's scalar order, so the stored rows are
+// the bits a sequential CPU loop produces.
 template <typename T>
 __global__ __launch_bounds__(256) void kv_append_norm_rope_kernel(
     uint16_t* __restrict__ k_dst, uint16_t* __restrict__ v_dst, const uint16_t* __restrict__ k_src,
@@ -57,7 +48,6 @@ __global__ __launch_bounds__(256) void kv_append_norm_rope_kernel(
     const uint32_t* __restrict__ positions, uint32_t n_tokens, uint32_t batch,
     uint32_t src_batch_pitch, uint32_t n_kv_heads, KvLayout layout, uint32_t position_index,
     uint32_t max_start, float eps) {
-#pragma clang fp contract(off)
   const uint32_t c = threadIdx.x & 15;
   const size_t rows = (size_t)n_tokens * batch * n_kv_heads;
   // every lane of a wave runs the same number of trips: the loop holds cross-lane reads
@@ -82,38 +72,7 @@ __global__ __launch_bounds__(256) void kv_append_norm_rope_kernel(
     const u32x4 kraw = load16_once(k_src + src);
     const u32x4 vraw = load16_once(v_src + src);
     const u32x4 rraw = load16(rope + (size_t)pos * kHeadDim + 8 * c);
-    float x[8], sq[8];
-#pragma unroll
-    for (int e = 0; e < 4; ++e) {
-      x[2 * e] = T::to_float((uint16_t)(kraw[e] & 0xffffu));
-      x[2 * e + 1] = T::to_float((uint16_t)(kraw[e] >> 16));
-    }
-#pragma unroll
-    for (int e = 0; e < 8; ++e) sq[e] = x[e] * x[e];
-    // Turn by turn every lane adds its eight squares to what its left neighbour held after the
-    // turn before (a row shift inside the 16-lane row, zero into lane 0): lane c's value is final
-    // from turn c on, so after sixteen turns lane 15 holds the sum over all 128 elements, added
-    // first to last.
-    float mine = 0.0f;
-#pragma unroll
-    for (int l = 0; l < 16; ++l) {
-      mine = from_left_neighbour(mine);
-#pragma unroll
-      for (int e = 0; e < 8; ++e) mine = mine + sq[e];
-    }
-    const float sum = __shfl(mine, 15, 16);
-    const float variance = sum / (float)kHeadDim;
-    const float rrms = 1.0f / (sqrtf(variance) + eps);
-    u32x4 out;
-#pragma unroll
-    for (int e = 0; e < 4; ++e) {
-      const float a = x[2 * e] * rrms, bb = x[2 * e + 1] * rrms;
-      const float cs = T::to_float((uint16_t)(rraw[e] & 0xffffu));
-      const float sn = T::to_float((uint16_t)(rraw[e] >> 16));
-      const float re = a * cs - bb * sn;
-      const float im = a * sn + bb * cs;
-      out[e] = T::pack2(re, im);
-    }
+    const u32x4 out = norm_rope_row16<typename T::storage>(kraw, rraw, eps);
     if (live) {
       store16_once(k_dst + dst, out);
       store16_once(v_dst + dst, vraw);

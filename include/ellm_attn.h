@@ -326,6 +326,33 @@ int ellm_kv_append_norm_rope(ellm_kv_cache* cache, size_t layer, size_t position
                              size_t rope_positions, float eps, const uint32_t* positions,
                              size_t max_position, void* stream);
 
+/*
+ * ellm_kv_append_norm_rope for one new token per sequence and the attention over the cache
+ * including that token (ellm_attn_run / ellm_attn_run_ragged with position_interval 1), as one
+ * launch: the workgroup of the attention kernel that holds a plane's last key normalises and
+ * rotates the new key row (the cache write's own arithmetic: the row in the cache carries the
+ * same bits), copies the new value row, writes both to the cache and takes them as the last
+ * key of its stream.  For callers that run their own projection and keep the two steps apart
+ * otherwise: a single-token step of a layer is then one launch instead of two (the reference
+ * does the write inside its projection, src/compiler/mul/matmul3.rs:243-254, and runs the
+ * attention operator next, src/qwen3_moe/attention.rs:126-174; with this library's projection
+ * the corresponding call is ellm_matmul3_attn_run).
+ * attn must have been created over this layer of this cache (k, v, kv_strides of ellm_kv_layer /
+ * ellm_kv_layer_ragged from the cache's first sequence, the cache's dtype); else
+ * ELLM_ERR_INVALID_ARGUMENT.  k_src, v_src: device, [batch_size][kv_head][128] rows of the new
+ * token; rope, rope_positions, eps, positions, max_position as in ellm_kv_append_norm_rope.
+ * The query rows in the operator's q are final (normalised and rotated by the caller's
+ * projection).  Results: the cache as ellm_kv_append_norm_rope leaves it, out / lse as
+ * ellm_attn_run leaves them (same tolerance; the new key is taken in a different chunk).
+ */
+int ellm_kv_append_attn_run(ellm_kv_cache* cache, size_t layer, ellm_attn* attn, size_t position_index,
+                            size_t batch_size, const void* k_src, const void* v_src, const void* rope,
+                            size_t rope_positions, float eps, void* stream);
+int ellm_kv_append_attn_run_ragged(ellm_kv_cache* cache, size_t layer, ellm_attn* attn,
+                                   const uint32_t* positions, size_t max_position, size_t batch_size,
+                                   const void* k_src, const void* v_src, const void* rope,
+                                   size_t rope_positions, float eps, void* stream);
+
 /* ------------------------------------------------------------------------ *
  * Position / chunk schedule and a recorded single-token step.
  * ------------------------------------------------------------------------ */
