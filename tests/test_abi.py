@@ -111,6 +111,9 @@ def test_null_arguments():
     assert lib.ellm_attn_run_ragged(None, None, 0, 1, None) == INVALID
     assert lib.ellm_attn_destroy(None) == OK
     assert lib.ellm_kv_destroy(None) == OK
+    assert lib.ellm_kv_append_attn_run(None, 0, None, 0, 1, None, None, None, 0, 1e-6, None) == INVALID
+    assert lib.ellm_kv_append_attn_run_ragged(None, 0, None, None, 0, 1, None, None, None, 0, 1e-6, None) == INVALID
+    assert lib.ellm_matmul3_attn_run(None, None, 0, 1, None) == INVALID
     c = ctypes.c_void_p()
     assert lib.ellm_kv_create(None, ctypes.byref(c)) == INVALID
     kd = _lib.KvDesc(1, 1, 1, 64, 16, 0)
