@@ -199,3 +199,37 @@ def test_entry_points_for_128_wide_16_bit_heads_refuse_other_shapes():
         ellm_amd.KVCache(1, 1, 1, 16, _lib.DTYPE_F16, head_size=64)
     assert e.value.status == 2
     torch.cuda.synchronize()
+
+
+def test_random_shapes_against_the_oracle():
+    """Seeded sweep over head sizes 1..256, the three storage types, group sizes, batches below capacity,
+    chunks and single-token steps with shared and per-sequence positions."""
+    rng = np.random.default_rng(2024)
+    for n in range(18):
+        dtype = (orc.F16, orc.BF16, orc.F32)[n % 3]
+        hs = int(rng.integers(1, 257))
+        hkv = int(rng.integers(1, 4))
+        hq = hkv * int(rng.integers(1, 5))
+        bcap = int(rng.integers(1, 4))
+        b = int(rng.integers(1, bcap + 1))
+        cap = int(rng.integers(8, 300))
+        q_seed = 100 + n
+        scale = float(rng.uniform(0.02, 0.3))
+        if n % 2 == 0:      # a chunk
+            s = int(rng.integers(1, min(cap, 40) + 1))
+            p0 = int(rng.integers(0, cap - s + 1))
+            name = f"rand{n}_chunk_h{hs}_g{hq // hkv}_s{s}_p{p0}"
+            print("case", name, flush=True)
+            q, k, v = _rand((s, bcap, hq, hs), q_seed, dtype), _rand((bcap, hkv, cap, hs), q_seed + 50, dtype), _rand((bcap, hkv, cap, hs), q_seed + 90, dtype)
+            want, want_lse = orc.attention(q, k, v, scale, dtype, position_index=p0, batch=b)
+            got, lse = _run(q, k, v, scale, dtype, p0=p0, batch=b)
+        else:               # one token per sequence at its own position
+            positions = [int(x) for x in rng.integers(0, cap, size=b)]
+            name = f"rand{n}_step_h{hs}_g{hq // hkv}_pos{positions}"
+            print("case", name, flush=True)
+            q, k, v = _rand((1, bcap, hq, hs), q_seed, dtype), _rand((bcap, hkv, cap, hs), q_seed + 50, dtype), _rand((bcap, hkv, cap, hs), q_seed + 90, dtype)
+            pos = np.zeros(bcap, dtype=np.uint32)
+            pos[:b] = positions
+            want, want_lse = orc.attention(q, k, v, scale, dtype, positions=pos, batch=b)
+            got, lse = _run(q, k, v, scale, dtype, batch=b, positions=positions)
+        _check(name, got, lse, want, want_lse, dtype, b)
