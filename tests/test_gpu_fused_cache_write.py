@@ -287,3 +287,39 @@ def test_fused_cache_write_refuses_an_operator_over_other_memory():
     finally:
         step.close()
         other.close()
+
+
+def test_random_shapes_against_the_two_calls_and_the_oracle():
+    """Seeded sweep: group sizes 1..32, batches below capacity, capacities from a few rows to a few
+    thousand, shared and per-sequence positions, both storage types."""
+    rng = np.random.default_rng(77)
+    for n in range(14):
+        dtype = orc.F16 if n % 2 == 0 else orc.BF16
+        hkv = int(rng.integers(1, 5))
+        hq = hkv * int(rng.choice([1, 2, 3, 4, 8, 16, 32]))
+        if hq > 64:
+            hq = hkv * 8
+        bcap = int(rng.integers(1, 7))
+        batch = int(rng.integers(1, bcap + 1))
+        cap = int(rng.choice([8, 65, 130, 700, 2100, 5000]))
+        if n % 3 == 0:
+            positions = int(rng.integers(0, cap))
+        else:
+            positions = [int(x) for x in rng.integers(0, cap, size=batch)]
+        name = f"rand{n}_b{batch}of{bcap}_h{hq}kv{hkv}_cap{cap}_{positions}"
+        print("case", name, flush=True)
+        step = _Step(dtype, bcap, hq, hkv, cap, seed=200 + n)
+        try:
+            shared = positions if np.isscalar(positions) else None
+            plist = [positions] * batch if shared is not None else list(positions)
+            dpos = None if shared is not None else _positions_dev(plist)
+            step.reset()
+            step.two_calls(dpos, batch, shared)
+            plain = step.snapshot()
+            step.reset()
+            step.fused(dpos, batch, shared)
+            fused = step.snapshot()
+            _compare(step, plain, fused, batch)
+            _oracle_check(step, fused, plist, batch)
+        finally:
+            step.close()
